@@ -1,0 +1,379 @@
+// C ABI of libtrittention_hip.so: argument checks, scratch layout, dispatch.
+// Declarations and the contract of each entry point: include/trittention_hip.h.
+#include "../../include/trittention_hip.h"
+
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace tritt {
+namespace {
+
+// Bump allocator over the caller's workspace; with base == nullptr it only measures.
+struct Arena {
+    char* base;
+    size_t off = 0;
+    explicit Arena(void* b) : base(static_cast<char*>(b)) {}
+    template <typename T>
+    T* take(size_t count) {
+        off = (off + 255) & ~size_t(255);
+        T* p = base ? reinterpret_cast<T*>(base + off) : nullptr;
+        off += count * sizeof(T);
+        return p;
+    }
+    size_t bytes() const { return (off + 255) & ~size_t(255); }
+};
+
+size_t elem_size(int dtype) { return dtype == TRITT_F32 ? 4 : 2; }
+
+int check_common(int B, int H, int T, int D, int dtype) {
+    if (B <= 0 || H <= 0 || T <= 0) return TRITT_ERR_INVALID;
+    if (dtype != TRITT_F32 && dtype != TRITT_BF16 && dtype != TRITT_F16) return TRITT_ERR_INVALID;
+    if (D != 16 && D != 32 && D != 64 && D != 128) return TRITT_ERR_HEAD_DIM;
+    if ((long long)B * H > 65535) return TRITT_ERR_INVALID;
+    return TRITT_OK;
+}
+
+// ---------------------------------------------------------------- elementwise helpers
+template <typename T, bool SILU>
+__global__ __launch_bounds__(256) void to_f32_kernel(const T* __restrict__ src, float* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        float v = to_float(src[i]);
+        dst[i] = SILU ? silu_f(v) : v;
+    }
+}
+
+// dst = src (* SiLU'(v1) when v1 != nullptr), converted to T
+template <typename T>
+__global__ __launch_bounds__(256) void from_f32_kernel(const float* __restrict__ src, const T* __restrict__ v1,
+                                                       T* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        float v = src[i];
+        if (v1) v *= silu_grad_f(to_float(v1[i]));
+        dst[i] = from_float<T>(v);
+    }
+}
+
+// delta[row] = sum_d a[row, d] * b[row, d]   (one wave per row)
+template <typename T>
+__global__ __launch_bounds__(256) void rowdot_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                     float* __restrict__ out, int rows, int D) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    float part = 0.f;
+    for (int d = lane; d < D; d += 64) part += to_float(a[(size_t)row * D + d]) * to_float(b[(size_t)row * D + d]);
+    part = wave_sum(part);
+    if (lane == 0) out[row] = part;
+}
+
+unsigned ew_grid(size_t n) {
+    size_t g = (n + 255) / 256;
+    return (unsigned)(g > 8192 ? 8192 : g);
+}
+
+template <bool SILU>
+void to_f32(const void* src, float* dst, size_t n, int dtype, hipStream_t st) {
+    if (dtype == TRITT_F32)
+        hipLaunchKernelGGL((to_f32_kernel<float, SILU>), dim3(ew_grid(n)), dim3(256), 0, st, (const float*)src, dst, n);
+    else if (dtype == TRITT_BF16)
+        hipLaunchKernelGGL((to_f32_kernel<bf16_t, SILU>), dim3(ew_grid(n)), dim3(256), 0, st, (const bf16_t*)src, dst, n);
+    else
+        hipLaunchKernelGGL((to_f32_kernel<f16_t, SILU>), dim3(ew_grid(n)), dim3(256), 0, st, (const f16_t*)src, dst, n);
+}
+
+void from_f32(const float* src, const void* v1, void* dst, size_t n, int dtype, hipStream_t st) {
+    if (dtype == TRITT_F32)
+        hipLaunchKernelGGL(from_f32_kernel<float>, dim3(ew_grid(n)), dim3(256), 0, st, src, (const float*)v1, (float*)dst, n);
+    else if (dtype == TRITT_BF16)
+        hipLaunchKernelGGL(from_f32_kernel<bf16_t>, dim3(ew_grid(n)), dim3(256), 0, st, src, (const bf16_t*)v1, (bf16_t*)dst, n);
+    else
+        hipLaunchKernelGGL(from_f32_kernel<f16_t>, dim3(ew_grid(n)), dim3(256), 0, st, src, (const f16_t*)v1, (f16_t*)dst, n);
+}
+
+void rowdot(const void* a, const void* b, float* out, int rows, int D, int dtype, hipStream_t st) {
+    dim3 grid((rows + 3) / 4);
+    if (dtype == TRITT_F32)
+        hipLaunchKernelGGL(rowdot_kernel<float>, grid, dim3(256), 0, st, (const float*)a, (const float*)b, out, rows, D);
+    else if (dtype == TRITT_BF16)
+        hipLaunchKernelGGL(rowdot_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)a, (const bf16_t*)b, out, rows, D);
+    else
+        hipLaunchKernelGGL(rowdot_kernel<f16_t>, grid, dim3(256), 0, st, (const f16_t*)a, (const f16_t*)b, out, rows, D);
+}
+
+// fp32 views of the five inputs: in place for fp32 tensors, scratch copies otherwise; u = SiLU(v1).
+struct F32Inputs {
+    const float *q, *k1, *k2, *u, *v2;
+};
+F32Inputs plan_inputs(Arena& ar, const void* q, const void* k1, const void* k2, const void* v2, size_t n, int dtype,
+                      float** copies /* [4] scratch or null */, float** u) {
+    F32Inputs r{};
+    *u = ar.take<float>(n);
+    r.u = *u;
+    if (dtype == TRITT_F32) {
+        r.q = (const float*)q; r.k1 = (const float*)k1; r.k2 = (const float*)k2; r.v2 = (const float*)v2;
+        for (int i = 0; i < 4; ++i) copies[i] = nullptr;
+    } else {
+        for (int i = 0; i < 4; ++i) copies[i] = ar.take<float>(n);
+        r.q = copies[0]; r.k1 = copies[1]; r.k2 = copies[2]; r.v2 = copies[3];
+    }
+    return r;
+}
+void fill_inputs(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, size_t n, int dtype,
+                 float* const* copies, float* u, hipStream_t st) {
+    to_f32<true>(v1, u, n, dtype, st);
+    if (dtype != TRITT_F32) {
+        to_f32<false>(q, copies[0], n, dtype, st);
+        to_f32<false>(k1, copies[1], n, dtype, st);
+        to_f32<false>(k2, copies[2], n, dtype, st);
+        to_f32<false>(v2, copies[3], n, dtype, st);
+    }
+}
+
+int clampw(int w, int T) { return w > T ? T : w; }
+
+// ---------------------------------------------------------------- triple-dot, fp32 VALU path
+int tdp_fwd_generic(Arena& ar, bool run, const void* q, const void* k1, const void* k2, const void* v1,
+                    const void* v2, void* o, float* lse, int B, int H, int T, int D, int dtype, float alpha,
+                    int causal, int w1, int w2, int kl, int kr, hipStream_t st) {
+    const size_t n = (size_t)B * H * T * D;
+    float *copies[4], *u;
+    F32Inputs in = plan_inputs(ar, q, k1, k2, v2, n, dtype, copies, &u);
+    float* o32 = dtype == TRITT_F32 ? (float*)o : ar.take<float>(n);
+    if (!run) return TRITT_OK;
+    fill_inputs(q, k1, k2, v1, v2, n, dtype, copies, u, st);
+    GenericTdpArgs a{};
+    a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
+    a.o = o32; a.lse = lse;
+    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha;
+    a.causal = causal; a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+    hipError_t e = generic_tdp_fwd(a, st);
+    if (e != hipSuccess) return (int)e;
+    if (dtype != TRITT_F32) from_f32(o32, nullptr, o, n, dtype, st);
+    return (int)hipGetLastError();
+}
+
+int tdp_bwd_generic(Arena& ar, bool run, const void* q, const void* k1, const void* k2, const void* v1,
+                    const void* v2, const void* o, const float* lse, const void* d_o, void* dq, void* dk1,
+                    void* dk2, void* dv1, void* dv2, int B, int H, int T, int D, int dtype, float alpha, int causal,
+                    int w1, int w2, int kl, int kr, hipStream_t st) {
+    const size_t n = (size_t)B * H * T * D;
+    float *copies[4], *u;
+    F32Inputs in = plan_inputs(ar, q, k1, k2, v2, n, dtype, copies, &u);
+    float* do32 = dtype == TRITT_F32 ? (float*)d_o : ar.take<float>(n);
+    float* delta = ar.take<float>((size_t)B * H * T);
+    float* du = ar.take<float>(n);
+    float *dq32 = (float*)dq, *dk132 = (float*)dk1, *dk232 = (float*)dk2, *dv232 = (float*)dv2;
+    if (dtype != TRITT_F32) {
+        dq32 = ar.take<float>(n); dk132 = ar.take<float>(n); dk232 = ar.take<float>(n); dv232 = ar.take<float>(n);
+    }
+    if (!run) return TRITT_OK;
+    fill_inputs(q, k1, k2, v1, v2, n, dtype, copies, u, st);
+    if (dtype != TRITT_F32) to_f32<false>(d_o, do32, n, dtype, st);
+    rowdot(d_o, o, delta, B * H * T, D, dtype, st);
+    GenericTdpArgs a{};
+    a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
+    a.lse_in = lse; a.d_o = do32; a.delta = delta;
+    a.dq = dq32; a.dk1 = dk132; a.dk2 = dk232; a.du = du; a.dv2 = dv232;
+    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha;
+    a.causal = causal; a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+    hipError_t e = generic_tdp_bwd(a, st);
+    if (e != hipSuccess) return (int)e;
+    from_f32(du, v1, dv1, n, dtype, st);
+    if (dtype != TRITT_F32) {
+        from_f32(dq32, nullptr, dq, n, dtype, st);
+        from_f32(dk132, nullptr, dk1, n, dtype, st);
+        from_f32(dk232, nullptr, dk2, n, dtype, st);
+        from_f32(dv232, nullptr, dv2, n, dtype, st);
+    }
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------- dot-product-sum
+int dps_fwd_impl(Arena& ar, bool run, const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                 void* o, float* lse, int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
+                 hipStream_t st) {
+    const size_t n = (size_t)B * H * T * D, rows = (size_t)B * H * T;
+    float *copies[4], *u;
+    F32Inputs in = plan_inputs(ar, q, k1, k2, v2, n, dtype, copies, &u);
+    float* o32 = dtype == TRITT_F32 ? (float*)o : ar.take<float>(n);
+    DpsArgs a{};
+    a.r = ar.take<float>(n);
+    a.w = ar.take<float>(n);
+    a.lse1 = ar.take<float>(rows);
+    if (!run) return TRITT_OK;
+    fill_inputs(q, k1, k2, v1, v2, n, dtype, copies, u, st);
+    a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
+    a.o = o32; a.lse = lse;
+    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal; a.k_diff = k_diff;
+    hipError_t e = dps_fwd(a, st);
+    if (e != hipSuccess) return (int)e;
+    if (dtype != TRITT_F32) from_f32(o32, nullptr, o, n, dtype, st);
+    return (int)hipGetLastError();
+}
+
+int dps_bwd_impl(Arena& ar, bool run, const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                 const void* o, const float* lse, const void* d_o, void* dq, void* dk1, void* dk2, void* dv1,
+                 void* dv2, int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
+                 hipStream_t st) {
+    const size_t n = (size_t)B * H * T * D, rows = (size_t)B * H * T;
+    float *copies[4], *u;
+    F32Inputs in = plan_inputs(ar, q, k1, k2, v2, n, dtype, copies, &u);
+    float* do32 = dtype == TRITT_F32 ? (float*)d_o : ar.take<float>(n);
+    DpsArgs a{};
+    a.r = ar.take<float>(n); a.w = ar.take<float>(n); a.dw = ar.take<float>(n); a.dr = ar.take<float>(n);
+    a.dk2_part = ar.take<float>(n);
+    a.lse1 = ar.take<float>(rows); a.delta = ar.take<float>(rows);
+    a.dlse1 = ar.take<float>(rows); a.delta1 = ar.take<float>(rows);
+    float* du = ar.take<float>(n);
+    float *dq32 = (float*)dq, *dk132 = (float*)dk1, *dk232 = (float*)dk2, *dv232 = (float*)dv2;
+    if (dtype != TRITT_F32) {
+        dq32 = ar.take<float>(n); dk132 = ar.take<float>(n); dk232 = ar.take<float>(n); dv232 = ar.take<float>(n);
+    }
+    if (!run) return TRITT_OK;
+    fill_inputs(q, k1, k2, v1, v2, n, dtype, copies, u, st);
+    if (dtype != TRITT_F32) to_f32<false>(d_o, do32, n, dtype, st);
+    rowdot(d_o, o, a.delta, (int)rows, D, dtype, st);
+    a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
+    a.lse = const_cast<float*>(lse); a.d_o = do32;
+    a.dq = dq32; a.dk1 = dk132; a.dk2 = dk232; a.du = du; a.dv2 = dv232;
+    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal; a.k_diff = k_diff;
+    hipError_t e = dps_bwd(a, st);
+    if (e != hipSuccess) return (int)e;
+    from_f32(du, v1, dv1, n, dtype, st);
+    if (dtype != TRITT_F32) {
+        from_f32(dq32, nullptr, dq, n, dtype, st);
+        from_f32(dk132, nullptr, dk1, n, dtype, st);
+        from_f32(dk232, nullptr, dk2, n, dtype, st);
+        from_f32(dv232, nullptr, dv2, n, dtype, st);
+    }
+    return (int)hipGetLastError();
+}
+
+bool any_null(std::initializer_list<const void*> ps) {
+    for (const void* p : ps)
+        if (!p) return true;
+    return false;
+}
+
+}  // namespace
+}  // namespace tritt
+
+using namespace tritt;
+
+extern "C" {
+
+int tritt_version(void) { return 100; }
+
+const char* tritt_status_string(int status) {
+    switch (status) {
+        case TRITT_OK: return "ok";
+        case TRITT_ERR_INVALID: return "invalid argument (null pointer, non-positive size, negative window or unknown dtype)";
+        case TRITT_ERR_HEAD_DIM: return "head dimension must be 16, 32, 64 or 128";
+        case TRITT_ERR_WORKSPACE: return "workspace missing or too small";
+        case TRITT_ERR_UNSUPPORTED: return "requested implementation does not support this configuration";
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "unknown status";
+}
+
+size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,
+                                     int kk_left, int kk_right, unsigned flags) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    Arena ar(nullptr);
+    tdp_fwd_generic(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f,
+                    causal, k1_window, k2_window, kk_left, kk_right, nullptr);
+    (void)flags;
+    return ar.bytes();
+}
+
+int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, void* o, float* lse,
+                  int B, int H, int T, int D, int dtype, float alpha, int causal, int k1_window, int k2_window,
+                  int kk_left, int kk_right, void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
+    if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
+    const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
+    if (flags & TRITT_FLAG_FORCE_MFMA) return TRITT_ERR_UNSUPPORTED;
+    const size_t need = tritt_tdp_fwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
+    if (need && (!workspace || workspace_bytes < need)) return TRITT_ERR_WORKSPACE;
+    Arena ar(workspace);
+    return tdp_fwd_generic(ar, true, q, k1, k2, v1, v2, o, lse, B, H, T, D, dtype, alpha, causal, w1, w2, kl, kr,
+                           (hipStream_t)stream);
+}
+
+size_t tritt_tdp_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,
+                                     int kk_left, int kk_right, unsigned flags) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    Arena ar(nullptr);
+    tdp_bwd_generic(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                    nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f, causal, k1_window, k2_window, kk_left, kk_right,
+                    nullptr);
+    (void)flags;
+    return ar.bytes();
+}
+
+int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, const void* o,
+                  const float* lse, const void* d_o, void* dq, void* dk1, void* dk2, void* dv1, void* dv2, int B, int H,
+                  int T, int D, int dtype, float alpha, int causal, int k1_window, int k2_window, int kk_left,
+                  int kk_right, void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
+    if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
+    const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
+    if (flags & TRITT_FLAG_FORCE_MFMA) return TRITT_ERR_UNSUPPORTED;
+    const size_t need = tritt_tdp_bwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
+    if (need && (!workspace || workspace_bytes < need)) return TRITT_ERR_WORKSPACE;
+    Arena ar(workspace);
+    return tdp_bwd_generic(ar, true, q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2, B, H, T, D, dtype, alpha,
+                           causal, w1, w2, kl, kr, (hipStream_t)stream);
+}
+
+size_t tritt_dps_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    Arena ar(nullptr);
+    dps_fwd_impl(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f, 1, T,
+                 nullptr);
+    (void)flags;
+    return ar.bytes();
+}
+
+int tritt_dps_fwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, void* o, float* lse,
+                  int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff, void* workspace,
+                  size_t workspace_bytes, unsigned flags, void* stream) {
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
+    if (causal && k_diff < 0) return TRITT_ERR_INVALID;
+    const size_t need = tritt_dps_fwd_workspace_bytes(B, H, T, D, dtype, flags);
+    if (!workspace || workspace_bytes < need) return TRITT_ERR_WORKSPACE;
+    Arena ar(workspace);
+    return dps_fwd_impl(ar, true, q, k1, k2, v1, v2, o, lse, B, H, T, D, dtype, alpha, causal, clampw(k_diff, T),
+                        (hipStream_t)stream);
+}
+
+size_t tritt_dps_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    Arena ar(nullptr);
+    dps_bwd_impl(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                 nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f, 1, T, nullptr);
+    (void)flags;
+    return ar.bytes();
+}
+
+int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, const void* o,
+                  const float* lse, const void* d_o, void* dq, void* dk1, void* dk2, void* dv1, void* dv2, int B, int H,
+                  int T, int D, int dtype, float alpha, int causal, int k_diff, void* workspace, size_t workspace_bytes,
+                  unsigned flags, void* stream) {
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
+    if (causal && k_diff < 0) return TRITT_ERR_INVALID;
+    const size_t need = tritt_dps_bwd_workspace_bytes(B, H, T, D, dtype, flags);
+    if (!workspace || workspace_bytes < need) return TRITT_ERR_WORKSPACE;
+    Arena ar(workspace);
+    return dps_bwd_impl(ar, true, q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2, B, H, T, D, dtype, alpha,
+                        causal, clampw(k_diff, T), (hipStream_t)stream);
+}
+
+}  // extern "C"

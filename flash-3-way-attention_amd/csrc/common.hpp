@@ -1,0 +1,71 @@
+// Shared device helpers for the trittention HIP kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tritt {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct bf16_t {
+    uint16_t bits;
+};
+using f16_t = _Float16;
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+__device__ __forceinline__ float to_float(f16_t v) { return (float)v; }
+
+// round-to-nearest-even fp32 -> bf16 (NaN kept quiet)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_float(float v);
+template <>
+__device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return bf16_t{f32_to_bf16_bits(v)}; }
+template <>
+__device__ __forceinline__ f16_t from_float<f16_t>(float v) { return (f16_t)v; }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float silu_grad_f(float x) {
+    float s = 1.0f / (1.0f + __expf(-x));
+    return s * (1.0f + x * (1.0f - s));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Window parameters of the triple-dot causal mask, expressed for a "staged"
+// index a and an "owner" index b (a = j, b = k in the natural orientation):
+//   valid  <=>  a<=q, b<=q, q<=a+wa, q<=b+wb, b<=a+lab, a<=b+rab
+struct TdpMask {
+    int causal;
+    int wa, wb, lab, rab;
+};
+
+__device__ __forceinline__ bool tdp_valid(const TdpMask& m, int q, int a, int b) {
+    if (!m.causal) return true;
+    return (a <= q) & (b <= q) & (q <= a + m.wa) & (q <= b + m.wb) & (b <= a + m.lab) & (a <= b + m.rab);
+}
+
+}  // namespace tritt

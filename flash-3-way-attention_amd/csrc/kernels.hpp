@@ -1,0 +1,41 @@
+// Internal launch interfaces between capi.hip and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+namespace tritt {
+
+// fp32 [BH, T, D] operands of the VALU triple-dot kernels (u = SiLU(V1)).
+struct GenericTdpArgs {
+    const float *q, *k1, *k2, *u, *v2;
+    float* o;            // forward output
+    float* lse;          // forward output [BH, T]
+    const float* lse_in; // backward input
+    const float* d_o;    // backward input
+    const float* delta;  // backward input [BH, T] = rowsum(dO * O)
+    float *dq, *dk1, *dk2, *du, *dv2;
+    int BH, T, D;
+    float alpha;
+    int causal, k1_window, k2_window, kk_left, kk_right;
+};
+hipError_t generic_tdp_fwd(const GenericTdpArgs& a, hipStream_t st);
+hipError_t generic_tdp_bwd(const GenericTdpArgs& a, hipStream_t st);
+
+// fp32 operands of the dot-product-sum kernels (two chained attention passes).
+struct DpsArgs {
+    const float *q, *k1, *k2, *u, *v2;
+    float* o;
+    float* lse;          // forward output / backward input (natural log) [BH, T]
+    const float* d_o;
+    const float* o_in;
+    float *dq, *dk1, *dk2, *du, *dv2;
+    // scratch, all fp32: r, w, dw, dr, dk2_part [BH,T,D]; lse1, delta, dlse1, delta1 [BH,T]
+    float *r, *w, *dw, *dr, *dk2_part, *lse1, *delta, *dlse1, *delta1;
+    int BH, T, D;
+    float alpha;
+    int causal, k_diff;
+};
+hipError_t dps_fwd(const DpsArgs& a, hipStream_t st);
+hipError_t dps_bwd(const DpsArgs& a, hipStream_t st);
+
+}  // namespace tritt

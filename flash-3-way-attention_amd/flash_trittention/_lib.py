@@ -1,0 +1,94 @@
+"""ctypes binding of libtrittention_hip.so (C ABI: include/trittention_hip.h).
+
+PyTorch is used only for device memory and the current HIP stream; tensors
+cross the boundary as raw pointers.  There is no fallback: if the library is
+missing every call raises.
+"""
+import ctypes
+import os
+import subprocess
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtrittention_hip.so")
+CSRC_DIR = os.path.join(os.path.dirname(_HERE), "csrc")
+
+TRITT_F32, TRITT_BF16, TRITT_F16 = 0, 1, 2
+FLAG_AUTO, FLAG_FORCE_GENERIC, FLAG_FORCE_MFMA = 0, 1, 2
+
+_DTYPES = {torch.float32: TRITT_F32, torch.bfloat16: TRITT_BF16, torch.float16: TRITT_F16}
+
+_vp, _i, _f, _sz, _u = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_uint
+
+_PROTOS = {
+    "tritt_version": (_i, []),
+    "tritt_status_string": (ctypes.c_char_p, [_i]),
+    "tritt_tdp_fwd_workspace_bytes": (_sz, [_i] * 10 + [_u]),
+    "tritt_tdp_fwd": (_i, [_vp] * 7 + [_i] * 5 + [_f] + [_i] * 5 + [_vp, _sz, _u, _vp]),
+    "tritt_tdp_bwd_workspace_bytes": (_sz, [_i] * 10 + [_u]),
+    "tritt_tdp_bwd": (_i, [_vp] * 13 + [_i] * 5 + [_f] + [_i] * 5 + [_vp, _sz, _u, _vp]),
+    "tritt_dps_fwd_workspace_bytes": (_sz, [_i] * 5 + [_u]),
+    "tritt_dps_fwd": (_i, [_vp] * 7 + [_i] * 5 + [_f] + [_i] * 2 + [_vp, _sz, _u, _vp]),
+    "tritt_dps_bwd_workspace_bytes": (_sz, [_i] * 5 + [_u]),
+    "tritt_dps_bwd": (_i, [_vp] * 13 + [_i] * 5 + [_f] + [_i] * 2 + [_vp, _sz, _u, _vp]),
+}
+
+_lib = None
+
+
+def build(verbose: bool = False) -> str:
+    """Compile the HIP sources for gfx950 (always recompiles)."""
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.check_call(["make", "-C", CSRC_DIR, "-B", "-j8"], stdout=out, stderr=out)
+    return LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {CSRC_DIR}` "
+                "(there is no fallback implementation)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _PROTOS.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def exported_symbols():
+    return list(_PROTOS)
+
+
+def dtype_code(dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype}; expected float32, bfloat16 or float16") from None
+
+
+def check(status: int, what: str):
+    if status != 0:
+        msg = lib().tritt_status_string(status).decode()
+        raise RuntimeError(f"{what} failed: {msg} (status {status})")
+
+
+def require_gpu(t: torch.Tensor, what: str):
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: tensors must live on a GPU (got {t.device}); "
+                           "this library has no CPU implementation")
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def workspace(nbytes: int, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)

@@ -1,0 +1,107 @@
+"""Triple-dot-product trittention on MI355X.
+
+Mirrors the reference's ``FlashTrittention`` autograd Function and the public
+``flash_trittention`` (triple_dot_product/flash_trittention.py:14-139 forward,
+:141-393 backward, :396-438 entry point): same argument order, defaults,
+return values and ValueErrors.  The work itself is one call into the HIP
+library per direction (SiLU, Delta and SiLU' are done inside it).
+"""
+import warnings
+
+import torch
+
+from .. import _lib
+from .utils import process_masking_variables
+
+
+def _validate(Q, others):
+    for name, t in others:
+        if t.shape != Q.shape:
+            raise ValueError(f"{name} shape {tuple(t.shape)} does not match Q shape {tuple(Q.shape)}")
+        if t.dtype != Q.dtype:
+            raise ValueError(f"{name} dtype {t.dtype} does not match Q dtype {Q.dtype}")
+        if t.device != Q.device:
+            raise ValueError(f"{name} device {t.device} does not match Q device {Q.device}")
+    if Q.dim() != 4:
+        raise ValueError(f"expected [batch, heads, seq_len, head_dim] tensors, got shape {tuple(Q.shape)}")
+    head_dim = Q.shape[-1]
+    if head_dim <= 0 or head_dim & (head_dim - 1):
+        raise ValueError(f"head_dim must be a power of 2, got {head_dim}")
+    if head_dim not in (16, 32, 64, 128):
+        raise ValueError(f"head_dim must be one of 16, 32, 64, 128, got {head_dim}")
+    _lib.dtype_code(Q.dtype)
+
+
+class FlashTrittention(torch.autograd.Function):
+    # set by tests/bench to pin an implementation: _lib.FLAG_AUTO / FORCE_GENERIC / FORCE_MFMA
+    impl_flags = _lib.FLAG_AUTO
+
+    @staticmethod
+    def forward(ctx, Q, K1, K2, V1, V2, softmax_scale, kk_left, kk_right, k1_window, k2_window, causal,
+                convert_to_float32):
+        _validate(Q, (("K1", K1), ("K2", K2), ("V1", V1), ("V2", V2)))
+        _lib.require_gpu(Q, "flash_trittention")
+        B, H, T, D = Q.shape
+        Q, K1, K2, V1, V2 = (t.contiguous() for t in (Q, K1, K2, V1, V2))
+        k1_window, k2_window, kk_left, kk_right = process_masking_variables(T, k1_window, k2_window, kk_left, kk_right)
+        causal = bool(causal)
+        flags = FlashTrittention.impl_flags
+        lib = _lib.lib()
+        code = _lib.dtype_code(Q.dtype)
+        O = torch.empty_like(Q)
+        LSE = torch.empty((B, H, T), dtype=torch.float32, device=Q.device)
+        with torch.cuda.device(Q.device):
+            need = lib.tritt_tdp_fwd_workspace_bytes(B, H, T, D, code, int(causal), k1_window, k2_window, kk_left,
+                                                     kk_right, flags)
+            ws = _lib.workspace(need, Q.device)
+            st = lib.tritt_tdp_fwd(_lib.ptr(Q), _lib.ptr(K1), _lib.ptr(K2), _lib.ptr(V1), _lib.ptr(V2), _lib.ptr(O),
+                                   _lib.ptr(LSE), B, H, T, D, code, float(softmax_scale), int(causal), k1_window,
+                                   k2_window, kk_left, kk_right, _lib.ptr(ws), ws.numel(), flags,
+                                   _lib.stream_ptr(Q.device))
+        _lib.check(st, "tritt_tdp_fwd")
+        ctx.save_for_backward(Q, K1, K2, V1, V2, O, LSE)
+        ctx.softmax_scale = float(softmax_scale)
+        ctx.windows = (k1_window, k2_window, kk_left, kk_right)
+        ctx.causal = causal
+        ctx.flags = flags
+        return O
+
+    @staticmethod
+    def backward(ctx, dO):
+        Q, K1, K2, V1, V2, O, LSE = ctx.saved_tensors
+        B, H, T, D = Q.shape
+        if dO.dtype != Q.dtype:
+            dO = dO.to(Q.dtype)
+        dO = dO.contiguous()
+        k1_window, k2_window, kk_left, kk_right = ctx.windows
+        lib = _lib.lib()
+        code = _lib.dtype_code(Q.dtype)
+        dq, dk1, dk2, dv1, dv2 = (torch.empty_like(Q) for _ in range(5))
+        with torch.cuda.device(Q.device):
+            need = lib.tritt_tdp_bwd_workspace_bytes(B, H, T, D, code, int(ctx.causal), k1_window, k2_window, kk_left,
+                                                     kk_right, ctx.flags)
+            ws = _lib.workspace(need, Q.device)
+            st = lib.tritt_tdp_bwd(_lib.ptr(Q), _lib.ptr(K1), _lib.ptr(K2), _lib.ptr(V1), _lib.ptr(V2), _lib.ptr(O),
+                                   _lib.ptr(LSE), _lib.ptr(dO), _lib.ptr(dq), _lib.ptr(dk1), _lib.ptr(dk2),
+                                   _lib.ptr(dv1), _lib.ptr(dv2), B, H, T, D, code, ctx.softmax_scale, int(ctx.causal),
+                                   k1_window, k2_window, kk_left, kk_right, _lib.ptr(ws), ws.numel(), ctx.flags,
+                                   _lib.stream_ptr(Q.device))
+        _lib.check(st, "tritt_tdp_bwd")
+        return dq, dk1, dk2, dv1, dv2, None, None, None, None, None, None, None
+
+
+def flash_trittention(q, k1, k2, v1, v2, softmax_scale=1 / 8, kk_left=1, kk_right=1, k1_window=1, k2_window=1,
+                      causal=True, convert_to_float32=False, input_precision=None):
+    """Triple-dot-product 3-way attention; returns O [B, H, T, D].
+
+    Window arguments: ``None`` (or any value >= seq_len) disables a window; note that the
+    literal defaults are 1, a narrow band, exactly as in the reference.  ``convert_to_float32``
+    is accepted for compatibility: scores and softmax are always computed in fp32 here.
+    ``input_precision`` is accepted and ignored with a warning, as in the reference.
+    """
+    if input_precision is not None:
+        warnings.warn(
+            "flash_trittention: `input_precision` is currently unused and has no effect "
+            f"(got {input_precision!r}).", stacklevel=2)
+    return FlashTrittention.apply(q, k1, k2, v1, v2, softmax_scale, kk_left, kk_right, k1_window, k2_window, causal,
+                                  convert_to_float32)

@@ -1,0 +1,115 @@
+/* trittention_hip.h — C ABI of libtrittention_hip.so (MI355X / gfx950).
+ *
+ * The library implements the "trittention" (3-way attention) hot path of
+ * flash-3-way-attention with hand-written HIP kernels.  Every entry point
+ * takes plain device pointers, sizes and a HIP stream; no framework types
+ * cross this boundary.  All tensors are contiguous row-major [B, H, T, D].
+ * `lse` is [B, H, T] fp32 (natural-log logsumexp of the scaled, masked
+ * scores of each query row).
+ *
+ * Each function names the reference interface it replaces (paths relative
+ * to the reference repository's src/flash_trittention/).
+ *
+ * Return value: 0 on success; a negative TRITT_ERR_* code when the
+ * arguments are rejected before anything is launched; a positive value is
+ * the hipError_t reported by the launch.  Nothing is allocated or freed by
+ * these calls: scratch memory is passed in by the caller (`workspace`), its
+ * required size is returned by the matching *_workspace_bytes function.
+ * Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ * null stream) and the calls do not synchronise.
+ */
+#ifndef TRITTENTION_HIP_H
+#define TRITTENTION_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of q,k1,k2,v1,v2,o,dO and of the five gradients */
+enum { TRITT_F32 = 0, TRITT_BF16 = 1, TRITT_F16 = 2 };
+
+enum {
+    TRITT_OK = 0,
+    TRITT_ERR_INVALID = -1,     /* null pointer, non-positive size, bad dtype              */
+    TRITT_ERR_HEAD_DIM = -2,    /* D not one of 16, 32, 64, 128                            */
+    TRITT_ERR_WORKSPACE = -3,   /* workspace missing or smaller than *_workspace_bytes     */
+    TRITT_ERR_UNSUPPORTED = -4  /* requested implementation cannot run this configuration */
+};
+
+/* `flags` bits */
+enum {
+    TRITT_FLAG_AUTO = 0,
+    TRITT_FLAG_FORCE_GENERIC = 1, /* use the fp32 VALU kernels even where an MFMA kernel exists */
+    TRITT_FLAG_FORCE_MFMA = 2     /* fail with TRITT_ERR_UNSUPPORTED instead of falling back    */
+};
+
+/* Library version (major*10000 + minor*100 + patch) and a static, human
+ * readable description of a return code. */
+int tritt_version(void);
+const char* tritt_status_string(int status);
+
+/* ---- triple-dot-product:  s[q,j,k] = alpha * sum_d Q[q,d] K1[j,d] K2[k,d] ----------------
+ * O[q] = sum_{j,k} softmax_{(j,k)}(s[q]) * SiLU(V1[j]) * V2[k].
+ * causal != 0 masks (reference triple_dot_product/trittention_pytorch.py:68-75)
+ *   j>q | k>q | q>j+k1_window | q>k+k2_window | j+kk_left<k | k+kk_right<j ;
+ * pass T (or more) for a window to disable it.  causal == 0: no mask, windows ignored.
+ *
+ * tritt_tdp_fwd replaces FlashTrittention.forward + the _tritt_fwd launch
+ *   (triple_dot_product/flash_trittention.py:16-139, kernels/fwd.py:9-225): it also
+ *   applies SiLU to V1 itself and writes the final lse (the reference's M + log L).
+ * tritt_tdp_bwd replaces FlashTrittention.backward and its five launches
+ *   (triple_dot_product/flash_trittention.py:141-393, kernels/bwd_{dq,dk1,dk2,dv1,dv2}.py),
+ *   including Delta = rowsum(dO*O) and the SiLU' factor on dV1.
+ */
+size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
+                                     int k1_window, int k2_window, int kk_left, int kk_right,
+                                     unsigned flags);
+int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                  void* o, float* lse,
+                  int B, int H, int T, int D, int dtype, float alpha, int causal,
+                  int k1_window, int k2_window, int kk_left, int kk_right,
+                  void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
+size_t tritt_tdp_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
+                                     int k1_window, int k2_window, int kk_left, int kk_right,
+                                     unsigned flags);
+int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                  const void* o, const float* lse, const void* d_o,
+                  void* dq, void* dk1, void* dk2, void* dv1, void* dv2,
+                  int B, int H, int T, int D, int dtype, float alpha, int causal,
+                  int k1_window, int k2_window, int kk_left, int kk_right,
+                  void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
+/* ---- dot-product-sum:  s[q,s,t] = alpha * (K2[t].Q[q] + K1[s].K2[t]) ---------------------
+ * O[q] = sum_{s,t} softmax_{(s,t)}(s[q]) * SiLU(V1[s]) * V2[t].
+ * causal != 0 keeps s <= t <= q and t - s <= k_diff
+ *   (reference dot_product_sum/trittention_pytorch.py:47-51); causal == 0: no mask.
+ *
+ * tritt_dps_fwd replaces TrittentionTritonFunction.forward + _tritt_fwd
+ *   (dot_product_sum/trittention_triton.py:17-125, kernels/fwd_kernel.py:225-375);
+ *   `lse` is the tensor that function returns as `m`.
+ * tritt_dps_bwd replaces TrittentionTritonFunction.backward with
+ *   _tritt_bwd_preprocess, _tritt_bwd_dq and _tritt_bwd_dk_dv
+ *   (dot_product_sum/trittention_triton.py:127-359, kernels/bwd_preprocess.py:6,
+ *   kernels/bwd_dq_kernel.py:30, kernels/bwd_dk1_dv1_kernel.py:31).  It uses no atomics:
+ *   results are bitwise reproducible from run to run.
+ */
+size_t tritt_dps_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags);
+int tritt_dps_fwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                  void* o, float* lse,
+                  int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
+                  void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
+size_t tritt_dps_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags);
+int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                  const void* o, const float* lse, const void* d_o,
+                  void* dq, void* dk1, void* dk2, void* dv1, void* dv2,
+                  int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
+                  void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRITTENTION_HIP_H */

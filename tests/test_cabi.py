@@ -1,0 +1,96 @@
+"""CPU-side checks of the boundary: the C-ABI library loads, exports every symbol that
+include/trittention_hip.h declares, rejects bad arguments before launching anything, and the
+Python host mirrors the reference's error behaviour.  No kernel runs here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from flash_trittention import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "trittention_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tritt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.lib()
+    names = declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_lib.exported_symbols()) == names
+
+
+def test_version_and_status_strings():
+    lib = _lib.lib()
+    assert lib.tritt_version() >= 100
+    assert lib.tritt_status_string(0) == b"ok"
+    assert b"head dimension" in lib.tritt_status_string(-2)
+
+
+def test_workspace_queries_scale_with_problem():
+    lib = _lib.lib()
+    a = lib.tritt_tdp_bwd_workspace_bytes(1, 2, 64, 32, _lib.TRITT_F32, 1, 64, 64, 64, 64, 1)
+    b = lib.tritt_tdp_bwd_workspace_bytes(2, 2, 64, 32, _lib.TRITT_F32, 1, 64, 64, 64, 64, 1)
+    assert 0 < a < b
+    assert lib.tritt_tdp_fwd_workspace_bytes(1, 2, 64, 24, _lib.TRITT_F32, 1, 64, 64, 64, 64, 0) == 0  # bad D
+    assert lib.tritt_dps_fwd_workspace_bytes(1, 2, 64, 32, _lib.TRITT_BF16, 0) > 0
+
+
+def test_argument_rejection_happens_before_any_launch():
+    lib = _lib.lib()
+    null = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(256)  # never dereferenced: rejected first
+    args7 = [one] * 7
+    assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 24, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -2
+    assert lib.tritt_tdp_fwd(*args7, 0, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
+    assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 7, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
+    assert lib.tritt_tdp_fwd(null, *args7[1:], 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
+    assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, -1, 16, 16, 16, null, 0, 0, null) == -1
+    assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 1, null) == -3  # no workspace
+    assert lib.tritt_dps_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, 16, null, 0, 0, null) == -3
+    assert lib.tritt_dps_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, -2, one, 1 << 30, 0, null) == -1
+
+
+def test_python_host_validation_matches_reference_errors():
+    from flash_trittention import TrittentionTriton, flash_trittention
+
+    q, k1, k2, v1, v2 = (torch.randn(2, 2, 32, 32) for _ in range(5))
+    with pytest.raises(ValueError):
+        flash_trittention(q, k1, k2, v1, v2[:, :, :16])
+    with pytest.raises(ValueError):
+        flash_trittention(q, k1, k2, v1, v2.double())
+    with pytest.raises(ValueError):
+        flash_trittention(*(torch.randn(2, 2, 32, 24) for _ in range(5)))
+    with pytest.raises(ValueError):
+        TrittentionTriton()(q, k1, k2, v1, v2[:, :, :16])
+    # well-formed CPU tensors: the product has no CPU path and says so
+    with pytest.raises(RuntimeError, match="GPU"):
+        flash_trittention(q, k1, k2, v1, v2)
+    with pytest.raises(RuntimeError, match="GPU"):
+        TrittentionTriton()(q, k1, k2, v1, v2)
+
+
+def test_lazy_package_exports():
+    import flash_trittention as ft
+
+    assert ft.__all__ == ["flash_trittention", "TrittentionTriton"]
+    assert callable(ft.flash_trittention) and callable(ft.TrittentionTriton)
+    with pytest.raises(AttributeError):
+        ft.nope
+
+
+def test_product_never_imports_oracle():
+    pkg = os.path.join(ROOT, "flash-3-way-attention_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)

@@ -1,0 +1,109 @@
+"""GPU parity: dot-product-sum trittention (HIP, through the C ABI) vs the CPU oracle.
+Case grid follows the reference's tests/test_dot_product_sum.py:70-142."""
+import math
+
+import pytest
+import torch
+
+from oracle import trittention_oracle as orc
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+FP32 = dict(rtol=1e-4, atol=2e-5)
+LOWP = dict(rtol=5e-2, atol=2e-2)
+
+
+def check_all(inputs, alpha, causal, k_diff, tol=FP32, rel=1e-4, factorised=False):
+    z, lse, grads = util.oracle_dps(inputs, alpha, causal, k_diff, factorised=factorised)
+    out, m, g = util.run_dps(inputs, alpha, causal, k_diff)
+    util.assert_close("out", out, z, **tol)
+    util.assert_close("m", m, lse, rtol=1e-3 if tol is LOWP else 1e-5, atol=2e-2 if tol is LOWP else 1e-4)
+    assert util.rel_err(out, z) <= rel
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_close(name, a, b, **tol)
+        assert util.rel_err(a, b) <= rel, (name, util.rel_err(a, b))
+
+
+@pytest.mark.parametrize("seq_len", [33, 64, 100])
+@pytest.mark.parametrize("causal", [True, False])
+def test_forward_and_backward_fp32(seq_len, causal):
+    print(f"case dps fp32 T={seq_len} causal={causal}", flush=True)
+    inputs = orc.make_inputs(2, 2, seq_len, 32, torch.float32, seed=seq_len + 1)
+    check_all(inputs, 1 / 8, causal, seq_len)
+
+
+@pytest.mark.parametrize("k_diff", [0, 2, 8])
+def test_narrow_k_diff_causal(k_diff):
+    print(f"case dps k_diff={k_diff}", flush=True)
+    inputs = orc.make_inputs(2, 2, 64, 32, torch.float32, seed=9)
+    check_all(inputs, 1 / 8, True, k_diff)
+
+
+@pytest.mark.parametrize("D", [16, 64, 128])
+def test_head_dims_fp32(D):
+    inputs = orc.make_inputs(1, 2, 80, D, torch.float32, seed=D + 1)
+    check_all(inputs, 1 / math.sqrt(D), True, 80)
+
+
+def test_large_logits_no_overflow():
+    inputs = orc.make_inputs(2, 2, 64, 32, torch.float32, seed=12)
+    inputs[1] = inputs[1] * 8.0
+    inputs[2] = inputs[2] * 8.0
+    z, lse, grads = util.oracle_dps(inputs, 1 / 8, True, 64)
+    out, m, g = util.run_dps(inputs, 1 / 8, True, 64)
+    assert torch.isfinite(out).all()
+    util.assert_close("out", out, z, rtol=1e-3, atol=1e-4)
+    for name, a, b in zip(util.NAMES, g, grads):
+        assert torch.isfinite(a).all(), name
+        util.assert_close(name, a, b, rtol=2e-3, atol=2e-3)
+
+
+def test_non_contiguous_inputs():
+    g = torch.Generator().manual_seed(13)
+    q, v1, v2, do = (torch.randn(2, 4, 64, 32, generator=g) for _ in range(4))
+    k1 = torch.randn(2, 64, 4, 32, generator=g).transpose(1, 2)
+    k2 = torch.randn(2, 64, 4, 32, generator=g).transpose(1, 2)
+    inputs = [q, k1, k2, v1, v2, do]
+    z, _, grads = util.oracle_dps([t.contiguous() for t in inputs], 1 / 8, True, 64)
+    out, m, g_ = util.run_dps(inputs, 1 / 8, True, 64)
+    util.assert_close("out", out, z, **FP32)
+    for name, a, b in zip(util.NAMES, g_, grads):
+        util.assert_close(name, a, b, **FP32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_lowp_forward_backward(dtype):
+    inputs = orc.make_inputs(2, 2, 256, 64, dtype, seed=14)
+    check_all(inputs, 1 / 8, True, 256, tol=LOWP, rel=2e-2)
+
+
+def test_config4_bf16_T1024():
+    """B=4 H=8 T=1024 D=64 bf16 causal.  Oracle: the factorised form (cross-checked against the
+    dense cube on the CPU at small T), on a subset of heads to keep the CPU time bounded."""
+    inputs = orc.make_inputs(4, 8, 1024, 64, torch.bfloat16, seed=15)
+    out, m, g = util.run_dps(inputs, 1 / 8, True, 1024)
+    for (b, h) in ((0, 0), (1, 3), (3, 7)):
+        sub = [t[b:b + 1, h:h + 1] for t in inputs]
+        z, lse, grads = util.oracle_dps(sub, 1 / 8, True, 1024, factorised=True)
+        util.assert_close("out", out[b:b + 1, h:h + 1], z, **LOWP)
+        util.assert_close("m", m[b:b + 1, h:h + 1], lse, rtol=1e-3, atol=2e-2)
+        for name, a, ref in zip(util.NAMES, g, grads):
+            util.assert_close(name, a[b:b + 1, h:h + 1], ref, **LOWP)
+
+
+def test_bitwise_reproducible():
+    inputs = orc.make_inputs(1, 2, 200, 64, torch.bfloat16, seed=16)
+    a = util.run_dps(inputs, 1 / 8, True, 200)
+    b = util.run_dps(inputs, 1 / 8, True, 200)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    for x, y in zip(a[2], b[2]):
+        assert torch.equal(x, y)
+
+
+def test_rejects_mismatched_shapes():
+    from flash_trittention import TrittentionTriton
+
+    q, k1, k2, v1, v2, _ = (t.cuda() for t in orc.make_inputs(2, 2, 32, 32))
+    with pytest.raises(ValueError):
+        TrittentionTriton()(q, k1, k2, v1, v2[:, :, :16, :].contiguous())

@@ -1,0 +1,142 @@
+"""GPU parity: triple-dot-product trittention (HIP, through the C ABI) vs the CPU oracle.
+
+Tolerances: fp32 tensors 1e-4 relative (rtol 1e-4 with a small atol, and
+max|err|/max|ref| <= 1e-4); bf16/fp16 tensors atol 2e-2 / rtol 5e-2 — the
+bars the task states.  The case grid follows the reference's own tests
+(tests/test_triple_dot_product.py:52-182)."""
+import math
+
+import pytest
+import torch
+
+from oracle import trittention_oracle as orc
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+FP32 = dict(rtol=1e-4, atol=2e-5)
+LOWP = dict(rtol=5e-2, atol=2e-2)
+
+
+def check_all(inputs, alpha, causal, windows=(None,) * 4, tol=FP32, rel=1e-4):
+    z, lse, grads = util.oracle_tdp(inputs, alpha, causal, windows)
+    out, g = util.run_tdp(inputs, alpha, causal, windows)
+    util.assert_close("out", out, z, **tol)
+    assert util.rel_err(out, z) <= rel, util.rel_err(out, z)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_close(name, a, b, **tol)
+        assert util.rel_err(a, b) <= rel, (name, util.rel_err(a, b))
+
+
+@pytest.mark.parametrize("seq_len", [33, 64, 100])
+@pytest.mark.parametrize("causal", [True, False])
+def test_forward_and_backward_fp32(seq_len, causal):
+    print(f"case fp32 T={seq_len} causal={causal}", flush=True)
+    inputs = orc.make_inputs(2, 2, seq_len, 32, torch.float32, seed=seq_len)
+    check_all(inputs, 1 / 8, causal)
+
+
+@pytest.mark.parametrize("seq_len", [64, 100])
+@pytest.mark.parametrize("windows", [(8, 8, 4, 4), (5, 3, 4, 1), (2, 70, 0, 3)])
+def test_narrow_windows_causal(seq_len, windows):
+    print(f"case windows T={seq_len} {windows}", flush=True)
+    inputs = orc.make_inputs(2, 2, seq_len, 32, torch.float32, seed=7)
+    check_all(inputs, 1 / 8, True, windows)
+
+
+def test_config1_forward_fp32():
+    """B=1 H=2 T=64 D=32 fp32, alpha = 1/sqrt(D), causal: output within 1e-4 relative."""
+    inputs = orc.make_inputs(1, 2, 64, 32, torch.float32, seed=1)
+    alpha = 1 / math.sqrt(32)
+    z, lse, _ = util.oracle_tdp(inputs, alpha, True)
+    out, _ = util.run_tdp(inputs, alpha, True, backward=False)
+    util.assert_close("out", out, z, **FP32)
+    assert util.rel_err(out, z) <= 1e-4
+
+
+@pytest.mark.parametrize("D", [16, 64, 128])
+def test_head_dims_fp32(D):
+    print(f"case fp32 D={D}", flush=True)
+    inputs = orc.make_inputs(1, 2, 48, D, torch.float32, seed=D)
+    check_all(inputs, 1 / math.sqrt(D), True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_config2_lowp_forward_backward(dtype):
+    """B=2 H=4 T=256 D=64, 16-bit tensors with fp32 accumulation, all five gradients."""
+    print(f"case config2 {dtype}", flush=True)
+    inputs = orc.make_inputs(2, 4, 256, 64, dtype, seed=2)
+    check_all(inputs, 1 / 8, True, tol=LOWP, rel=2e-2)
+
+
+def test_forward_fp16_loose():
+    inputs = orc.make_inputs(2, 2, 64, 32, torch.float16, seed=3)
+    z, _, _ = util.oracle_tdp(inputs, 1 / 8, True)
+    out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False)
+    util.assert_close("out", out, z, **LOWP)
+
+
+def test_lse_matches_oracle():
+    from flash_trittention.triple_dot_product.flash_trittention import FlashTrittention
+
+    inputs = orc.make_inputs(1, 2, 40, 32, torch.float32, seed=4)
+    z, lse, _ = util.oracle_tdp(inputs, 0.2, True)
+
+    class Ctx:
+        def save_for_backward(self, *t):
+            self.saved = t
+
+    ctx = Ctx()
+    FlashTrittention.forward(ctx, *(t.cuda() for t in inputs[:5]), 0.2, None, None, None, None, True, False)
+    util.assert_close("lse", ctx.saved[6].cpu(), lse, rtol=1e-5, atol=1e-5)
+
+
+def test_bitwise_reproducible():
+    inputs = orc.make_inputs(1, 2, 96, 64, torch.bfloat16, seed=5)
+    a = util.run_tdp(inputs, 1 / 8, True)
+    b = util.run_tdp(inputs, 1 / 8, True)
+    assert torch.equal(a[0], b[0])
+    for x, y in zip(a[1], b[1]):
+        assert torch.equal(x, y)
+
+
+def test_non_contiguous_inputs():
+    g = torch.Generator().manual_seed(11)
+    q, v1, v2, do = (torch.randn(2, 4, 64, 32, generator=g) for _ in range(4))
+    k1 = torch.randn(2, 64, 4, 32, generator=g).transpose(1, 2)
+    k2 = torch.randn(2, 64, 4, 32, generator=g).transpose(1, 2)
+    inputs = [q, k1, k2, v1, v2, do]
+    z, _, grads = util.oracle_tdp([t.contiguous() for t in inputs], 1 / 8, True)
+    out, g_ = util.run_tdp(inputs, 1 / 8, True)
+    util.assert_close("out", out, z, **FP32)
+    for name, a, b in zip(util.NAMES, g_, grads):
+        util.assert_close(name, a, b, **FP32)
+
+
+def test_rejects_mismatched_shapes():
+    from flash_trittention import flash_trittention
+
+    q, k1, k2, v1, v2, _ = (t.cuda() for t in orc.make_inputs(2, 2, 32, 32))
+    with pytest.raises(ValueError):
+        flash_trittention(q, k1, k2, v1, v2[:, :, :16, :].contiguous())
+    with pytest.raises(ValueError):
+        flash_trittention(q, k1, k2, v1, v2.half())
+
+
+def test_rejects_non_pow2_head_dim():
+    from flash_trittention import flash_trittention
+
+    q, k1, k2, v1, v2, _ = (t.cuda() for t in orc.make_inputs(2, 2, 32, 24))
+    with pytest.raises(ValueError):
+        flash_trittention(q, k1, k2, v1, v2)
+
+
+def test_input_precision_warns_and_is_ignored():
+    from flash_trittention import flash_trittention
+
+    q, k1, k2, v1, v2, _ = (t.cuda() for t in orc.make_inputs(1, 1, 16, 16))
+    with pytest.warns(UserWarning):
+        a = flash_trittention(q, k1, k2, v1, v2, k1_window=None, k2_window=None, kk_left=None, kk_right=None,
+                              input_precision="ieee")
+    b = flash_trittention(q, k1, k2, v1, v2, k1_window=None, k2_window=None, kk_left=None, kk_right=None)
+    assert torch.equal(a, b)

@@ -1,0 +1,78 @@
+"""Shared helpers for the GPU parity tests: seeded CPU inputs, oracle results,
+and runners that go through the Python host -> ctypes -> C ABI -> HIP path."""
+import torch
+
+from oracle import trittention_oracle as orc
+
+NAMES = ("dq", "dk1", "dk2", "dv1", "dv2")
+
+
+def oracle_tdp(inputs, alpha, causal, windows=(None,) * 4, per_head=True):
+    """Oracle in fp32 on the already-rounded inputs (what the reference's tests do:
+    tests/test_triple_dot_product.py:47).  Evaluated head by head to bound memory."""
+    q, k1, k2, v1, v2, do = (t.float() for t in inputs)
+    kw = dict(zip(("k1_window", "k2_window", "kk_left", "kk_right"), windows))
+    B, H, T, D = q.shape
+    z = torch.empty_like(q)
+    lse = torch.empty(B, H, T)
+    grads = [torch.empty_like(q) for _ in range(5)]
+    for b in range(B):
+        for h in range(H):
+            zz, ll, gg = orc.tdp_forward_backward(*(t[b, h] for t in (q, k1, k2, v1, v2, do)), alpha, causal, **kw)
+            z[b, h], lse[b, h] = zz, ll
+            for g, x in zip(grads, gg):
+                g[b, h] = x
+    return z, lse, grads
+
+
+def oracle_dps(inputs, alpha, causal, k_diff, factorised=False):
+    q, k1, k2, v1, v2, do = (t.float() for t in inputs)
+    B, H, T, D = q.shape
+    z = torch.empty_like(q)
+    lse = torch.empty(B, H, T)
+    grads = [torch.empty_like(q) for _ in range(5)]
+    for b in range(B):
+        for h in range(H):
+            zz, ll, gg = orc.dps_forward_backward(*(t[b, h] for t in (q, k1, k2, v1, v2, do)), alpha, causal,
+                                                  k_diff=k_diff, factorised=factorised)
+            z[b, h], lse[b, h] = zz, ll
+            for g, x in zip(grads, gg):
+                g[b, h] = x
+    return z, lse, grads
+
+
+def run_tdp(inputs, alpha, causal, windows=(None,) * 4, backward=True, device="cuda"):
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    q, k1, k2, v1, v2, do = (t.to(device) for t in inputs)
+    leaves = [t.detach().clone().requires_grad_(backward) for t in (q, k1, k2, v1, v2)]
+    out = flash_trittention(*leaves, softmax_scale=alpha, k1_window=windows[0], k2_window=windows[1],
+                            kk_left=windows[2], kk_right=windows[3], causal=causal)
+    grads = None
+    if backward:
+        out.backward(do)
+        grads = [t.grad.float().cpu() for t in leaves]
+    torch.cuda.synchronize()
+    return out.detach().float().cpu(), grads
+
+
+def run_dps(inputs, alpha, causal, k_diff, backward=True, device="cuda"):
+    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
+
+    q, k1, k2, v1, v2, do = (t.to(device) for t in inputs)
+    leaves = [t.detach().clone().requires_grad_(backward) for t in (q, k1, k2, v1, v2)]
+    out, m = TrittentionTriton(causal=causal, softmax_scale=alpha, k_diff=k_diff)(*leaves)
+    grads = None
+    if backward:
+        out.backward(do)
+        grads = [t.grad.float().cpu() for t in leaves]
+    torch.cuda.synchronize()
+    return out.detach().float().cpu(), m.detach().cpu(), grads
+
+
+def assert_close(name, got, want, rtol, atol):
+    torch.testing.assert_close(got, want, rtol=rtol, atol=atol, msg=lambda m: f"{name}: {m}")
+
+
+def rel_err(got, want):
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
