@@ -248,6 +248,16 @@ int dps_bwd_impl(Arena& ar, bool run, const void* q, const void* k1, const void*
     return (int)hipGetLastError();
 }
 
+// windows that cannot exclude any pair once j,k <= q holds
+bool full_windows(int T, int causal, int w1, int w2, int kl, int kr) {
+    return !causal || (w1 >= T - 1 && w2 >= T - 1 && kl >= T - 1 && kr >= T - 1);
+}
+
+bool use_mfma_fwd(int T, int D, int dtype, int causal, int w1, int w2, int kl, int kr, unsigned flags) {
+    if (flags & TRITT_FLAG_FORCE_GENERIC) return false;
+    return mfma_tdp_fwd_supported(D, dtype != TRITT_F32) && full_windows(T, causal, w1, w2, kl, kr);
+}
+
 bool any_null(std::initializer_list<const void*> ps) {
     for (const void* p : ps)
         if (!p) return true;
@@ -278,6 +288,8 @@ const char* tritt_status_string(int status) {
 size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,
                                      int kk_left, int kk_right, unsigned flags) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (use_mfma_fwd(T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags))
+        return mfma_tdp_fwd_workspace(B * H, T, D);
     Arena ar(nullptr);
     tdp_fwd_generic(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f,
                     causal, k1_window, k2_window, kk_left, kk_right, nullptr);
@@ -293,9 +305,17 @@ int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1,
     if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
     if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
-    if (flags & TRITT_FLAG_FORCE_MFMA) return TRITT_ERR_UNSUPPORTED;
+    const bool mfma = use_mfma_fwd(T, D, dtype, causal, w1, w2, kl, kr, flags);
+    if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;
     const size_t need = tritt_tdp_fwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
     if (need && (!workspace || workspace_bytes < need)) return TRITT_ERR_WORKSPACE;
+    if (mfma) {
+        MfmaFwdArgs a{};
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.lse = lse; a.ut = workspace;
+        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0;
+        a.is_bf16 = dtype == TRITT_BF16;
+        return (int)mfma_tdp_fwd(a, (hipStream_t)stream);
+    }
     Arena ar(workspace);
     return tdp_fwd_generic(ar, true, q, k1, k2, v1, v2, o, lse, B, H, T, D, dtype, alpha, causal, w1, w2, kl, kr,
                            (hipStream_t)stream);

@@ -38,4 +38,19 @@ struct DpsArgs {
 hipError_t dps_fwd(const DpsArgs& a, hipStream_t st);
 hipError_t dps_bwd(const DpsArgs& a, hipStream_t st);
 
+// 16-bit MFMA triple-dot forward (full causal windows or no mask; D = 64 or 128).
+struct MfmaFwdArgs {
+    const void *q, *k1, *k2, *v1, *v2;
+    void* o;
+    float* lse;
+    void* ut;  // scratch: mfma_tdp_fwd_workspace() bytes
+    int BH, T, D;
+    float alpha;
+    int causal;
+    int is_bf16;  // else fp16
+};
+size_t mfma_tdp_fwd_workspace(int BH, int T, int D);
+bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit);
+hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st);
+
 }  // namespace tritt

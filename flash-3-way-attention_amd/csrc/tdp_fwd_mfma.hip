@@ -1,0 +1,386 @@
+// Triple-dot-product trittention forward on MFMA (gfx950), 16-bit tensors, full causal
+// windows or no mask.
+//
+// Formulation.  For a fixed key-2 row k the scores of query q are an ordinary attention row:
+//   s[q,j,k] = (alpha * Q[q] (.) K2[k]) . K1[j]
+// so every pair (q,k) is a "virtual query row" with its own online softmax over j and its own
+// accumulator  Tv[(q,k), :] = sum_j P U[j, :]   (U = SiLU(V1)).  The rows of one query are
+// merged once per k-tile:  O[q] = sum_k w_k * V2[k] (.) Tv[(q,k)],  w_k = exp2(m_qk - M_q).
+//
+// Work decomposition.  One workgroup = 8 waves = BQ = 8*NT queries of one (batch, head).
+// A wave owns NT queries; a 32x32 MFMA tile is 32 consecutive k (columns) of ONE query, so the
+// causal bound j <= q is uniform over a tile and the k-merge stays inside the wave.
+// Outer loop: k-tiles of 32.  Inner loop: 64-row stages of K1 and U^T, staged through LDS and
+// shared by all 8 waves (double buffered, one barrier per stage).
+//
+// Per 32-key step and tile:  S^T = K1 * QK2^T  (rows = j, cols = virtual rows), accumulated on
+// top of C = -m (the running reference maximum), so the MFMA result is already s - m.  The
+// reference maximum is only raised when some score exceeds it by more than 2^8 ("lazy" max),
+// which keeps max/rescale work off the common path.  P = exp2(S) is packed to 16 bit in the
+// registers it already occupies and fed straight back as the A operand of Tv += P * U.
+#include "kernels.hpp"
+#include "mfma.hpp"
+
+namespace tritt {
+
+template <typename E>
+struct FwdParams {
+    const E *q, *k1, *k2, *v2;
+    const E* ut;  // [BH][D][Tp]  SiLU(V1) transposed, zero padded to Tp (multiple of 64)
+    E* o;
+    float* lse;
+    int T, Tp, BH, nqt;
+    float scale_log2;
+    int causal;
+};
+
+constexpr float kLazyThreshold = 8.0f;
+
+template <typename E, int D, int NT>
+__global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
+    using M = Mma<E>;
+    using v8 = typename M::v8;
+    using v2 = typename M::v2;
+    constexpr int KS = D / 16;   // k-steps of the score product
+    constexpr int DT = D / 32;   // 32-wide d tiles of the value product
+    constexpr int BQ = 8 * NT;
+    constexpr int LDK = D + 8;   // LDS row stride (elements) of row-major [rows][D] tiles
+    constexpr int LDU = 64 + 8;  // LDS row stride of the U^T stage ([D][64 keys])
+    constexpr int CH = D / 64;   // 16-byte chunks per thread per staged tensor
+
+    extern __shared__ __align__(16) char smem[];
+    E* sK1 = reinterpret_cast<E*>(smem);  // [2][64][LDK]
+    E* sUT = sK1 + 2 * 64 * LDK;          // [2][D][LDU]
+    E* sK2 = sUT + 2 * D * LDU;           // [2][32][LDK]
+    E* sV2 = sK2 + 2 * 32 * LDK;          // [2][32][LDK]
+    E* sQ = sV2 + 2 * 32 * LDK;           // [BQ][LDK]
+
+    // heavy-first, XCD-aware block order: consecutive block ids go to different XCDs, so give
+    // every XCD its own set of heads (their K/V stay in that XCD's L2) and hand out the
+    // longest query tiles first.
+    const int groups = (p.BH + 7) / 8;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int bh = (slot % groups) * 8 + xcd;
+    const int qt = p.nqt - 1 - slot / groups;
+    if (bh >= p.BH) return;
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int T = p.T;
+    const size_t base = (size_t)bh * T * D;
+    const E* __restrict__ Q = p.q + base;
+    const E* __restrict__ K1 = p.k1 + base;
+    const E* __restrict__ K2 = p.k2 + base;
+    const E* __restrict__ V2 = p.v2 + base;
+    const E* __restrict__ UT = p.ut + (size_t)bh * D * p.Tp;
+
+    const int q0 = qt * BQ;
+    const int jend = p.causal ? min(T - 1, q0 + BQ - 1) : T - 1;  // last key any query here needs
+    const int nst = jend / 64 + 1, nkt = jend / 32 + 1;
+
+    int qrow[NT], jmax[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        qrow[t] = q0 + wave * NT + t;
+        jmax[t] = p.causal ? min(qrow[t], T - 1) : T - 1;  // bound on j and on k
+    }
+
+    // ---- staging helpers ------------------------------------------------------------------
+    uint4 rk[CH], ru[CH], rkv[CH];
+    auto issue_stage = [&](int st) {
+        const int jb = st * 64;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int idx = tid + c * 512;
+            const int r = idx / (D / 8), ch = idx % (D / 8);
+            rk[c] = *reinterpret_cast<const uint4*>(K1 + (size_t)min(jb + r, T - 1) * D + ch * 8);
+            const int d = idx / 8, cj = idx % 8;
+            ru[c] = *reinterpret_cast<const uint4*>(UT + (size_t)d * p.Tp + jb + cj * 8);
+        }
+    };
+    auto commit_stage = [&](int buf) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int idx = tid + c * 512;
+            const int r = idx / (D / 8), ch = idx % (D / 8);
+            *reinterpret_cast<uint4*>(sK1 + (buf * 64 + r) * LDK + ch * 8) = rk[c];
+            const int d = idx / 8, cj = idx % 8;
+            *reinterpret_cast<uint4*>(sUT + (buf * D + d) * LDU + cj * 8) = ru[c];
+        }
+    };
+    auto issue_ktile = [&](int kt) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int idx = tid + c * 512;
+            const int which = idx / (4 * D), rem = idx % (4 * D);
+            const int r = rem / (D / 8), ch = rem % (D / 8);
+            const E* src = which ? V2 : K2;
+            rkv[c] = *reinterpret_cast<const uint4*>(src + (size_t)min(kt * 32 + r, T - 1) * D + ch * 8);
+        }
+    };
+    auto commit_ktile = [&](int buf) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int idx = tid + c * 512;
+            const int which = idx / (4 * D), rem = idx % (4 * D);
+            const int r = rem / (D / 8), ch = rem % (D / 8);
+            E* dst = which ? sV2 : sK2;
+            *reinterpret_cast<uint4*>(dst + (buf * 32 + r) * LDK + ch * 8) = rkv[c];
+        }
+    };
+
+    // ---- prologue: Q tile, first k-tile, first stage ------------------------------------------
+    for (int idx = tid; idx < BQ * (D / 8); idx += 512) {
+        const int r = idx / (D / 8), ch = idx % (D / 8);
+        *reinterpret_cast<uint4*>(sQ + r * LDK + ch * 8) =
+            *reinterpret_cast<const uint4*>(Q + (size_t)min(q0 + r, T - 1) * D + ch * 8);
+    }
+    issue_ktile(0);
+    issue_stage(0);
+    commit_ktile(0);
+    commit_stage(0);
+    __syncthreads();
+
+    float Mrun[NT], Lrun[NT], Orun[NT][DT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        Mrun[t] = -INFINITY;
+        Lrun[t] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) Orun[t][dt] = 0.f;
+    }
+
+    const int krow_off = key_of_row(n);  // K1 row (within a 32-key step) this lane feeds to the MFMA
+
+    int gstage = 0;  // running stage counter (buffer = gstage & 1)
+    for (int kt = 0; kt < nkt; ++kt) {
+        const int kb = kt & 1;
+        if (kt + 1 < nkt) issue_ktile(kt + 1);
+
+        // B operands: QK2[(q, k), d] = Q[q,d] * K2[k,d] * alpha*log2(e), k = 32*kt + n
+        v8 bq[NT][KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const v8 kv = *reinterpret_cast<const v8*>(sK2 + (kb * 32 + n) * LDK + ks * 16 + g * 8);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const v8 qv = *reinterpret_cast<const v8*>(sQ + (wave * NT + t) * LDK + ks * 16 + g * 8);
+                v8 r;
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const v2 pr = M::pack((float)kv[e] * (float)qv[e] * p.scale_log2,
+                                          (float)kv[e + 1] * (float)qv[e + 1] * p.scale_log2);
+                    r[e] = pr[0];
+                    r[e + 1] = pr[1];
+                }
+                bq[t][ks] = r;
+            }
+        }
+
+        f32x16 acc[NT][DT], cm[NT];
+        float mref[NT], lsum[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            mref[t] = 0.f;
+            lsum[t] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) cm[t][i] = 0.f;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[t][dt][i] = 0.f;
+        }
+
+        for (int st = 0; st < nst; ++st, ++gstage) {
+            const int sb = gstage & 1;
+            const bool more = (st + 1 < nst) || (kt + 1 < nkt);
+            if (more) issue_stage(st + 1 < nst ? st + 1 : 0);
+
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int jb = st * 64 + half * 32;
+                if (jb > jend) break;
+                const bool first = (jb == 0);
+                v8 k1a[KS];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    k1a[ks] = *reinterpret_cast<const v8*>(sK1 + (sb * 64 + half * 32 + krow_off) * LDK + ks * 16 + g * 8);
+                v8 ub[DT][2];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        ub[dt][h] = *reinterpret_cast<const v8*>(sUT + (sb * D + dt * 32 + n) * LDU + half * 32 + h * 16 + g * 8);
+
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    if (jb > jmax[t]) continue;  // tile entirely above the causal bound (wave-uniform)
+                    f32x16 s = M::mma(k1a[0], bq[t][0], cm[t]);
+#pragma unroll
+                    for (int ks = 1; ks < KS; ++ks) s = M::mma(k1a[ks], bq[t][ks], s);
+                    if (jb + 31 > jmax[t]) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) s[i] = (jb + key_of(g, i) <= jmax[t]) ? s[i] : -INFINITY;
+                    }
+                    float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+                    for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
+                    if (first || __any(mx > kLazyThreshold)) {
+                        // raise the reference maximum of the rows that need it
+                        const float rmax = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                        const float delta = first ? rmax : fmaxf(rmax, 0.f);
+                        mref[t] += delta;
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            cm[t][i] = -mref[t];
+                            s[i] -= delta;
+                        }
+                        if (!first) {
+                            const float f = fast_exp2(-delta);
+                            lsum[t] *= f;
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) {
+                                const float fr = __shfl(f, c_row(g, i), 64);
+#pragma unroll
+                                for (int dt = 0; dt < DT; ++dt) acc[t][dt][i] *= fr;
+                            }
+                        }
+                    }
+                    v8 pa[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                        for (int e = 0; e < 8; e += 2) {
+                            const v2 pr = M::pack(fast_exp2(s[h * 8 + e]), fast_exp2(s[h * 8 + e + 1]));
+                            lsum[t] = M::add_pair(pr, lsum[t]);
+                            pa[h][e] = pr[0];
+                            pa[h][e + 1] = pr[1];
+                        }
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        acc[t][dt] = M::mma(pa[0], ub[dt][0], acc[t][dt]);
+                        acc[t][dt] = M::mma(pa[1], ub[dt][1], acc[t][dt]);
+                    }
+                }
+            }
+
+            if (more) commit_stage(sb ^ 1);
+            __syncthreads();
+        }
+
+        // ---- merge the 32 virtual rows (q, k) of each tile into the running O[q] -------------
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const float lk = lsum[t] + __shfl_xor(lsum[t], 32, 64);
+            const bool kval = (kt * 32 + n) <= jmax[t];
+            float mt = kval ? mref[t] : -INFINITY;
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1) mt = fmaxf(mt, __shfl_xor(mt, off, 64));
+            const float mnew = fmaxf(Mrun[t], mt);
+            const float f = fast_exp2(Mrun[t] - mnew);
+            const float w = kval ? fast_exp2(mref[t] - mnew) : 0.f;
+            float wl = w * lk;
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1) wl += __shfl_xor(wl, off, 64);
+            Lrun[t] = Lrun[t] * f + wl;
+            Mrun[t] = mnew;
+            float part[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) part[dt] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int r = c_row(g, i);
+                const float wr = __shfl(w, r, 64);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const float v = (float)sV2[(kb * 32 + r) * LDK + dt * 32 + n];
+                    // select, not multiply: rows past the causal bound may hold anything
+                    part[dt] += (wr > 0.f) ? wr * v * acc[t][dt][i] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) Orun[t][dt] = Orun[t][dt] * f + part[dt];
+        }
+
+        if (kt + 1 < nkt) commit_ktile(kb ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue ---------------------------------------------------------------------------
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int q = qrow[t];
+        const float inv = 1.0f / Lrun[t];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const float o = (Orun[t][dt] + __shfl_xor(Orun[t][dt], 32, 64)) * inv;
+            if (q < T && g == 0) p.o[base + (size_t)q * D + dt * 32 + n] = (E)o;
+        }
+        if (q < T && lane == 0) p.lse[(size_t)bh * T + q] = (Mrun[t] + fast_log2(Lrun[t])) * kLn2;
+    }
+}
+
+// U^T[bh][d][j] = SiLU(V1[bh][j][d]) for j < T, 0 for T <= j < Tp
+template <typename E>
+__global__ __launch_bounds__(256) void silu_transpose_kernel(const E* __restrict__ v1, E* __restrict__ ut, int T,
+                                                             int Tp, int D) {
+    const int bh = blockIdx.y, j0 = blockIdx.x * 64;
+    const E* src = v1 + (size_t)bh * T * D;
+    E* dst = ut + (size_t)bh * D * Tp;
+    for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
+        const int d = idx >> 6, jj = idx & 63, j = j0 + jj;
+        float v = 0.f;
+        if (j < T) v = silu_f((float)src[(size_t)j * D + d]);
+        dst[(size_t)d * Tp + j] = (E)v;
+    }
+}
+
+template <int D, int NT>
+constexpr size_t fwd_smem_bytes() {
+    return sizeof(uint16_t) * (2 * 64 * (D + 8) + 2 * D * 72 + 4 * 32 * (D + 8) + 8 * NT * (D + 8));
+}
+
+template <typename E, int D, int NT>
+static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
+    const int Tp = (a.T + 63) / 64 * 64;
+    hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
+                       a.T, Tp, D);
+    FwdParams<E> p;
+    p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
+    p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse;
+    p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 8 * NT - 1) / (8 * NT);
+    p.scale_log2 = a.alpha * kLog2e;
+    p.causal = a.causal;
+    constexpr size_t smem = fwd_smem_bytes<D, NT>();
+    auto kern = tdp_fwd_mfma_kernel<E, D, NT>;
+    static bool attr_set = false;  // per (E, D, NT) instantiation
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int groups = (a.BH + 7) / 8;
+    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p);
+    return hipGetLastError();
+}
+
+size_t mfma_tdp_fwd_workspace(int BH, int T, int D) {
+    const size_t Tp = (size_t)(T + 63) / 64 * 64;
+    return (size_t)BH * D * Tp * 2;
+}
+
+bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
+
+hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
+    if (a.is_bf16) {
+        if (a.D == 64) return launch<__bf16, 64, 2>(a, st);
+        if (a.D == 128) return launch<__bf16, 128, 1>(a, st);
+    } else {
+        if (a.D == 64) return launch<_Float16, 64, 2>(a, st);
+        if (a.D == 128) return launch<_Float16, 128, 1>(a, st);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace tritt

@@ -140,3 +140,67 @@ def test_input_precision_warns_and_is_ignored():
                               input_precision="ieee")
     b = flash_trittention(q, k1, k2, v1, v2, k1_window=None, k2_window=None, kk_left=None, kk_right=None)
     assert torch.equal(a, b)
+
+
+# ---------------------------------------------------------------- MFMA kernels (16-bit tensors)
+FORCE_GENERIC, FORCE_MFMA = 1, 2
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("seq_len", [1, 16, 33, 100, 129, 256])
+def test_mfma_forward_bf16(seq_len, causal, D):
+    """The MFMA forward alone (FORCE_MFMA: no fallback), ragged lengths included."""
+    print(f"case mfma fwd T={seq_len} causal={causal} D={D}", flush=True)
+    inputs = orc.make_inputs(1, 3, seq_len, D, torch.bfloat16, seed=seq_len + D)
+    alpha = 1 / math.sqrt(D)
+    z, _, _ = util.oracle_tdp(inputs, alpha, causal)
+    out, _ = util.run_tdp(inputs, alpha, causal, backward=False, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    assert util.rel_err(out, z) <= 2e-2, util.rel_err(out, z)
+
+
+def test_mfma_forward_fp16():
+    inputs = orc.make_inputs(2, 2, 200, 64, torch.float16, seed=21)
+    z, _, _ = util.oracle_tdp(inputs, 1 / 8, True)
+    out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+
+
+def test_mfma_forward_large_logits():
+    """Scores spanning hundreds: the lazily raised reference maximum must keep everything finite."""
+    inputs = orc.make_inputs(1, 2, 160, 64, torch.bfloat16, seed=22)
+    inputs[1] = (inputs[1].float() * 6).bfloat16()
+    inputs[2] = (inputs[2].float() * 6).bfloat16()
+    z, _, _ = util.oracle_tdp(inputs, 1 / 8, True)
+    out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
+    assert torch.isfinite(out).all()
+    # with logits this large the softmax is nearly one-hot and the 16-bit rounding of Q*K2 can swap
+    # near-tied winners (the reference's test notes the same), so bound the error statistically
+    err = (out - z).abs()
+    assert (err > 5e-2).float().mean() < 0.01 and err.max() < 0.5, (err.max(), (err > 5e-2).float().mean())
+
+
+def test_mfma_and_generic_agree_bf16():
+    inputs = orc.make_inputs(1, 2, 192, 64, torch.bfloat16, seed=23)
+    a, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
+    b, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_GENERIC)
+    util.assert_close("out", a, b, **LOWP)
+
+
+def test_force_mfma_refuses_unsupported():
+    inputs = orc.make_inputs(1, 1, 32, 32, torch.float32, seed=24)
+    with pytest.raises(RuntimeError, match="does not support"):
+        util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
+
+
+def test_config3_headline_forward_subset():
+    """B=4 H=8 T=1024 D=64 bf16 causal on the GPU; the oracle (chunked dense, CPU) checks all rows
+    of three heads."""
+    print("case config3 forward", flush=True)
+    inputs = orc.make_inputs(4, 8, 1024, 64, torch.bfloat16, seed=3)
+    out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False)
+    for (b, h) in ((0, 0), (2, 5), (3, 7)):
+        z, lse, _ = orc.tdp_forward_backward_chunked(*(t[b, h].float() for t in inputs), 1 / 8, True,
+                                                     q_chunk=64, need_grads=False)
+        util.assert_close(f"out[{b},{h}]", out[b, h], z, **LOWP)

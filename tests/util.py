@@ -41,8 +41,17 @@ def oracle_dps(inputs, alpha, causal, k_diff, factorised=False):
     return z, lse, grads
 
 
-def run_tdp(inputs, alpha, causal, windows=(None,) * 4, backward=True, device="cuda"):
-    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+def run_tdp(inputs, alpha, causal, windows=(None,) * 4, backward=True, device="cuda", flags=0):
+    from flash_trittention.triple_dot_product.flash_trittention import FlashTrittention, flash_trittention
+
+    FlashTrittention.impl_flags = flags
+    try:
+        return _run_tdp(flash_trittention, inputs, alpha, causal, windows, backward, device)
+    finally:
+        FlashTrittention.impl_flags = 0
+
+
+def _run_tdp(flash_trittention, inputs, alpha, causal, windows, backward, device):
 
     q, k1, k2, v1, v2, do = (t.to(device) for t in inputs)
     leaves = [t.detach().clone().requires_grad_(backward) for t in (q, k1, k2, v1, v2)]
