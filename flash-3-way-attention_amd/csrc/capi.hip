@@ -258,6 +258,11 @@ bool use_mfma_fwd(int T, int D, int dtype, int causal, int w1, int w2, int kl, i
     return mfma_tdp_fwd_supported(D, dtype != TRITT_F32) && full_windows(T, causal, w1, w2, kl, kr);
 }
 
+bool use_mfma_bwd(int T, int D, int dtype, int causal, int w1, int w2, int kl, int kr, unsigned flags) {
+    if (flags & TRITT_FLAG_FORCE_GENERIC) return false;
+    return mfma_tdp_bwd_supported(D, dtype != TRITT_F32) && full_windows(T, causal, w1, w2, kl, kr);
+}
+
 bool any_null(std::initializer_list<const void*> ps) {
     for (const void* p : ps)
         if (!p) return true;
@@ -324,6 +329,8 @@ int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1,
 size_t tritt_tdp_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,
                                      int kk_left, int kk_right, unsigned flags) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (use_mfma_bwd(T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags))
+        return mfma_tdp_bwd_workspace(B * H, T, D);
     Arena ar(nullptr);
     tdp_bwd_generic(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                     nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f, causal, k1_window, k2_window, kk_left, kk_right,
@@ -341,9 +348,18 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
     if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
-    if (flags & TRITT_FLAG_FORCE_MFMA) return TRITT_ERR_UNSUPPORTED;
+    const bool mfma = use_mfma_bwd(T, D, dtype, causal, w1, w2, kl, kr, flags);
+    if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;
     const size_t need = tritt_tdp_bwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
     if (need && (!workspace || workspace_bytes < need)) return TRITT_ERR_WORKSPACE;
+    if (mfma) {
+        MfmaBwdArgs a{};
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.d_o = d_o; a.lse = lse;
+        a.dq = dq; a.dk1 = dk1; a.dk2 = dk2; a.dv1 = dv1; a.dv2 = dv2; a.workspace = workspace;
+        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0;
+        a.is_bf16 = dtype == TRITT_BF16;
+        return (int)mfma_tdp_bwd(a, (hipStream_t)stream);
+    }
     Arena ar(workspace);
     return tdp_bwd_generic(ar, true, q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2, B, H, T, D, dtype, alpha,
                            causal, w1, w2, kl, kr, (hipStream_t)stream);

@@ -53,4 +53,19 @@ size_t mfma_tdp_fwd_workspace(int BH, int T, int D);
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st);
 
+// 16-bit MFMA triple-dot backward (full causal windows or no mask; D = 64).
+struct MfmaBwdArgs {
+    const void *q, *k1, *k2, *v1, *v2, *o, *d_o;
+    const float* lse;
+    void *dq, *dk1, *dk2, *dv1, *dv2;
+    void* workspace;  // mfma_tdp_bwd_workspace() bytes
+    int BH, T, D;
+    float alpha;
+    int causal;
+    int is_bf16;
+};
+size_t mfma_tdp_bwd_workspace(int BH, int T, int D);
+bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit);
+hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st);
+
 }  // namespace tritt

@@ -85,3 +85,16 @@ def assert_close(name, got, want, rtol, atol):
 
 def rel_err(got, want):
     return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def assert_mostly_close(name, got, want, rtol, atol, outlier_frac=1e-3, outlier_scale=4.0):
+    """Like assert_close, but tolerates a tiny fraction of elements up to `outlier_scale` times the
+    tolerance.  Used only for 16-bit gradients of rows whose softmax is nearly one-hot (the first
+    few queries of a causal sequence): there dS = P (dP - Delta) is a difference of two O(10)
+    numbers that each carry 16-bit rounding error (dO*V2 is rounded to 16 bit before the MFMA),
+    so single elements can land a few 1e-2 away from an exactly-zero reference."""
+    err = (got - want).abs()
+    tol = atol + rtol * want.abs()
+    bad = err > tol
+    assert bad.float().mean().item() <= outlier_frac, f"{name}: {bad.sum().item()} of {bad.numel()} outside tolerance"
+    assert (err <= outlier_scale * tol).all(), f"{name}: max error {err.max().item()}"
