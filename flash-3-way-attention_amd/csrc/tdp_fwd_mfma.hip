@@ -18,6 +18,9 @@
 // reference maximum is only raised when some score exceeds it by more than 2^8 ("lazy" max),
 // which keeps max/rescale work off the common path.  P = exp2(S) is packed to 16 bit in the
 // registers it already occupies and fed straight back as the A operand of Tv += P * U.
+#include <stdlib.h>
+#include <string.h>
+
 #include "kernels.hpp"
 #include "mfma.hpp"
 
@@ -36,24 +39,30 @@ struct FwdParams {
 
 constexpr float kLazyThreshold = 8.0f;
 
-template <typename E, int D, int NT>
-__global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
+// MINW (second launch-bounds argument): waves per SIMD the register allocator must leave room for
+template <typename E, int D, int NT, int WAVES, int MINW, int JS>
+__global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using v2 = typename M::v2;
+    constexpr int NTH = 64 * WAVES;
     constexpr int KS = D / 16;   // k-steps of the score product
     constexpr int DT = D / 32;   // 32-wide d tiles of the value product
-    constexpr int BQ = 8 * NT;
+    constexpr int BQ = WAVES * NT;
     constexpr int LDK = D + 8;   // LDS row stride (elements) of row-major [rows][D] tiles
-    constexpr int LDU = 64 + 8;  // LDS row stride of the U^T stage ([D][64 keys])
-    constexpr int CH = D / 64;   // 16-byte chunks per thread per staged tensor
+    constexpr int LDU = JS + 8;  // LDS row stride of the U^T stage ([D][JS keys])
+    constexpr int K1_CHUNKS = JS * D / 8;      // 16-byte chunks of a K1 stage [JS][D]
+    constexpr int STAGE_CHUNKS = 2 * K1_CHUNKS;  // ... followed by the U^T stage [D][JS]
+    constexpr int KTILE_CHUNKS = 8 * D;   // K2 [32][D] then V2 [32][D]
+    constexpr int CS = (STAGE_CHUNKS + NTH - 1) / NTH, CK = (KTILE_CHUNKS + NTH - 1) / NTH;
 
     extern __shared__ __align__(16) char smem[];
-    E* sK1 = reinterpret_cast<E*>(smem);  // [2][64][LDK]
-    E* sUT = sK1 + 2 * 64 * LDK;          // [2][D][LDU]
+    E* sK1 = reinterpret_cast<E*>(smem);  // [2][JS][LDK]
+    E* sUT = sK1 + 2 * JS * LDK;          // [2][D][LDU]
     E* sK2 = sUT + 2 * D * LDU;           // [2][32][LDK]
     E* sV2 = sK2 + 2 * 32 * LDK;          // [2][32][LDK]
     E* sQ = sV2 + 2 * 32 * LDK;           // [BQ][LDK]
+    float* sW = reinterpret_cast<float*>(sQ + BQ * LDK);  // [WAVES][32] per-wave scratch
 
     // heavy-first, XCD-aware block order: consecutive block ids go to different XCDs, so give
     // every XCD its own set of heads (their K/V stay in that XCD's L2) and hand out the
@@ -64,7 +73,8 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     const int qt = p.nqt - 1 - slot / groups;
     if (bh >= p.BH) return;
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it scalar
     const int T = p.T;
     const size_t base = (size_t)bh * T * D;
     const E* __restrict__ Q = p.q + base;
@@ -72,10 +82,11 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     const E* __restrict__ K2 = p.k2 + base;
     const E* __restrict__ V2 = p.v2 + base;
     const E* __restrict__ UT = p.ut + (size_t)bh * D * p.Tp;
+    float* sWw = sW + wave * 32;
 
     const int q0 = qt * BQ;
     const int jend = p.causal ? min(T - 1, q0 + BQ - 1) : T - 1;  // last key any query here needs
-    const int nst = jend / 64 + 1, nkt = jend / 32 + 1;
+    const int nst = jend / JS + 1, nkt = jend / 32 + 1;
 
     int qrow[NT], jmax[NT];
 #pragma unroll
@@ -85,51 +96,73 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     }
 
     // ---- staging helpers ------------------------------------------------------------------
-    uint4 rk[CH], ru[CH], rkv[CH];
+    uint4 rs[CS], rkv[CK];
     auto issue_stage = [&](int st) {
-        const int jb = st * 64;
+        const int jb = st * JS;
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int r = idx / (D / 8), ch = idx % (D / 8);
-            rk[c] = *reinterpret_cast<const uint4*>(K1 + (size_t)min(jb + r, T - 1) * D + ch * 8);
-            const int d = idx / 8, cj = idx % 8;
-            ru[c] = *reinterpret_cast<const uint4*>(UT + (size_t)d * p.Tp + jb + cj * 8);
+        for (int c = 0; c < CS; ++c) {
+            const int item = tid + c * NTH;
+            if (item < K1_CHUNKS) {
+                const int r = item / (D / 8), ch = item % (D / 8);
+                rs[c] = *reinterpret_cast<const uint4*>(K1 + (size_t)min(jb + r, T - 1) * D + ch * 8);
+            } else if (item < STAGE_CHUNKS) {
+                const int i2 = item - K1_CHUNKS, d = i2 / (JS / 8), cj = i2 % (JS / 8);
+                rs[c] = *reinterpret_cast<const uint4*>(UT + (size_t)d * p.Tp + jb + cj * 8);
+            }
         }
     };
     auto commit_stage = [&](int buf) {
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int r = idx / (D / 8), ch = idx % (D / 8);
-            *reinterpret_cast<uint4*>(sK1 + (buf * 64 + r) * LDK + ch * 8) = rk[c];
-            const int d = idx / 8, cj = idx % 8;
-            *reinterpret_cast<uint4*>(sUT + (buf * D + d) * LDU + cj * 8) = ru[c];
+        for (int c = 0; c < CS; ++c) {
+            const int item = tid + c * NTH;
+            if (item < K1_CHUNKS) {
+                const int r = item / (D / 8), ch = item % (D / 8);
+                *reinterpret_cast<uint4*>(sK1 + (buf * JS + r) * LDK + ch * 8) = rs[c];
+            } else if (item < STAGE_CHUNKS) {
+                const int i2 = item - K1_CHUNKS, d = i2 / (JS / 8), cj = i2 % (JS / 8);
+                *reinterpret_cast<uint4*>(sUT + (buf * D + d) * LDU + cj * 8) = rs[c];
+            }
         }
     };
     auto issue_ktile = [&](int kt) {
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int which = idx / (4 * D), rem = idx % (4 * D);
-            const int r = rem / (D / 8), ch = rem % (D / 8);
-            const E* src = which ? V2 : K2;
-            rkv[c] = *reinterpret_cast<const uint4*>(src + (size_t)min(kt * 32 + r, T - 1) * D + ch * 8);
+        for (int c = 0; c < CK; ++c) {
+            const int item = tid + c * NTH;
+            if (item < KTILE_CHUNKS) {
+                const int which = item / (4 * D), rem = item % (4 * D);
+                const int r = rem / (D / 8), ch = rem % (D / 8);
+                const E* src = which ? V2 : K2;
+                rkv[c] = *reinterpret_cast<const uint4*>(src + (size_t)min(kt * 32 + r, T - 1) * D + ch * 8);
+            }
         }
     };
     auto commit_ktile = [&](int buf) {
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int which = idx / (4 * D), rem = idx % (4 * D);
-            const int r = rem / (D / 8), ch = rem % (D / 8);
-            E* dst = which ? sV2 : sK2;
-            *reinterpret_cast<uint4*>(dst + (buf * 32 + r) * LDK + ch * 8) = rkv[c];
+        for (int c = 0; c < CK; ++c) {
+            const int item = tid + c * NTH;
+            if (item < KTILE_CHUNKS) {
+                const int which = item / (4 * D), rem = item % (4 * D);
+                const int r = rem / (D / 8), ch = rem % (D / 8);
+                E* dst = which ? sV2 : sK2;
+                *reinterpret_cast<uint4*>(dst + (buf * 32 + r) * LDK + ch * 8) = rkv[c];
+            }
         }
+    };
+    // broadcast a per-virtual-row scalar (held by lane n) to the C/D layout (rows in registers):
+    // out[i] = value of row c_row(g, i).  Goes through this wave's own LDS scratch.
+    auto rows_of = [&](float v, float (&out)[16]) {
+        if (g == 0) sWw[n] = v;
+        __builtin_amdgcn_wave_barrier();  // same wave, same LDS queue: program order is enough
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const float4 f4 = *reinterpret_cast<const float4*>(sWw + 8 * b + 4 * g);
+            out[4 * b] = f4.x; out[4 * b + 1] = f4.y; out[4 * b + 2] = f4.z; out[4 * b + 3] = f4.w;
+        }
+        __builtin_amdgcn_wave_barrier();
     };
 
     // ---- prologue: Q tile, first k-tile, first stage ------------------------------------------
-    for (int idx = tid; idx < BQ * (D / 8); idx += 512) {
+    for (int idx = tid; idx < BQ * (D / 8); idx += NTH) {
         const int r = idx / (D / 8), ch = idx % (D / 8);
         *reinterpret_cast<uint4*>(sQ + r * LDK + ch * 8) =
             *reinterpret_cast<const uint4*>(Q + (size_t)min(q0 + r, T - 1) * D + ch * 8);
@@ -154,7 +187,6 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     int gstage = 0;  // running stage counter (buffer = gstage & 1)
     for (int kt = 0; kt < nkt; ++kt) {
         const int kb = kt & 1;
-        if (kt + 1 < nkt) issue_ktile(kt + 1);
 
         // B operands: QK2[(q, k), d] = Q[q,d] * K2[k,d] * alpha*log2(e), k = 32*kt + n
         v8 bq[NT][KS];
@@ -176,14 +208,12 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
             }
         }
 
-        f32x16 acc[NT][DT], cm[NT];
+        f32x16 acc[NT][DT];
         float mref[NT], lsum[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             mref[t] = 0.f;
             lsum[t] = 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) cm[t][i] = 0.f;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -194,29 +224,25 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
             const int sb = gstage & 1;
             const bool more = (st + 1 < nst) || (kt + 1 < nkt);
             if (more) issue_stage(st + 1 < nst ? st + 1 : 0);
+            if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
 
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int jb = st * 64 + half * 32;
+            for (int half = 0; half < JS / 32; ++half) {
+                const int jb = st * JS + half * 32;
                 if (jb > jend) break;
                 const bool first = (jb == 0);
-                v8 k1a[KS];
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    k1a[ks] = *reinterpret_cast<const v8*>(sK1 + (sb * 64 + half * 32 + krow_off) * LDK + ks * 16 + g * 8);
-                v8 ub[DT][2];
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-                        ub[dt][h] = *reinterpret_cast<const v8*>(sUT + (sb * D + dt * 32 + n) * LDU + half * 32 + h * 16 + g * 8);
+                const E* k1p = sK1 + (sb * JS + half * 32 + krow_off) * LDK + g * 8;
+                const E* utp = sUT + (sb * D + n) * LDU + half * 32 + g * 8;
 
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
                     if (jb > jmax[t]) continue;  // tile entirely above the causal bound (wave-uniform)
-                    f32x16 s = M::mma(k1a[0], bq[t][0], cm[t]);
+                    f32x16 s;
 #pragma unroll
-                    for (int ks = 1; ks < KS; ++ks) s = M::mma(k1a[ks], bq[t][ks], s);
+                    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        s = M::mma(*reinterpret_cast<const v8*>(k1p + ks * 16), bq[t][ks], s);
                     if (jb + 31 > jmax[t]) {
 #pragma unroll
                         for (int i = 0; i < 16; ++i) s[i] = (jb + key_of(g, i) <= jmax[t]) ? s[i] : -INFINITY;
@@ -224,25 +250,20 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
                     float mx = fmaxf(s[0], s[1]);
 #pragma unroll
                     for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
-                    if (first || __any(mx > kLazyThreshold)) {
-                        // raise the reference maximum of the rows that need it
+                    if (first || __any(mx - mref[t] > kLazyThreshold)) {
+                        // raise the reference maximum of the rows that need it (rare)
                         const float rmax = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                        const float delta = first ? rmax : fmaxf(rmax, 0.f);
+                        const float delta = first ? rmax - mref[t] : fmaxf(rmax - mref[t], 0.f);
                         mref[t] += delta;
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) {
-                            cm[t][i] = -mref[t];
-                            s[i] -= delta;
-                        }
                         if (!first) {
                             const float f = fast_exp2(-delta);
                             lsum[t] *= f;
+                            float fr[16];
+                            rows_of(f, fr);
 #pragma unroll
-                            for (int i = 0; i < 16; ++i) {
-                                const float fr = __shfl(f, c_row(g, i), 64);
+                            for (int i = 0; i < 16; ++i)
 #pragma unroll
-                                for (int dt = 0; dt < DT; ++dt) acc[t][dt][i] *= fr;
-                            }
+                                for (int dt = 0; dt < DT; ++dt) acc[t][dt][i] *= fr[i];
                         }
                     }
                     v8 pa[2];
@@ -250,7 +271,8 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
                     for (int h = 0; h < 2; ++h) {
 #pragma unroll
                         for (int e = 0; e < 8; e += 2) {
-                            const v2 pr = M::pack(fast_exp2(s[h * 8 + e]), fast_exp2(s[h * 8 + e + 1]));
+                            const v2 pr = M::pack(fast_exp2(s[h * 8 + e] - mref[t]),
+                                                  fast_exp2(s[h * 8 + e + 1] - mref[t]));
                             lsum[t] = M::add_pair(pr, lsum[t]);
                             pa[h][e] = pr[0];
                             pa[h][e + 1] = pr[1];
@@ -258,8 +280,10 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
                     }
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
-                        acc[t][dt] = M::mma(pa[0], ub[dt][0], acc[t][dt]);
-                        acc[t][dt] = M::mma(pa[1], ub[dt][1], acc[t][dt]);
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            acc[t][dt] = M::mma(pa[h], *reinterpret_cast<const v8*>(utp + dt * 32 * LDU + h * 16),
+                                                acc[t][dt]);
                     }
                 }
             }
@@ -284,22 +308,19 @@ __global__ __launch_bounds__(512) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
             for (int off = 16; off > 0; off >>= 1) wl += __shfl_xor(wl, off, 64);
             Lrun[t] = Lrun[t] * f + wl;
             Mrun[t] = mnew;
-            float part[DT];
+            float wr[16];
+            rows_of(w, wr);
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) part[dt] = 0.f;
+            for (int dt = 0; dt < DT; ++dt) {
+                float part = 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int r = c_row(g, i);
-                const float wr = __shfl(w, r, 64);
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const float v = (float)sV2[(kb * 32 + r) * LDK + dt * 32 + n];
+                for (int i = 0; i < 16; ++i) {
+                    const float v = (float)sV2[(kb * 32 + c_row(g, i)) * LDK + dt * 32 + n];
                     // select, not multiply: rows past the causal bound may hold anything
-                    part[dt] += (wr > 0.f) ? wr * v * acc[t][dt][i] : 0.f;
+                    part += (wr[i] > 0.f) ? wr[i] * v * acc[t][dt][i] : 0.f;
                 }
+                Orun[t][dt] = Orun[t][dt] * f + part;
             }
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) Orun[t][dt] = Orun[t][dt] * f + part[dt];
         }
 
         if (kt + 1 < nkt) commit_ktile(kb ^ 1);
@@ -335,25 +356,29 @@ __global__ __launch_bounds__(256) void silu_transpose_kernel(const E* __restrict
     }
 }
 
-template <int D, int NT>
+template <int D, int NT, int WAVES, int JS>
 constexpr size_t fwd_smem_bytes() {
-    return sizeof(uint16_t) * (2 * 64 * (D + 8) + 2 * D * 72 + 4 * 32 * (D + 8) + 8 * NT * (D + 8));
+    return sizeof(uint16_t) * (2 * JS * (D + 8) + 2 * D * (JS + 8) + 4 * 32 * (D + 8) + WAVES * NT * (D + 8)) +
+           sizeof(float) * WAVES * 32;
 }
 
-template <typename E, int D, int NT>
+constexpr int kTpad = 128;  // U^T rows are padded to a multiple of the largest stage
+
+template <typename E, int D, int NT, int WAVES, int MINW, int JS>
 static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
-    const int Tp = (a.T + 63) / 64 * 64;
+    const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
                        a.T, Tp, D);
+    constexpr int BQ = WAVES * NT;
     FwdParams<E> p;
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
     p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse;
-    p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 8 * NT - 1) / (8 * NT);
+    p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + BQ - 1) / BQ;
     p.scale_log2 = a.alpha * kLog2e;
     p.causal = a.causal;
-    constexpr size_t smem = fwd_smem_bytes<D, NT>();
-    auto kern = tdp_fwd_mfma_kernel<E, D, NT>;
-    static bool attr_set = false;  // per (E, D, NT) instantiation
+    constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS>();
+    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS>;
+    static bool attr_set = false;  // per instantiation
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -361,24 +386,53 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
         attr_set = true;
     }
     const int groups = (a.BH + 7) / 8;
-    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p);
+    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(64 * WAVES), smem, st, p);
     return hipGetLastError();
 }
 
 size_t mfma_tdp_fwd_workspace(int BH, int T, int D) {
-    const size_t Tp = (size_t)(T + 63) / 64 * 64;
+    const size_t Tp = (size_t)(T + kTpad - 1) / kTpad * kTpad;
     return (size_t)BH * D * Tp * 2;
 }
 
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
 
+// Tile shape used for D = 64.  TRITT_FWD_VARIANT (read once) selects another instantiation for
+// tuning sweeps: "nt1w16", "nt2w8", "nt1w8", "nt1w16j128", "nt1w8j128", "nt2w8j128", "nt2w16j128".
+static int fwd_variant() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = getenv("TRITT_FWD_VARIANT");
+        v = 0;
+        if (e) {
+            const char* names[] = {"nt1w16", "nt2w8", "nt1w8", "nt1w16j128", "nt1w8j128", "nt2w8j128", "nt2w16j128"};
+            for (int i = 0; i < 7; ++i)
+                if (!strcmp(e, names[i])) v = i;
+        }
+    }
+    return v;
+}
+
+template <typename E>
+static hipError_t launch_d64(const MfmaFwdArgs& a, hipStream_t st) {
+    switch (fwd_variant()) {
+        case 1: return launch<E, 64, 2, 8, 2, 64>(a, st);
+        case 2: return launch<E, 64, 1, 8, 4, 64>(a, st);
+        case 3: return launch<E, 64, 1, 16, 4, 128>(a, st);
+        case 4: return launch<E, 64, 1, 8, 4, 128>(a, st);
+        case 5: return launch<E, 64, 2, 8, 2, 128>(a, st);
+        case 6: return launch<E, 64, 2, 16, 2, 128>(a, st);
+        default: return launch<E, 64, 1, 16, 4, 64>(a, st);
+    }
+}
+
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
     if (a.is_bf16) {
-        if (a.D == 64) return launch<__bf16, 64, 2>(a, st);
-        if (a.D == 128) return launch<__bf16, 128, 1>(a, st);
+        if (a.D == 64) return launch_d64<__bf16>(a, st);
+        if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64>(a, st);
     } else {
-        if (a.D == 64) return launch<_Float16, 64, 2>(a, st);
-        if (a.D == 128) return launch<_Float16, 128, 1>(a, st);
+        if (a.D == 64) return launch_d64<_Float16>(a, st);
+        if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64>(a, st);
     }
     return hipErrorInvalidValue;
 }
