@@ -27,7 +27,7 @@ namespace tritt {
 template <typename E>
 struct BwdParams {
     const E *q, *k1, *k2, *v2, *d_o;
-    const E *u, *ut, *k1t;     // scratch: SiLU(V1) [BH][T][D]; transposes [BH][D][Tp]
+    const E *u, *ut, *k1t, *k2t, *v2t;  // scratch: SiLU(V1) [BH][T][D]; transposes [BH][D][Tp]
     const float *lse, *delta;  // [BH][T]
     E* dq;
     float *dk2acc, *dv2acc;    // [BH][T][D] fp32, zero on entry
@@ -277,44 +277,63 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
 }
 
 // ------------------------------------------------------------------------------------------
+// Owner = 256 rows j of K1/V1 (32 per wave).  For one query q at a time ("round") the wave
+// builds its B operands in registers
+//   k1q[j, d] = alpha*log2e * Q[q,d] K1[j,d],   uq[j, d] = dO[q,d] U[j,d]
+// and sweeps the k axis in stages of 64 rows shared by the whole workgroup:
+//   S[k, j]  = K2[k,:] . k1q[j,:]        dP[k, j] = V2[k,:] . uq[j,:]
+//   P = exp2(S - LSE2[q]),  dS = P (dP - Delta[q])
+//   dK1[j, :] += dS^T (K2 (.) Q[q])      dU[j, :]  += P^T (V2 (.) dO[q])
+// The two Hadamard-scaled transposed operands are written to LDS by the stage loader (from the
+// pre-transposed K2^T / V2^T scratch, 8 keys per thread), so dK1/dU accumulate directly in
+// registers over all rounds.  Workgroups split the queries NQC ways (round robin) and write fp32
+// partial results that the finishing kernel adds in a fixed order.
 template <typename E, int D>
 __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using v2 = typename M::v2;
     constexpr int KS = D / 16, DT = D / 32, JB = 256;
-    constexpr int LDK = D + 8, LDT = 32 + 8;
-    static_assert(D == 64, "tile builder below assumes 64 columns (16 threads x 4)");
+    constexpr int LDK = D + 8, LDU = 64 + 8;
+    static_assert(D == 64, "stage loader below assumes 512 threads x one 16-byte chunk per tensor");
 
-    __shared__ __align__(16) E sA[2][32][LDK];
-    __shared__ __align__(16) E sG[2][32][LDK];
-    __shared__ __align__(16) E sAT[2][D][LDT];
-    __shared__ __align__(16) E sGT[2][D][LDT];
-    __shared__ float sMeta[2][2];
+    extern __shared__ __align__(16) char smem[];
+    E* sK2 = reinterpret_cast<E*>(smem);   // [2][64][LDK]  rows k
+    E* sV2 = sK2 + 2 * 64 * LDK;           // [2][64][LDK]
+    E* sAT = sV2 + 2 * 64 * LDK;           // [2][D][LDU]   K2^T (.) Q[q]
+    E* sGT = sAT + 2 * D * LDU;            // [2][D][LDU]   V2^T (.) dO[q]
+    E* sQr = sGT + 2 * D * LDU;            // [2][D]  Q[q] of the round that starts in this buffer
+    E* sOr = sQr + 2 * D;                  // [2][D]  dO[q]
+    float* sMeta = reinterpret_cast<float*>(sOr + 2 * D);  // [2][2]  LSE2[q], Delta[q]
 
     const int njb = (p.T + JB - 1) / JB;
     int bid = blockIdx.x;
+    // heaviest first: low j blocks see the most queries
     const int chunk = bid % p.nqc; bid /= p.nqc;
-    const int jb = bid % njb;
-    const int bh = bid / njb;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int bh = bid % p.BH;
+    const int jb = bid / p.BH;
+    (void)njb;
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
-    const size_t base = (size_t)bh * T * D;
+    const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
     const E* __restrict__ Q = p.q + base;
     const E* __restrict__ dO = p.d_o + base;
     const E* __restrict__ K2 = p.k2 + base;
     const E* __restrict__ V2 = p.v2 + base;
+    const E* __restrict__ K2T = p.k2t + tbase;
+    const E* __restrict__ V2T = p.v2t + tbase;
     const float* __restrict__ LSE = p.lse + (size_t)bh * T;
     const float* __restrict__ DEL = p.delta + (size_t)bh * T;
     const float scale_log2 = p.alpha * kLog2e;
 
     const int j0 = jb * JB, jw = j0 + wave * 32;
     const int jrow = min(jw + n, T - 1);
-    v8 k1b[KS], ub[KS];
+    v8 k1raw[KS], uraw[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        k1b[ks] = *reinterpret_cast<const v8*>(p.k1 + base + (size_t)jrow * D + ks * 16 + g * 8);
-        ub[ks] = *reinterpret_cast<const v8*>(p.u + base + (size_t)jrow * D + ks * 16 + g * 8);
+        k1raw[ks] = *reinterpret_cast<const v8*>(p.k1 + base + (size_t)jrow * D + ks * 16 + g * 8);
+        uraw[ks] = *reinterpret_cast<const v8*>(p.u + base + (size_t)jrow * D + ks * 16 + g * 8);
     }
     f32x16 accK[DT], accU[DT];
 #pragma unroll
@@ -325,128 +344,154 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
             accU[dt][i] = 0.f;
         }
 
-    // virtual-row tiles handled by this workgroup: queries q = q_first + chunk + nqc*m, and for
-    // each of them the k-tiles 0 .. kmax(q)/32
+    // rounds: q = q_first + chunk + nqc*m ; stages of round q: 0 .. kmax(q)/64
     const int q_first = p.causal ? j0 : 0;
-    int bq_ = q_first + chunk, bkt = 0;  // builder cursor (next tile to build)
     auto kmax_of = [&](int q) { return p.causal ? q : T - 1; };
 
-    // builder: thread -> (k offset pk, 4 columns c4)
-    const int pk = tid >> 4, c4 = (tid & 15) * 4;
-    const int prow = c_row((pk >> 3) & 1, ((pk >> 4) << 3) | (pk & 7));  // MFMA row that holds k offset pk
-    uint2 lk, lv, lq, ld;
-    auto issue_tile = [&](int q, int kt) {
-        const size_t ko = (size_t)min(kt * 32 + pk, T - 1) * D + c4, qo = (size_t)q * D + c4;
-        lk = *reinterpret_cast<const uint2*>(K2 + ko);
-        lv = *reinterpret_cast<const uint2*>(V2 + ko);
-        lq = *reinterpret_cast<const uint2*>(Q + qo);
-        ld = *reinterpret_cast<const uint2*>(dO + qo);
+    // stage loader: thread -> one 16-byte chunk of each of the four tensors
+    const int lr = tid >> 3, lc = tid & 7;  // K2/V2: row lr, chunk lc ; K2T/V2T: d = lr, key chunk lc
+    uint4 l1, l2, l3, l4;
+    E lqd, lod;
+    auto issue_stage = [&](int q, int st) {
+        const int kb = st * 64;
+        const size_t off = (size_t)min(kb + lr, T - 1) * D + lc * 8;
+        l1 = *reinterpret_cast<const uint4*>(K2 + off);
+        l2 = *reinterpret_cast<const uint4*>(V2 + off);
+        const size_t offt = (size_t)lr * p.Tp + kb + lc * 8;
+        l3 = *reinterpret_cast<const uint4*>(K2T + offt);
+        l4 = *reinterpret_cast<const uint4*>(V2T + offt);
+        lqd = Q[(size_t)q * D + lr];
+        lod = dO[(size_t)q * D + lr];
     };
-    auto commit_tile = [&](int buf, int q) {
-        typedef __attribute__((ext_vector_type(4))) E v4;
-        const v4 kv = *reinterpret_cast<const v4*>(&lk), vv = *reinterpret_cast<const v4*>(&lv);
-        const v4 qv = *reinterpret_cast<const v4*>(&lq), dv = *reinterpret_cast<const v4*>(&ld);
-        v4 a, gg;
+    auto commit_stage = [&](int buf, int q, int st) {
+        *reinterpret_cast<uint4*>(sK2 + (buf * 64 + lr) * LDK + lc * 8) = l1;
+        *reinterpret_cast<uint4*>(sV2 + (buf * 64 + lr) * LDK + lc * 8) = l2;
+        const v8 kt = *reinterpret_cast<const v8*>(&l3), vt = *reinterpret_cast<const v8*>(&l4);
+        const float qd = (float)lqd, od = (float)lod;
+        v8 a, gg;
 #pragma unroll
-        for (int e = 0; e < 4; e += 2) {
-            const v2 pa = M::pack((float)kv[e] * (float)qv[e] * scale_log2,
-                                  (float)kv[e + 1] * (float)qv[e + 1] * scale_log2);
-            const v2 pb = M::pack((float)vv[e] * (float)dv[e], (float)vv[e + 1] * (float)dv[e + 1]);
+        for (int e = 0; e < 8; e += 2) {
+            const v2 pa = M::pack((float)kt[e] * qd, (float)kt[e + 1] * qd);
+            const v2 pb = M::pack((float)vt[e] * od, (float)vt[e + 1] * od);
             a[e] = pa[0]; a[e + 1] = pa[1];
             gg[e] = pb[0]; gg[e + 1] = pb[1];
         }
-        *reinterpret_cast<v4*>(&sA[buf][prow][c4]) = a;
-        *reinterpret_cast<v4*>(&sG[buf][prow][c4]) = gg;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            sAT[buf][c4 + e][pk] = a[e];
-            sGT[buf][c4 + e][pk] = gg[e];
-        }
-        if (tid == 0) {
-            sMeta[buf][0] = LSE[q] * kLog2e;
-            sMeta[buf][1] = DEL[q];
+        *reinterpret_cast<v8*>(sAT + (buf * D + lr) * LDU + lc * 8) = a;
+        *reinterpret_cast<v8*>(sGT + (buf * D + lr) * LDU + lc * 8) = gg;
+        if (st == 0) {  // first stage of a round also carries the round's query row and scalars
+            if (lc == 0) {
+                sQr[buf * D + lr] = lqd;
+                sOr[buf * D + lr] = lod;
+            }
+            if (tid == 0) {
+                sMeta[buf * 2] = LSE[q] * kLog2e;
+                sMeta[buf * 2 + 1] = DEL[q];
+            }
         }
     };
 
-    if (bq_ >= T) {
-        // no query for this chunk: still write (zero) partials below
-    }
-    int cq = bq_, ckt = 0;  // consumer cursor
+    int cq = q_first + chunk, cst = 0;  // current (round, stage)
     bool have = cq < T;
     if (have) {
-        issue_tile(bq_, bkt);
-        commit_tile(0, bq_);
+        issue_stage(cq, 0);
+        commit_stage(0, cq, 0);
     }
     __syncthreads();
+
+    const int krow_off = key_of_row(n);
+    v8 k1q[KS], uq[KS];
+    float lse2 = 0.f, delta = 0.f;
     int buf = 0;
     while (have) {
-        // advance the builder cursor to the tile after (cq, ckt)
-        int nq = cq, nkt_ = ckt + 1;
-        if (nkt_ * 32 > kmax_of(cq)) {
+        const int kmax = kmax_of(cq), jlim = p.causal ? cq : T - 1;
+        const bool active = (jw <= jlim) && (jw < T);  // wave-uniform
+        int nq = cq, nst = cst + 1;
+        if (nst * 64 > kmax) {
             nq = cq + p.nqc;
-            nkt_ = 0;
+            nst = 0;
         }
         const bool next = nq < T;
-        if (next) issue_tile(nq, nkt_);
+        if (next) issue_stage(nq, nst);
 
-        const int kmax = kmax_of(cq), jlim = p.causal ? cq : T - 1;
-        if (jw <= jlim && jw < T) {
-            const float lse2 = sMeta[buf][0], delta = sMeta[buf][1];
-            f32x16 s, dp;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                s[i] = 0.f;
-                dp[i] = 0.f;
-            }
+        if (cst == 0 && active) {
+            // new round: operands of this wave for query cq
+            lse2 = sMeta[buf * 2];
+            delta = sMeta[buf * 2 + 1];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const v8 a = *reinterpret_cast<const v8*>(&sA[buf][n][ks * 16 + g * 8]);
-                s = M::mma(a, k1b[ks], s);
-            }
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const v8 a = *reinterpret_cast<const v8*>(&sG[buf][n][ks * 16 + g * 8]);
-                dp = M::mma(a, ub[ks], dp);
-            }
-            const bool diag = (ckt * 32 + 31 > kmax) || (jw + 31 > jlim) || (jw + 31 >= T);
-            const bool jok = (jw + n <= jlim) && (jw + n < T);
-            v8 pa[2], da[2];
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
+                const v8 qv = *reinterpret_cast<const v8*>(sQr + buf * D + ks * 16 + g * 8);
+                const v8 ov = *reinterpret_cast<const v8*>(sOr + buf * D + ks * 16 + g * 8);
+                v8 a, b;
 #pragma unroll
                 for (int e = 0; e < 8; e += 2) {
-                    const int i = h * 8 + e;
-                    float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
-                    if (diag) {
-                        p0 = (jok && ckt * 32 + key_of(g, i) <= kmax) ? p0 : 0.f;
-                        p1 = (jok && ckt * 32 + key_of(g, i + 1) <= kmax) ? p1 : 0.f;
-                    }
-                    const v2 pp = M::pack(p0, p1);
-                    const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
-                    pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
-                    da[h][e] = dd[0]; da[h][e + 1] = dd[1];
+                    const v2 pa = M::pack((float)k1raw[ks][e] * (float)qv[e] * scale_log2,
+                                          (float)k1raw[ks][e + 1] * (float)qv[e + 1] * scale_log2);
+                    const v2 pb = M::pack((float)uraw[ks][e] * (float)ov[e], (float)uraw[ks][e + 1] * (float)ov[e + 1]);
+                    a[e] = pa[0]; a[e + 1] = pa[1];
+                    b[e] = pb[0]; b[e + 1] = pb[1];
                 }
+                k1q[ks] = a;
+                uq[ks] = b;
             }
+        }
+
+        if (active) {
+            const bool jok = (jw + n <= jlim) && (jw + n < T);
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
+            for (int half = 0; half < 2; ++half) {
+                const int kb = cst * 64 + half * 32;
+                if (kb > kmax) break;
+                f32x16 s, dp;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = 0.f;
+                    dp[i] = 0.f;
+                }
+                const int rowoff = (buf * 64 + half * 32 + krow_off) * LDK + g * 8;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    s = M::mma(*reinterpret_cast<const v8*>(sK2 + rowoff + ks * 16), k1q[ks], s);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    dp = M::mma(*reinterpret_cast<const v8*>(sV2 + rowoff + ks * 16), uq[ks], dp);
+                const bool diag = (kb + 31 > kmax) || (jw + 31 > jlim) || (jw + 31 >= T);
+                v8 pa[2], da[2];
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const v8 at = *reinterpret_cast<const v8*>(&sAT[buf][dt * 32 + n][h * 16 + g * 8]);
-                    const v8 gt = *reinterpret_cast<const v8*>(&sGT[buf][dt * 32 + n][h * 16 + g * 8]);
-                    accK[dt] = M::mma(da[h], at, accK[dt]);
-                    accU[dt] = M::mma(pa[h], gt, accU[dt]);
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2) {
+                        const int i = h * 8 + e;
+                        float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
+                        if (diag) {
+                            p0 = (jok && kb + key_of(g, i) <= kmax) ? p0 : 0.f;
+                            p1 = (jok && kb + key_of(g, i + 1) <= kmax) ? p1 : 0.f;
+                        }
+                        const v2 pp = M::pack(p0, p1);
+                        const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
+                        pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
+                        da[h][e] = dd[0]; da[h][e + 1] = dd[1];
+                    }
+                }
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int toff = (buf * D + dt * 32 + n) * LDU + half * 32 + h * 16 + g * 8;
+                        accK[dt] = M::mma(da[h], *reinterpret_cast<const v8*>(sAT + toff), accK[dt]);
+                        accU[dt] = M::mma(pa[h], *reinterpret_cast<const v8*>(sGT + toff), accU[dt]);
+                    }
                 }
             }
         }
-        if (next) commit_tile(buf ^ 1, nq);
+        if (next) commit_stage(buf ^ 1, nq, nst);
         __syncthreads();
         buf ^= 1;
         cq = nq;
-        ckt = nkt_;
+        cst = nst;
         have = next;
     }
 
-    // partial results of this query chunk
+    // partial results of this query chunk (dK1 still lacks the factor alpha: applied by the finisher)
     float* outK = p.dk1part + ((size_t)chunk * p.BH + bh) * T * D;
     float* outU = p.dupart + ((size_t)chunk * p.BH + bh) * T * D;
 #pragma unroll
@@ -467,21 +512,28 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
 // zero the fp32 accumulators.
 template <typename E>
 __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1, const E* __restrict__ k1,
+                                                       const E* __restrict__ k2, const E* __restrict__ v2,
                                                        const E* __restrict__ o, const E* __restrict__ d_o,
                                                        E* __restrict__ u, E* __restrict__ ut, E* __restrict__ k1t,
+                                                       E* __restrict__ k2t, E* __restrict__ v2t,
                                                        float* __restrict__ delta, float* __restrict__ zero_a,
                                                        float* __restrict__ zero_b, int T, int Tp, int D) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * Tp;
     for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
         const int d = idx >> 6, jj = idx & 63, j = j0 + jj;
-        float uv = 0.f, kv = 0.f;
+        float uv = 0.f, kv = 0.f, k2v = 0.f, v2v = 0.f;
         if (j < T) {
-            uv = silu_f((float)v1[base + (size_t)j * D + d]);
-            kv = (float)k1[base + (size_t)j * D + d];
+            const size_t off = base + (size_t)j * D + d;
+            uv = silu_f((float)v1[off]);
+            kv = (float)k1[off];
+            k2v = (float)k2[off];
+            v2v = (float)v2[off];
         }
         ut[tbase + (size_t)d * Tp + j] = (E)uv;
         k1t[tbase + (size_t)d * Tp + j] = (E)kv;
+        k2t[tbase + (size_t)d * Tp + j] = (E)k2v;
+        v2t[tbase + (size_t)d * Tp + j] = (E)v2v;
     }
     for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
         const int jj = idx / D, d = idx % D, j = j0 + jj;
@@ -504,21 +556,21 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
     }
 }
 
-// dK1 = ln2 * sum_c part_c ; dV1 = SiLU'(V1) * sum_c part_c ; dK2, dV2 = converted accumulators
+// dK1 = alpha * sum_c part_c ; dV1 = SiLU'(V1) * sum_c part_c ; dK2, dV2 = converted accumulators
 template <typename E>
 __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict__ dk1part,
                                                          const float* __restrict__ dupart,
                                                          const float* __restrict__ dk2acc,
                                                          const float* __restrict__ dv2acc, const E* __restrict__ v1,
                                                          E* __restrict__ dk1, E* __restrict__ dv1, E* __restrict__ dk2,
-                                                         E* __restrict__ dv2, size_t n, int nqc) {
+                                                         E* __restrict__ dv2, size_t n, int nqc, float alpha) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
         float a = 0.f, b = 0.f;
         for (int c = 0; c < nqc; ++c) {
             a += dk1part[(size_t)c * n + i];
             b += dupart[(size_t)c * n + i];
         }
-        dk1[i] = (E)(a * kLn2);
+        dk1[i] = (E)(a * alpha);
         dv1[i] = (E)(b * silu_grad_f((float)v1[i]));
         dk2[i] = (E)dk2acc[i];
         dv2[i] = (E)dv2acc[i];
@@ -528,7 +580,7 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
 constexpr int kNqc = 8;
 
 struct BwdLayout {
-    size_t u, ut, k1t, delta, dk2acc, dv2acc, dk1part, dupart, total;
+    size_t u, ut, k1t, k2t, v2t, delta, dk2acc, dv2acc, dk1part, dupart, total;
 };
 static BwdLayout bwd_layout(int BH, int T, int D) {
     const size_t Tp = (size_t)(T + 63) / 64 * 64, n = (size_t)BH * T * D;
@@ -543,6 +595,8 @@ static BwdLayout bwd_layout(int BH, int T, int D) {
     l.u = take(n * 2);
     l.ut = take((size_t)BH * D * Tp * 2);
     l.k1t = take((size_t)BH * D * Tp * 2);
+    l.k2t = take((size_t)BH * D * Tp * 2);
+    l.v2t = take((size_t)BH * D * Tp * 2);
     l.delta = take((size_t)BH * T * 4);
     l.dk2acc = take(n * 4);
     l.dv2acc = take(n * 4);
@@ -561,6 +615,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
     p.d_o = (const E*)a.d_o;
     p.u = (const E*)(ws + l.u); p.ut = (const E*)(ws + l.ut); p.k1t = (const E*)(ws + l.k1t);
+    p.k2t = (const E*)(ws + l.k2t); p.v2t = (const E*)(ws + l.v2t);
     p.lse = a.lse; p.delta = (const float*)(ws + l.delta);
     p.dq = (E*)a.dq;
     p.dk2acc = (float*)(ws + l.dk2acc); p.dv2acc = (float*)(ws + l.dv2acc);
@@ -569,7 +624,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.alpha = a.alpha; p.causal = a.causal;
 
     hipLaunchKernelGGL(bwd_prep_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (const E*)a.k1,
-                       (const E*)a.o, (const E*)a.d_o, (E*)(ws + l.u), (E*)(ws + l.ut), (E*)(ws + l.k1t),
+                       (const E*)a.k2, (const E*)a.v2, (const E*)a.o, (const E*)a.d_o, (E*)(ws + l.u),
+                       (E*)(ws + l.ut), (E*)(ws + l.k1t), (E*)(ws + l.k2t), (E*)(ws + l.v2t),
                        (float*)(ws + l.delta), p.dk2acc, p.dv2acc, a.T, Tp, D);
 
     constexpr size_t smem = 2 * (size_t)(2 * 2 * 64 * (D + 8) + 2 * 2 * D * 72 + 2 * 2 * 32 * (D + 8) + 2 * 8 * (D + 8)) +
@@ -586,14 +642,23 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p);
 
     const int njb = (a.T + 255) / 256;
-    hipLaunchKernelGGL((tdp_bwd_j_kernel<E, D>), dim3(a.BH * njb * kNqc), dim3(512), 0, st, p);
+    constexpr size_t smem_j = 2 * (size_t)(2 * 2 * 64 * (D + 8) + 2 * 2 * D * 72 + 2 * 2 * D) + 16;
+    auto kern_j = tdp_bwd_j_kernel<E, D>;
+    static bool attr_j = false;
+    if (!attr_j) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_j),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_j);
+        if (e != hipSuccess) return e;
+        attr_j = true;
+    }
+    hipLaunchKernelGGL(kern_j, dim3(a.BH * njb * kNqc), dim3(512), smem_j, st, p);
 
     const size_t n = (size_t)a.BH * a.T * D;
     size_t gridf = (n + 255) / 256;
     if (gridf > 4096) gridf = 4096;
     hipLaunchKernelGGL(bwd_finish_kernel<E>, dim3((unsigned)gridf), dim3(256), 0, st, (const float*)p.dk1part,
                        (const float*)p.dupart, (const float*)p.dk2acc, (const float*)p.dv2acc, (const E*)a.v1,
-                       (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n, kNqc);
+                       (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n, kNqc, a.alpha);
     return hipGetLastError();
 }
 
