@@ -19,6 +19,8 @@
 //    transposes are built cooperatively in LDS.  dK1/dU stay in registers; the query range is
 //    split over NQC workgroups whose fp32 partial results are summed by the finishing kernel
 //    (no atomics, fixed order).
+#include <type_traits>
+
 #include "kernels.hpp"
 #include "mfma.hpp"
 
@@ -65,7 +67,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
     const int qt = p.nqt - 1 - slot / groups;
     if (bh >= p.BH) return;
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
     const E* __restrict__ K1 = p.k1 + base;
@@ -214,24 +217,33 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
                     const v8 ua = *reinterpret_cast<const v8*>(sU + rowoff + ks * 16);
                     dp = M::mma(ua, bg[ks], dp);
                 }
-                const bool diag = jb + 31 > jmax;
                 v8 pa[2], da[2];
+                // P = exp2(S - LSE2), dS = P (dP - Delta), both packed as A operands of the next
+                // products.  The masked variant is a separate (wave-uniform) branch so that interior
+                // steps carry no predication at all.
+                auto softmax_grad = [&](auto masked_tag) {
+                    constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
+                    for (int h = 0; h < 2; ++h) {
 #pragma unroll
-                    for (int e = 0; e < 8; e += 2) {
-                        const int i = h * 8 + e;
-                        float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
-                        if (diag) {
-                            p0 = (jb + key_of(g, i) <= jmax) ? p0 : 0.f;
-                            p1 = (jb + key_of(g, i + 1) <= jmax) ? p1 : 0.f;
+                        for (int e = 0; e < 8; e += 2) {
+                            const int i = h * 8 + e;
+                            float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
+                            if constexpr (MASKED) {
+                                p0 = (jb + key_of(g, i) <= jmax) ? p0 : 0.f;
+                                p1 = (jb + key_of(g, i + 1) <= jmax) ? p1 : 0.f;
+                            }
+                            const v2 pp = M::pack(p0, p1);
+                            const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
+                            pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
+                            da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                         }
-                        const v2 pp = M::pack(p0, p1);
-                        const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
-                        pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
-                        da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                     }
-                }
+                };
+                if (__builtin_amdgcn_readfirstlane(jb + 31 > jmax))
+                    softmax_grad(std::true_type{});
+                else
+                    softmax_grad(std::false_type{});
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -456,22 +468,29 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
                     dp = M::mma(*reinterpret_cast<const v8*>(sV2 + rowoff + ks * 16), uq[ks], dp);
                 const bool diag = (kb + 31 > kmax) || (jw + 31 > jlim) || (jw + 31 >= T);
                 v8 pa[2], da[2];
+                auto softmax_grad = [&](auto masked_tag) {
+                    constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
+                    for (int h = 0; h < 2; ++h) {
 #pragma unroll
-                    for (int e = 0; e < 8; e += 2) {
-                        const int i = h * 8 + e;
-                        float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
-                        if (diag) {
-                            p0 = (jok && kb + key_of(g, i) <= kmax) ? p0 : 0.f;
-                            p1 = (jok && kb + key_of(g, i + 1) <= kmax) ? p1 : 0.f;
+                        for (int e = 0; e < 8; e += 2) {
+                            const int i = h * 8 + e;
+                            float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
+                            if constexpr (MASKED) {
+                                p0 = (jok && kb + key_of(g, i) <= kmax) ? p0 : 0.f;
+                                p1 = (jok && kb + key_of(g, i + 1) <= kmax) ? p1 : 0.f;
+                            }
+                            const v2 pp = M::pack(p0, p1);
+                            const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
+                            pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
+                            da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                         }
-                        const v2 pp = M::pack(p0, p1);
-                        const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
-                        pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
-                        da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                     }
-                }
+                };
+                if (__builtin_amdgcn_readfirstlane(diag))
+                    softmax_grad(std::true_type{});
+                else
+                    softmax_grad(std::false_type{});
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
