@@ -156,6 +156,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) dqpart[dt] = 0.f;
     const int krow_off = key_of_row(n);
+    const v8 ones = ones_operand<E>(g), off_lse = offset_operand<E>(lse2, g), off_delta = offset_operand<E>(delta, g);
 
     int gstage = 0;
     for (int kt = 0; kt < nkt; ++kt) {
@@ -207,11 +208,14 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
                     dp[i] = 0.f;
                 }
                 const int rowoff = (sb * 64 + half * 32 + krow_off) * LDK + g * 8;
+                // the extra k-step subtracts LSE2[q] from S and Delta[q] from dP inside the MFMA
+                s = M::mma(ones, off_lse, s);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const v8 ka = *reinterpret_cast<const v8*>(sK1 + rowoff + ks * 16);
                     s = M::mma(ka, bq[ks], s);
                 }
+                dp = M::mma(ones, off_delta, dp);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const v8 ua = *reinterpret_cast<const v8*>(sU + rowoff + ks * 16);
@@ -228,13 +232,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
 #pragma unroll
                         for (int e = 0; e < 8; e += 2) {
                             const int i = h * 8 + e;
-                            float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
+                            float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
                             if constexpr (MASKED) {
                                 p0 = (jb + key_of(g, i) <= jmax) ? p0 : 0.f;
                                 p1 = (jb + key_of(g, i + 1) <= jmax) ? p1 : 0.f;
                             }
                             const v2 pp = M::pack(p0, p1);
-                            const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
+                            const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
                             pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
                             da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                         }
@@ -412,7 +416,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
 
     const int krow_off = key_of_row(n);
     v8 k1q[KS], uq[KS];
-    float lse2 = 0.f, delta = 0.f;
+    const v8 ones = ones_operand<E>(g);
+    v8 off_lse = ones, off_delta = ones;
     int buf = 0;
     while (have) {
         const int kmax = kmax_of(cq), jlim = p.causal ? cq : T - 1;
@@ -427,8 +432,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
 
         if (cst == 0 && active) {
             // new round: operands of this wave for query cq
-            lse2 = sMeta[buf * 2];
-            delta = sMeta[buf * 2 + 1];
+            off_lse = offset_operand<E>(sMeta[buf * 2], g);
+            off_delta = offset_operand<E>(sMeta[buf * 2 + 1], g);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const v8 qv = *reinterpret_cast<const v8*>(sQr + buf * D + ks * 16 + g * 8);
@@ -460,9 +465,11 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
                     dp[i] = 0.f;
                 }
                 const int rowoff = (buf * 64 + half * 32 + krow_off) * LDK + g * 8;
+                s = M::mma(ones, off_lse, s);  // S - LSE2[q], dP - Delta[q] come out of the MFMA
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks)
                     s = M::mma(*reinterpret_cast<const v8*>(sK2 + rowoff + ks * 16), k1q[ks], s);
+                dp = M::mma(ones, off_delta, dp);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks)
                     dp = M::mma(*reinterpret_cast<const v8*>(sV2 + rowoff + ks * 16), uq[ks], dp);
@@ -475,13 +482,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
 #pragma unroll
                         for (int e = 0; e < 8; e += 2) {
                             const int i = h * 8 + e;
-                            float p0 = fast_exp2(s[i] - lse2), p1 = fast_exp2(s[i + 1] - lse2);
+                            float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
                             if constexpr (MASKED) {
                                 p0 = (jok && kb + key_of(g, i) <= kmax) ? p0 : 0.f;
                                 p1 = (jok && kb + key_of(g, i + 1) <= kmax) ? p1 : 0.f;
                             }
                             const v2 pp = M::pack(p0, p1);
-                            const v2 dd = M::pack(p0 * (dp[i] - delta), p1 * (dp[i + 1] - delta));
+                            const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
                             pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
                             da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                         }
