@@ -7,20 +7,14 @@
 //   S, dP, dQK2 = dS K1, Tv = P U, dK1 += dS^T A, dU += P^T G
 // They are evaluated by two kernels, each recomputing S and dP (8 products executed for 6):
 //
-//  * tdp_bwd_qk_kernel: owner = 8 queries (one per wave); same loop nest as the forward
-//    (k-tiles of 32 outside, 64-row stages of K1/U inside).  Accumulates dQK2 and Tv over the
-//    whole j loop in registers, then per k-tile:  dQ[q] += sum_k dQK2 (.) K2[k] (registers,
-//    owner-computes), and the two per-k sums  dK2[k] += dQK2 (.) Q[q],  dV2[k] += Tv (.) dO[q]
-//    are first reduced over the workgroup's 8 queries in LDS and then added to fp32 global
-//    accumulators (one returnless atomic per element per (query group, k-tile)).
-//
-//  * tdp_bwd_j_kernel: owner = 256 K1/V1 rows (32 per wave, operands held in registers for the
-//    whole kernel); streams virtual-row tiles (one q, 32 k) whose operands A, G and their
-//    transposes are built cooperatively in LDS.  dK1/dU stay in registers; the query range is
-//    split over NQC workgroups whose fp32 partial results are summed by the finishing kernel
-//    (no atomics, fixed order).
+//  * tdp_bwd_qk_kernel: owner = 32 queries; tiles are (32 q) x (1 k), j is streamed.  Produces dQ
+//    (owner-computes) and dK2 / dV2 (one fp32 atomic per element per (query tile, k)).
+//  * tdp_bwd_j_kernel: owner = 256 K1/V1 rows; per query, k is streamed.  Produces dK1 / dV1 with
+//    no atomics (fp32 partials per query chunk, summed in a fixed order by the finishing kernel).
+// See the comment above each kernel.
 #include <type_traits>
 
+#include "direct_lds.hpp"
 #include "kernels.hpp"
 #include "mfma.hpp"
 
@@ -40,31 +34,39 @@ struct BwdParams {
 };
 
 // ------------------------------------------------------------------------------------------
+// Owner = 32 consecutive queries (the columns of every MFMA tile of the workgroup).  The eight
+// waves take eight consecutive K2/V2 rows k per "round" (one k per wave), so a tile is
+// (32 q) x (1 k), and sweep j in 64-row stages of K1 / U (and their transposes) shared by the
+// workgroup.  Per round and wave, over the whole j sweep:
+//   Yq[(q,k), :] = sum_j dS K1[j, :]        Tv[(q,k), :] = sum_j P U[j, :]
+// and then
+//   dQ[q]  += Yq (.) K2[k]                      (registers, all rounds; reduced over waves at the end)
+//   dK2[k] += alpha * sum_q Yq (.) Q[q]         (sum over the tile's 32 rows in registers, then ONE
+//   dV2[k] += sum_q Tv (.) dO[q]                 returnless fp32 atomic per element per (q-tile, k))
 template <typename E, int D>
 __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using v2 = typename M::v2;
-    constexpr int KS = D / 16, DT = D / 32, BQ = 8;
-    constexpr int LDK = D + 8, LDU = 64 + 8, LDA = D + 4;
-    constexpr int CH = D / 64;
+    constexpr int KS = D / 16, DT = D / 32, BQ = 32;
+    constexpr int LDK = D + 8, LDF = D + 4;
+    constexpr int TILE = 64 * 64;  // elements of one dense, swizzled 64x64 stage tile (see direct_lds.hpp)
+    constexpr int NBUF = 3, LW = 4;  // stages in flight; direct loads per wave per stage
+    static_assert(D == 64, "stages are four 64x64 tiles = 32 blocks of 1 KB, four per wave");
 
     extern __shared__ __align__(16) char smem[];
-    E* sK1 = reinterpret_cast<E*>(smem);   // [2][64][LDK]
-    E* sU = sK1 + 2 * 64 * LDK;            // [2][64][LDK]
-    E* sK1T = sU + 2 * 64 * LDK;           // [2][D][LDU]
-    E* sUT = sK1T + 2 * D * LDU;           // [2][D][LDU]
-    E* sK2 = sUT + 2 * D * LDU;            // [2][32][LDK]
-    E* sV2 = sK2 + 2 * 32 * LDK;           // [2][32][LDK]
-    E* sQ = sV2 + 2 * 32 * LDK;            // [BQ][LDK]
-    E* sDO = sQ + BQ * LDK;                // [BQ][LDK]
-    float* sAccK = reinterpret_cast<float*>(sDO + BQ * LDK);  // [32][LDA]
-    float* sAccV = sAccK + 32 * LDA;                          // [32][LDA]
+    E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][4 tensors: K1, U, K1^T, U^T][TILE]
+    E* sKr = sStage + NBUF * 4 * TILE;       // [2][8][D]  K2 rows of a round (one per wave), dense
+    E* sVr = sKr + 2 * 8 * D;                // [2][8][D]  V2 rows
+    E* sQb = sVr + 2 * 8 * LDK;            // [BQ][LDK]    Q tile (operand build)
+    E* sOb = sQb + BQ * LDK;               // [BQ][LDK]    dO tile
+    float* sQf = reinterpret_cast<float*>(sOb + BQ * LDK);  // [BQ][LDF]  alpha * Q, fp32 (epilogue)
+    float* sOf = sQf + BQ * LDF;                            // [BQ][LDF]  dO, fp32
 
     const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;
+    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
     if (bh >= p.BH) return;
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
@@ -79,98 +81,87 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
     const E* __restrict__ UT = p.ut + tbase;
 
     const int q0 = qt * BQ;
-    const int jend = p.causal ? min(T - 1, q0 + BQ - 1) : T - 1;
-    const int nst = jend / 64 + 1, nkt = jend / 32 + 1;
-    const int q = q0 + wave;
+    const int qlast = min(T - 1, q0 + BQ - 1);
+    const int jend = p.causal ? qlast : T - 1;  // last j (and last k) any query of the tile needs
+    const int nst = jend / 64 + 1, nrounds = jend / 8 + 1;
+    const int q = q0 + n;                        // this lane's column
     const bool q_ok = q < T;
-    const int qc = min(q, T - 1);
-    const int jmax = p.causal ? qc : T - 1;
-    const float lse2 = p.lse[(size_t)bh * T + qc] * kLog2e;
-    const float delta = p.delta[(size_t)bh * T + qc];
+    const int jq = p.causal ? min(q, T - 1) : T - 1;  // per-lane bound on j and k
     const float scale_log2 = p.alpha * kLog2e;
 
-    uint4 r1[CH], r2[CH], r3[CH], r4[CH], rkv[CH];
-    auto issue_stage = [&](int st) {
+    // stage loader: wave w fetches blocks 4*(w%2) .. +3 (8 rows each) of tensor w/2, direct to LDS
+    const int tensor = wave >> 1;
+    const bool rowmajor = tensor < 2;  // K1 / U: row = key j (read with permuted rows); else row = d
+    const E* gsrc = uniform_ptr(tensor == 0 ? K1 : tensor == 1 ? U : tensor == 2 ? K1T : UT);
+    auto issue_stage = [&](int st, int buf) {
         const int jb = st * 64;
+        int ln = lane;
+        asm volatile("" : "+v"(ln));  // keep this address arithmetic inside the loops (no spilled invariants)
+        const int pos = ln & 7, rr = ln >> 3;
+        E* dst = sStage + (buf * 4 + tensor) * TILE;
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int r = idx / (D / 8), ch = idx % (D / 8);
-            const size_t off = (size_t)min(jb + r, T - 1) * D + ch * 8;
-            r1[c] = *reinterpret_cast<const uint4*>(K1 + off);
-            r2[c] = *reinterpret_cast<const uint4*>(U + off);
-            const int d = idx / 8, cj = idx % 8;
-            const size_t offt = (size_t)d * p.Tp + jb + cj * 8;
-            r3[c] = *reinterpret_cast<const uint4*>(K1T + offt);
-            r4[c] = *reinterpret_cast<const uint4*>(UT + offt);
+        for (int c = 0; c < LW; ++c) {
+            const int blk = (wave & 1) * 4 + c, r = blk * 8 + rr;
+            const unsigned off = rowmajor ? (unsigned)min(jb + r, T - 1) * (D * 2) + ((pos ^ swz_perm(r)) * 16)
+                                          : ((unsigned)r * p.Tp + jb) * 2 + ((pos ^ swz_seq(r)) * 16);
+            direct_load_16(gsrc, off, dst + blk * 512);
         }
     };
-    auto commit_stage = [&](int buf) {
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int r = idx / (D / 8), ch = idx % (D / 8);
-            *reinterpret_cast<uint4*>(sK1 + (buf * 64 + r) * LDK + ch * 8) = r1[c];
-            *reinterpret_cast<uint4*>(sU + (buf * 64 + r) * LDK + ch * 8) = r2[c];
-            const int d = idx / 8, cj = idx % 8;
-            *reinterpret_cast<uint4*>(sK1T + (buf * D + d) * LDU + cj * 8) = r3[c];
-            *reinterpret_cast<uint4*>(sUT + (buf * D + d) * LDU + cj * 8) = r4[c];
-        }
-    };
-    auto issue_ktile = [&](int kt) {
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int which = idx / (4 * D), rem = idx % (4 * D);
-            const int r = rem / (D / 8), ch = rem % (D / 8);
-            const E* src = which ? V2 : K2;
-            rkv[c] = *reinterpret_cast<const uint4*>(src + (size_t)min(kt * 32 + r, T - 1) * D + ch * 8);
-        }
-    };
-    auto commit_ktile = [&](int buf) {
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int idx = tid + c * 512;
-            const int which = idx / (4 * D), rem = idx % (4 * D);
-            const int r = rem / (D / 8), ch = rem % (D / 8);
-            E* dst = which ? sV2 : sK2;
-            *reinterpret_cast<uint4*>(dst + (buf * 32 + r) * LDK + ch * 8) = rkv[c];
+    auto issue_round = [&](int m, int buf) {  // waves 0, 1: K2 / V2 rows 8m .. 8m+7 (1 KB each)
+        if (wave < 2) {
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const unsigned off = (unsigned)min(m * 8 + (ln >> 3), T - 1) * (D * 2) + (ln & 7) * 16;
+            direct_load_16(uniform_ptr(wave ? V2 : K2), off, (wave ? sVr : sKr) + buf * 8 * D);
         }
     };
 
-    // prologue: Q and dO rows of the group, zeroed LDS accumulators, first k-tile and stage
-    for (int idx = tid; idx < 2 * BQ * (D / 8); idx += 512) {
-        const int which = idx / (BQ * (D / 8)), rem = idx % (BQ * (D / 8));
-        const int r = rem / (D / 8), ch = rem % (D / 8);
-        const E* src = (which ? p.d_o : p.q) + base + (size_t)min(q0 + r, T - 1) * D + ch * 8;
-        *reinterpret_cast<uint4*>((which ? sDO : sQ) + r * LDK + ch * 8) = *reinterpret_cast<const uint4*>(src);
+    // prologue: Q / dO tiles in both forms, first round, first stage
+    for (int idx = tid; idx < BQ * D; idx += 512) {
+        const int r = idx / D, d = idx % D;
+        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
+        const E qv = p.q[off], ov = p.d_o[off];
+        sQb[r * LDK + d] = qv;
+        sOb[r * LDK + d] = ov;
+        sQf[r * LDF + d] = (float)qv * p.alpha;
+        sOf[r * LDF + d] = (float)ov;
     }
-    for (int idx = tid; idx < 2 * 32 * LDA; idx += 512) sAccK[idx] = 0.f;  // sAccK and sAccV are adjacent
-    issue_ktile(0);
-    issue_stage(0);
-    commit_ktile(0);
-    commit_stage(0);
+    issue_stage(0, 0);
+    issue_stage(nst > 1 ? 1 : 0, 1);
+    issue_round(0, 0);
+    wait_vmcnt<0>();
     __syncthreads();
 
-    float dqpart[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) dqpart[dt] = 0.f;
-    const int krow_off = key_of_row(n);
+    // per-column constants folded into the score products (see offset_operand); a column past the
+    // end of the sequence gets a huge LSE so that its P underflows to exactly 0
+    const float lse2 = q_ok ? p.lse[(size_t)bh * T + q] * kLog2e : 3.0e4f;  // representable in fp16 too
+    const float delta = q_ok ? p.delta[(size_t)bh * T + q] : 0.f;
     const v8 ones = ones_operand<E>(g), off_lse = offset_operand<E>(lse2, g), off_delta = offset_operand<E>(delta, g);
+    const int krow_off = key_of_row(n);
+    const int fperm = swz_perm(krow_off), fseq = swz_seq(n);
+
+    f32x16 dQacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dQacc[dt][i] = 0.f;
 
     int gstage = 0;
-    for (int kt = 0; kt < nkt; ++kt) {
-        const int kb = kt & 1;
-        if (kt + 1 < nkt) issue_ktile(kt + 1);
+    for (int m = 0; m < nrounds; ++m) {
+        const int mb = m & 1;
+        const int k = m * 8 + wave;                 // this wave's K2/V2 row
+        const bool k_active = k <= jend;            // wave-uniform
+        const bool k_diag = p.causal && k > q0;     // some columns of the tile have q < k
+        const bool kv_ok = !p.causal || k <= jq;    // per lane
 
         v8 bq[KS], bg[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int off = ks * 16 + g * 8;
-            const v8 kv = *reinterpret_cast<const v8*>(sK2 + (kb * 32 + n) * LDK + off);
-            const v8 vv = *reinterpret_cast<const v8*>(sV2 + (kb * 32 + n) * LDK + off);
-            const v8 qv = *reinterpret_cast<const v8*>(sQ + wave * LDK + off);
-            const v8 dv = *reinterpret_cast<const v8*>(sDO + wave * LDK + off);
+            const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * 8 + wave) * D + off);
+            const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * 8 + wave) * D + off);
+            const v8 qv = *reinterpret_cast<const v8*>(sQb + n * LDK + off);
+            const v8 dv = *reinterpret_cast<const v8*>(sOb + n * LDK + off);
             v8 a, b;
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
@@ -194,101 +185,121 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
             }
 
         for (int st = 0; st < nst; ++st, ++gstage) {
-            const int sb = gstage & 1;
-            const bool more = (st + 1 < nst) || (kt + 1 < nkt);
-            if (more) issue_stage(st + 1 < nst ? st + 1 : 0);
+            const int sb = gstage % NBUF;
+            // this stage has landed for every wave and the buffer two stages ahead is free; the j
+            // sweep repeats every round, so the stages fetched ahead simply cycle
+            barrier_keep_loads<LW>();
+            if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads below
+            int st2 = st + 2;
+            if (st2 >= nst) st2 -= nst;
+            if (st2 >= nst) st2 = 0;
+            issue_stage(st2, (gstage + 2) % NBUF);
+            const E* sK1 = sStage + (sb * 4 + 0) * TILE;
+            const E* sU = sStage + (sb * 4 + 1) * TILE;
+            const E* sK1T = sStage + (sb * 4 + 2) * TILE;
+            const E* sUT = sStage + (sb * 4 + 3) * TILE;
+            if (k_active) {
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int jb = st * 64 + half * 32;
-                if (jb > jmax) break;  // wave-uniform: nothing at or below the causal bound
-                f32x16 s, dp;
+                for (int half = 0; half < 2; ++half) {
+                    const int jb = st * 64 + half * 32;
+                    if (jb > jend) break;
+                    f32x16 s, dp;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    s[i] = 0.f;
-                    dp[i] = 0.f;
-                }
-                const int rowoff = (sb * 64 + half * 32 + krow_off) * LDK + g * 8;
-                // the extra k-step subtracts LSE2[q] from S and Delta[q] from dP inside the MFMA
-                s = M::mma(ones, off_lse, s);
+                    for (int i = 0; i < 16; ++i) {
+                        s[i] = 0.f;
+                        dp[i] = 0.f;
+                    }
+                    const int rowoff = (half * 32 + krow_off) * 64;
+                    // the extra k-step subtracts LSE2[q] from S and Delta[q] from dP inside the MFMA
+                    s = M::mma(ones, off_lse, s);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const v8 ka = *reinterpret_cast<const v8*>(sK1 + rowoff + ks * 16);
-                    s = M::mma(ka, bq[ks], s);
-                }
-                dp = M::mma(ones, off_delta, dp);
+                    for (int ks = 0; ks < KS; ++ks)
+                        s = M::mma(*reinterpret_cast<const v8*>(sK1 + rowoff + (((ks * 2 + g) ^ fperm) * 8)), bq[ks], s);
+                    dp = M::mma(ones, off_delta, dp);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const v8 ua = *reinterpret_cast<const v8*>(sU + rowoff + ks * 16);
-                    dp = M::mma(ua, bg[ks], dp);
-                }
-                v8 pa[2], da[2];
-                // P = exp2(S - LSE2), dS = P (dP - Delta), both packed as A operands of the next
-                // products.  The masked variant is a separate (wave-uniform) branch so that interior
-                // steps carry no predication at all.
-                auto softmax_grad = [&](auto masked_tag) {
-                    constexpr bool MASKED = decltype(masked_tag)::value;
+                    for (int ks = 0; ks < KS; ++ks)
+                        dp = M::mma(*reinterpret_cast<const v8*>(sU + rowoff + (((ks * 2 + g) ^ fperm) * 8)), bg[ks], dp);
+                    v8 pa[2], da[2];
+                    // P = exp2(S - LSE2), dS = P (dP - Delta), packed as A operands of the next products.
+                    // The masked variant is a separate (wave-uniform) branch: interior steps carry no
+                    // predication.
+                    auto softmax_grad = [&](auto masked_tag) {
+                        constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) {
+                        for (int h = 0; h < 2; ++h) {
 #pragma unroll
-                        for (int e = 0; e < 8; e += 2) {
-                            const int i = h * 8 + e;
-                            float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
-                            if constexpr (MASKED) {
-                                p0 = (jb + key_of(g, i) <= jmax) ? p0 : 0.f;
-                                p1 = (jb + key_of(g, i + 1) <= jmax) ? p1 : 0.f;
+                            for (int e = 0; e < 8; e += 2) {
+                                const int i = h * 8 + e;
+                                float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
+                                if constexpr (MASKED) {
+                                    p0 = (kv_ok && jb + key_of(g, i) <= jq) ? p0 : 0.f;
+                                    p1 = (kv_ok && jb + key_of(g, i + 1) <= jq) ? p1 : 0.f;
+                                }
+                                const v2 pp = M::pack(p0, p1);
+                                const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
+                                pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
+                                da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                             }
-                            const v2 pp = M::pack(p0, p1);
-                            const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
-                            pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
-                            da[h][e] = dd[0]; da[h][e + 1] = dd[1];
+                        }
+                    };
+                    if (__builtin_amdgcn_readfirstlane(k_diag || (p.causal && jb + 31 > q0) || jb + 31 > T - 1))
+                        softmax_grad(std::true_type{});
+                    else
+                        softmax_grad(std::false_type{});
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int toff = (dt * 32 + n) * 64 + (((half * 4 + h * 2 + g) ^ fseq) * 8);
+                            accT[dt] = M::mma(pa[h], *reinterpret_cast<const v8*>(sUT + toff), accT[dt]);
+                            accQ[dt] = M::mma(da[h], *reinterpret_cast<const v8*>(sK1T + toff), accQ[dt]);
                         }
                     }
-                };
-                if (__builtin_amdgcn_readfirstlane(jb + 31 > jmax))
-                    softmax_grad(std::true_type{});
-                else
-                    softmax_grad(std::false_type{});
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        const int toff = (sb * D + dt * 32 + n) * LDU + half * 32 + h * 16 + g * 8;
-                        const v8 ub = *reinterpret_cast<const v8*>(sUT + toff);
-                        const v8 kb1 = *reinterpret_cast<const v8*>(sK1T + toff);
-                        accT[dt] = M::mma(pa[h], ub, accT[dt]);
-                        accQ[dt] = M::mma(da[h], kb1, accQ[dt]);
-                    }
                 }
             }
-            if (more) commit_stage(sb ^ 1);
-            __syncthreads();
         }
 
-        // ---- k-tile epilogue ------------------------------------------------------------------
+        // ---- round epilogue (rows of the accumulators = the 32 queries, column = d) ---------------
+        if (k_active) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const int d = dt * 32 + n;
-            const float qd = (float)sQ[wave * LDK + d] * p.alpha;
-            const float dod = (float)sDO[wave * LDK + d];
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = dt * 32 + n;
+                const float kd = (float)sKr[(mb * 8 + wave) * D + d];
+                float sk = 0.f, sv = 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int r = c_row(g, i);
-                const int k = kt * 32 + r;
-                if (q_ok && k <= jmax) {
-                    dqpart[dt] += accQ[dt][i] * (float)sK2[(kb * 32 + r) * LDK + d];
-                    unsafeAtomicAdd(p.dk2acc + base + (size_t)k * D + d, accQ[dt][i] * qd);
-                    unsafeAtomicAdd(p.dv2acc + base + (size_t)k * D + d, accT[dt][i] * dod);
+                for (int i = 0; i < 16; ++i) {
+                    const int r = c_row(g, i);
+                    dQacc[dt][i] += accQ[dt][i] * kd;
+                    sk += accQ[dt][i] * sQf[r * LDF + d];
+                    sv += accT[dt][i] * sOf[r * LDF + d];
+                }
+                sk += __shfl_xor(sk, 32, 64);
+                sv += __shfl_xor(sv, 32, 64);
+                if (g == 0) {
+                    unsafeAtomicAdd(p.dk2acc + base + (size_t)k * D + d, sk);
+                    unsafeAtomicAdd(p.dv2acc + base + (size_t)k * D + d, sv);
                 }
             }
         }
-        if (kt + 1 < nkt) commit_ktile(kb ^ 1);
-        __syncthreads();
+        // all waves are done with this round's K2/V2 rows and with the last stage
+        barrier_keep_loads<LW>();
     }
+    wait_vmcnt<0>();  // the stages fetched ahead land in the buffers reused below
+    __syncthreads();
 
+    // ---- dQ: sum the eight waves' partial tiles through LDS (the stage buffers are free now) ------
+    float* red = reinterpret_cast<float*>(smem);  // [8][32][LDF]
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        const float v = (dqpart[dt] + __shfl_xor(dqpart[dt], 32, 64)) * p.alpha;
-        if (q_ok && g == 0) p.dq[base + (size_t)q * D + dt * 32 + n] = (E)v;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) red[(wave * 32 + c_row(g, i)) * LDF + dt * 32 + n] = dQacc[dt][i];
+    __syncthreads();
+    for (int idx = tid; idx < BQ * D; idx += 512) {
+        const int r = idx / D, d = idx % D;
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) v += red[(w * 32 + r) * LDF + d];
+        if (q0 + r < T) p.dq[base + (size_t)(q0 + r) * D + d] = (E)(v * p.alpha);
     }
 }
 
@@ -646,7 +657,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.dq = (E*)a.dq;
     p.dk2acc = (float*)(ws + l.dk2acc); p.dv2acc = (float*)(ws + l.dv2acc);
     p.dk1part = (float*)(ws + l.dk1part); p.dupart = (float*)(ws + l.dupart);
-    p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 7) / 8; p.nqc = kNqc;
+    p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32; p.nqc = kNqc;
     p.alpha = a.alpha; p.causal = a.causal;
 
     hipLaunchKernelGGL(bwd_prep_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (const E*)a.k1,
@@ -654,8 +665,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
                        (E*)(ws + l.ut), (E*)(ws + l.k1t), (E*)(ws + l.k2t), (E*)(ws + l.v2t),
                        (float*)(ws + l.delta), p.dk2acc, p.dv2acc, a.T, Tp, D);
 
-    constexpr size_t smem = 2 * (size_t)(2 * 2 * 64 * (D + 8) + 2 * 2 * D * 72 + 2 * 2 * 32 * (D + 8) + 2 * 8 * (D + 8)) +
-                            2 * 32 * (D + 4) * 4;
+    constexpr size_t smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8)) + 4 * (size_t)(2 * 32 * (D + 4));
+    static_assert(smem >= 4 * 8 * 32 * (D + 4), "dQ reduction reuses the stage buffers");
     auto kern = tdp_bwd_qk_kernel<E, D>;
     static bool attr_set = false;
     if (!attr_set) {
