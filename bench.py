@@ -80,8 +80,9 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["both", "fwd"], default="both",
-                    help="fwd: time only the forward (for profiling runs); the JSON line then reports the forward")
+    ap.add_argument("--mode", choices=["both", "fwd", "copy"], default="both",
+                    help="fwd: time only the forward (for profiling runs); copy: a plain 256 MiB device copy, "
+                         "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     ap.add_argument("--B", type=int, default=4)
     ap.add_argument("--H", type=int, default=8)
     ap.add_argument("--T", type=int, default=1024)
@@ -100,6 +101,14 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     _lib.lib()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
+    if args.mode == "copy":
+        nbytes = 256 << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        ms = time_events(lambda: dst.copy_(src), args.steps, args.warmup, torch)
+        print(json.dumps({"metric": "device copy", "bytes_read": nbytes, "bytes_written": nbytes,
+                          "ms_per_step": ms, "value": 2 * nbytes / ms / 1e6, "unit": "GB/s"}), flush=True)
+        return
     B, H, T, D = args.B, args.H, args.T, args.D
     alpha = 1 / math.sqrt(D)
     q, k1, k2, v1, v2, do = (t.to(dev) for t in orc.make_inputs(B, H, T, D, torch.bfloat16, seed=0))

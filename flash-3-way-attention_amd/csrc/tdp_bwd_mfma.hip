@@ -58,7 +58,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_qk_kernel(BwdParams<E> p) {
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][4 tensors: K1, U, K1^T, U^T][TILE]
     E* sKr = sStage + NBUF * 4 * TILE;       // [2][8][D]  K2 rows of a round (one per wave), dense
     E* sVr = sKr + 2 * 8 * D;                // [2][8][D]  V2 rows
-    E* sQb = sVr + 2 * 8 * LDK;            // [BQ][LDK]    Q tile (operand build)
+    E* sQb = sVr + 2 * 8 * D;                // [BQ][LDK]  Q tile (operand build)
     E* sOb = sQb + BQ * LDK;               // [BQ][LDK]    dO tile
     float* sQf = reinterpret_cast<float*>(sOb + BQ * LDK);  // [BQ][LDF]  alpha * Q, fp32 (epilogue)
     float* sOf = sQf + BQ * LDF;                            // [BQ][LDF]  dO, fp32
@@ -333,13 +333,15 @@ __global__ __launch_bounds__(512) void tdp_bwd_j_kernel(BwdParams<E> p) {
     E* sOr = sQr + 2 * D;                  // [2][D]  dO[q]
     float* sMeta = reinterpret_cast<float*>(sOr + 2 * D);  // [2][2]  LSE2[q], Delta[q]
 
-    const int njb = (p.T + JB - 1) / JB;
-    int bid = blockIdx.x;
-    // heaviest first: low j blocks see the most queries
-    const int chunk = bid % p.nqc; bid /= p.nqc;
-    const int bh = bid % p.BH;
-    const int jb = bid / p.BH;
-    (void)njb;
+    // XCD-aware, heaviest-first block order: consecutive block ids go to different XCDs, so each
+    // XCD keeps its own heads (their K2/V2 streams stay in that XCD's L2); low j blocks (which see
+    // the most queries) are handed out first
+    const int groups = (p.BH + 7) / 8;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int bh = (slot % groups) * 8 + xcd;
+    const int rest = slot / groups;
+    const int chunk = rest % p.nqc, jb = rest / p.nqc;
+    if (bh >= p.BH) return;
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
@@ -688,7 +690,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         if (e != hipSuccess) return e;
         attr_j = true;
     }
-    hipLaunchKernelGGL(kern_j, dim3(a.BH * njb * kNqc), dim3(512), smem_j, st, p);
+    hipLaunchKernelGGL(kern_j, dim3(8 * groups * njb * kNqc), dim3(512), smem_j, st, p);
 
     const size_t n = (size_t)a.BH * a.T * D;
     size_t gridf = (n + 255) / 256;
