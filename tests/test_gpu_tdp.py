@@ -92,17 +92,16 @@ def test_lse_matches_oracle():
 
 
 def test_reproducible():
-    """Forward, dQ, dK1 and dV1 have a single owner per element and a fixed summation order:
-    bitwise equal from run to run.  dK2/dV2 of the MFMA path are summed with fp32 atomics over
-    query groups, so they are only reproducible to rounding; the fp32 VALU path is bitwise
-    reproducible throughout."""
+    """Forward and dQ have a single owner per element and a fixed summation order: bitwise equal
+    from run to run.  dK1/dV1/dK2/dV2 of the MFMA path are summed over query tiles with fp32
+    atomics, so they are only reproducible to rounding; the fp32 VALU path is bitwise reproducible
+    throughout."""
     inputs = orc.make_inputs(1, 2, 96, 64, torch.bfloat16, seed=5)
     a = util.run_tdp(inputs, 1 / 8, True)
     b = util.run_tdp(inputs, 1 / 8, True)
     assert torch.equal(a[0], b[0])
-    for i in (0, 1, 3):
-        assert torch.equal(a[1][i], b[1][i]), util.NAMES[i]
-    for i in (2, 4):
+    assert torch.equal(a[1][0], b[1][0]), "dq"
+    for i in (1, 2, 3, 4):
         util.assert_close(util.NAMES[i], a[1][i], b[1][i], rtol=1e-2, atol=1e-2)
     c = util.run_tdp(inputs, 1 / 8, True, flags=1)
     d = util.run_tdp(inputs, 1 / 8, True, flags=1)
