@@ -24,6 +24,10 @@ for _p in (ROOT, os.path.join(ROOT, "flash-3-way-attention_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# scaled by a plain 256 MiB copy (see the summaries under profiles/); not measured live
+TRAFFIC_FWD = 67.9e6        # 34.5 MiB fetched + 30.3 MiB written
+TRAFFIC_BWD_ROWS = 2.748e9   # average of the two launches (the WITH_DQ one re-fetches spilled registers)
 
 
 def triples(B, H, T, causal=True):
@@ -180,12 +184,17 @@ def main():
         "fwd_hbm_gbs": bytes_fwd / ms_fwd / 1e6, "bwd_hbm_gbs": bytes_bwd / ms_bwd / 1e6,
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "clock_mhz": getattr(props, "clock_rate", 0) / 1e3},
-        "roofline": {"bound": "mfma", "kernel": "tdp_fwd_mfma_kernel<bf16,64,2>", "achieved": fwd_tf,
-                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": fwd_tf / PEAK_BF16_TFLOPS,
-                     "traffic": None, "flops_per_launch": f_fwd, "ms_per_launch": ms_fwd},
-        "roofline_bwd": {"bound": "mfma", "kernel": "triple-dot backward (all launches)", "achieved": bwd_tf,
-                         "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": bwd_tf / PEAK_BF16_TFLOPS,
-                         "traffic": None, "flops_per_launch": f_bwd, "ms_per_launch": ms_bwd},
+        # dominant kernel by time: tdp_bwd_rows_kernel, launched twice per backward (dQ,dK2,dV2 then
+        # dK1,dU).  Each launch is credited half of the backward's algorithmic flops (6*D*N) and
+        # half of the event-timed backward (the prep/finish kernels in that time are < 1 %).
+        "roofline": {"bound": "mfma", "kernel": "tdp_bwd_rows_kernel<bf16,64> (avg of its 2 launches)",
+                     "achieved": bwd_tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": bwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BWD_ROWS,
+                     "flops_per_launch": f_bwd // 2, "ms_per_launch": ms_bwd / 2},
+        "roofline_fwd": {"bound": "mfma", "kernel": "tdp_fwd_mfma_kernel<bf16,64,NT=1,16 waves>",
+                         "achieved": fwd_tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": fwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_FWD,
+                         "flops_per_launch": f_fwd, "ms_per_launch": ms_fwd},
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(T, D, alpha)
