@@ -5,8 +5,9 @@ A step = one triple-dot-product forward + backward over one synthetic batch at
 B=4 H=8 T=1024 D=64 bf16 causal (inputs resident in HBM before the timed
 region).  Prints ONE JSON line.  `value` is the algorithmic TFLOP/s of the
 whole step: 16*D*N / time with N = B*H*T(T+1)(2T+1)/6 valid (q,j,k) triples
-(forward 4*D*N, backward 12*D*N).  `roofline` covers the forward MFMA kernel,
-`roofline_bwd` the backward; both divide by the MI355X dense bf16 MFMA peak.
+(forward 4*D*N, backward 12*D*N).  `roofline` covers the dominant kernel (the backward rows
+kernel, launched twice per step), `roofline_fwd` the forward kernel; both divide by the
+MI355X dense bf16 MFMA peak.
 `cpu_baseline` times the CPU oracle (the reference's naive dense formulation)
 on a bounded sample on this box's host cores.
 """

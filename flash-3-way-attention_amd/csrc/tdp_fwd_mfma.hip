@@ -7,17 +7,19 @@
 // accumulator  Tv[(q,k), :] = sum_j P U[j, :]   (U = SiLU(V1)).  The rows of one query are
 // merged once per k-tile:  O[q] = sum_k w_k * V2[k] (.) Tv[(q,k)],  w_k = exp2(m_qk - M_q).
 //
-// Work decomposition.  One workgroup = 8 waves = BQ = 8*NT queries of one (batch, head).
-// A wave owns NT queries; a 32x32 MFMA tile is 32 consecutive k (columns) of ONE query, so the
-// causal bound j <= q is uniform over a tile and the k-merge stays inside the wave.
-// Outer loop: k-tiles of 32.  Inner loop: 64-row stages of K1 and U^T, staged through LDS and
-// shared by all 8 waves (double buffered, one barrier per stage).
+// Work decomposition.  One workgroup = WAVES waves = BQ = WAVES*NT queries of one (batch, head)
+// (D=64: 16 waves x 1 query at 4 waves per SIMD; D=128: 8 waves x 1 query).  A wave owns NT
+// queries; a 32x32 MFMA tile is 32 consecutive k (columns) of ONE query, so the causal bound
+// j <= q is uniform over a tile and the k-merge stays inside the wave.
+// Outer loop: k-tiles of 32.  Inner loop: JS-row stages of K1 and U^T, staged through LDS and
+// shared by all waves (double buffered, one barrier per stage).
 //
-// Per 32-key step and tile:  S^T = K1 * QK2^T  (rows = j, cols = virtual rows), accumulated on
-// top of C = -m (the running reference maximum), so the MFMA result is already s - m.  The
-// reference maximum is only raised when some score exceeds it by more than 2^8 ("lazy" max),
-// which keeps max/rescale work off the common path.  P = exp2(S) is packed to 16 bit in the
-// registers it already occupies and fed straight back as the A operand of Tv += P * U.
+// Per 32-key step and tile:  S^T = K1 * QK2^T  (rows = j, cols = virtual rows).  The common
+// (FAST) sweep takes P = exp2(S) with no reference maximum at all and only records whether
+// some row left the safe exponent range; if one did, the workgroup repeats that k-tile with the
+// CAREFUL sweep: online softmax whose reference maximum is raised only when a score exceeds it
+// by more than 2^8 ("lazy" max).  P is packed to 16 bit in the registers it already occupies
+// and fed straight back as the A operand of Tv += P * U.
 #include <stdlib.h>
 #include <string.h>
 

@@ -61,7 +61,9 @@ const char* tritt_status_string(int status);
  *   applies SiLU to V1 itself and writes the final lse (the reference's M + log L).
  * tritt_tdp_bwd replaces FlashTrittention.backward and its five launches
  *   (triple_dot_product/flash_trittention.py:141-393, kernels/bwd_{dq,dk1,dk2,dv1,dv2}.py),
- *   including Delta = rowsum(dO*O) and the SiLU' factor on dV1.
+ *   including Delta = rowsum(dO*O) and the SiLU' factor on dV1.  On the 16-bit MFMA path
+ *   (D = 64, full windows) dK1/dV1/dK2/dV2 are accumulated with fp32 atomics: equal to rounding
+ *   from run to run, not bitwise; dQ and every fp32-tensor result are bitwise reproducible.
  */
 size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
                                      int k1_window, int k2_window, int kk_left, int kk_right,

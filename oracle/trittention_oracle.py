@@ -33,8 +33,11 @@ T=1 closed form, Q=0 prefix-mean product, K2=1 reduction to
 finite differences, and for dot-product-sum the dense-vs-factorised identity
 and the K1=0 reduction to biased SDPA.  The windowed-mask conventions
 (``kk_left``/``kk_right``/``k1_window``/``k2_window``/``k_diff``) are pinned by
-the committed fixture ``tests/golden/windowed_masks.npz`` when present;
-without it they are "parity unpinned" at the value level.
+the committed fixture ``tests/golden/windowed_masks.npz``: outputs and all five
+input gradients of the reference's own naive modules (float64, tiny shapes,
+seven window settings for triple-dot and four ``k_diff`` values for
+dot-product-sum), written by ``tests/golden/make_reference_vectors.py`` and
+checked in ``tests/test_golden.py``.
 """
 
 from __future__ import annotations
