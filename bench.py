@@ -85,9 +85,11 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["both", "fwd", "copy"], default="both",
+    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "dps"], default="both",
                     help="fwd: time only the forward (for profiling runs); copy: a plain 256 MiB device copy, "
-                         "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
+                         "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against; "
+                         "sweep: triple-dot forward at B=1 H=16 D=128 bf16 over T in 512..4096; "
+                         "dps: dot-product-sum forward+backward at --B --H --T --D")
     ap.add_argument("--B", type=int, default=4)
     ap.add_argument("--H", type=int, default=8)
     ap.add_argument("--T", type=int, default=1024)
@@ -116,6 +118,50 @@ def main():
         return
     B, H, T, D = args.B, args.H, args.T, args.D
     alpha = 1 / math.sqrt(D)
+    if args.mode == "sweep":
+        rows = []
+        for Ts in (512, 1024, 2048, 4096):
+            ins = [t.to(dev) for t in orc.make_inputs(1, 16, Ts, 128, torch.bfloat16, seed=0, n=5)]
+            torch.cuda.reset_peak_memory_stats()
+            base_mem = torch.cuda.memory_allocated()
+
+            def f():
+                with torch.no_grad():
+                    return flash_trittention(*ins, softmax_scale=1 / math.sqrt(128), k1_window=None, k2_window=None,
+                                             kk_left=None, kk_right=None, causal=True)
+
+            ms = time_events(f, max(2, min(args.steps, 32768 // Ts)), 1, torch)
+            fl = 4 * 128 * triples(1, 16, Ts)
+            rows.append({"T": Ts, "ms": ms, "tflops": fl / ms / 1e9, "frac_of_bf16_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS,
+                         "extra_device_bytes": torch.cuda.max_memory_allocated() - base_mem,
+                         "one_tensor_bytes": 16 * Ts * 128 * 2})
+        print(json.dumps({"metric": "triple-dot trittention fwd TFLOP/s vs T", "unit": "TFLOP/s",
+                          "config": {"workload": "triple-dot fwd B=1 H=16 D=128 bf16 causal"}, "rows": rows}), flush=True)
+        return
+    if args.mode == "dps":
+        from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
+
+        ins = [t.to(dev) for t in orc.make_inputs(B, H, T, D, torch.bfloat16, seed=0)]
+        lv = [t.clone().requires_grad_(True) for t in ins[:5]]
+        mod = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=T)
+        hold = {}
+
+        def f():
+            hold["o"] = mod(*lv)[0]
+
+        def b():
+            hold["o"].backward(ins[5], retain_graph=True)
+
+        ms_f = time_events(f, args.steps, max(args.warmup, 3), torch)
+        ms_b = time_events(b, args.steps, max(args.warmup, 3), torch)  # the first backward pays one-time set-up
+        n3 = B * H * T * (T + 1) * (T + 2) // 6   # valid (q,s,t) triples of the reference's formulation
+        n2 = B * H * T * (T + 1) // 2              # (row, column) pairs of the factorised one
+        print(json.dumps({"metric": "dot-product-sum trittention fwd / bwd ms", "unit": "ms", "fwd_ms": ms_f, "bwd_ms": ms_b,
+                          "executed_fwd_tflops": 8 * D * n2 / ms_f / 1e9, "executed_bwd_tflops": 20 * D * n2 / ms_b / 1e9,
+                          "reference_formulation_fwd_tflops_equiv": 4 * D * n3 / ms_f / 1e9,
+                          "io_gbs_fwd": (6 * B * H * T * D * 2) / ms_f / 1e6,
+                          "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} bf16 causal"}}), flush=True)
+        return
     q, k1, k2, v1, v2, do = (t.to(dev) for t in orc.make_inputs(B, H, T, D, torch.bfloat16, seed=0))
     leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
     kw = dict(softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True)

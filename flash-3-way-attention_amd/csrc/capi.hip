@@ -263,6 +263,11 @@ bool use_mfma_bwd(int T, int D, int dtype, int causal, int w1, int w2, int kl, i
     return mfma_tdp_bwd_supported(D, dtype != TRITT_F32) && full_windows(T, causal, w1, w2, kl, kr);
 }
 
+bool use_mfma_dps(int D, int dtype, unsigned flags) {
+    if (flags & TRITT_FLAG_FORCE_GENERIC) return false;
+    return mfma_dps_supported(D, dtype != TRITT_F32);
+}
+
 bool any_null(std::initializer_list<const void*> ps) {
     for (const void* p : ps)
         if (!p) return true;
@@ -367,6 +372,7 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
 
 size_t tritt_dps_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (use_mfma_dps(D, dtype, flags)) return mfma_dps_fwd_workspace(B * H, T, D);
     Arena ar(nullptr);
     dps_fwd_impl(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f, 1, T,
                  nullptr);
@@ -381,8 +387,17 @@ int tritt_dps_fwd(const void* q, const void* k1, const void* k2, const void* v1,
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
     if (causal && k_diff < 0) return TRITT_ERR_INVALID;
+    const bool mfma = use_mfma_dps(D, dtype, flags);
+    if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;
     const size_t need = tritt_dps_fwd_workspace_bytes(B, H, T, D, dtype, flags);
     if (!workspace || workspace_bytes < need) return TRITT_ERR_WORKSPACE;
+    if (mfma) {
+        MfmaDpsArgs a{};
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o_out = o; a.lse_out = lse; a.workspace = workspace;
+        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0; a.k_diff = clampw(k_diff, T);
+        a.is_bf16 = dtype == TRITT_BF16;
+        return (int)mfma_dps_fwd(a, (hipStream_t)stream);
+    }
     Arena ar(workspace);
     return dps_fwd_impl(ar, true, q, k1, k2, v1, v2, o, lse, B, H, T, D, dtype, alpha, causal, clampw(k_diff, T),
                         (hipStream_t)stream);
@@ -390,6 +405,7 @@ int tritt_dps_fwd(const void* q, const void* k1, const void* k2, const void* v1,
 
 size_t tritt_dps_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (use_mfma_dps(D, dtype, flags)) return mfma_dps_bwd_workspace(B * H, T, D);
     Arena ar(nullptr);
     dps_bwd_impl(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                  nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f, 1, T, nullptr);
@@ -405,8 +421,18 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
     if (causal && k_diff < 0) return TRITT_ERR_INVALID;
+    const bool mfma = use_mfma_dps(D, dtype, flags);
+    if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;
     const size_t need = tritt_dps_bwd_workspace_bytes(B, H, T, D, dtype, flags);
     if (!workspace || workspace_bytes < need) return TRITT_ERR_WORKSPACE;
+    if (mfma) {
+        MfmaDpsArgs a{};
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.d_o = d_o; a.lse_in = lse;
+        a.dq = dq; a.dk1 = dk1; a.dk2 = dk2; a.dv1 = dv1; a.dv2 = dv2; a.workspace = workspace;
+        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0; a.k_diff = clampw(k_diff, T);
+        a.is_bf16 = dtype == TRITT_BF16;
+        return (int)mfma_dps_bwd(a, (hipStream_t)stream);
+    }
     Arena ar(workspace);
     return dps_bwd_impl(ar, true, q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2, B, H, T, D, dtype, alpha,
                         causal, clampw(k_diff, T), (hipStream_t)stream);

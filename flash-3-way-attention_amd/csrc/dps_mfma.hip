@@ -1,0 +1,751 @@
+// Dot-product-sum trittention on MFMA (gfx950) for 16-bit tensors, D = 64 or 128.
+//
+// The score separates,  exp(alpha (Q_q.K2_t + K1_s.K2_t)) = exp(alpha Q_q.K2_t) exp(alpha K1_s.K2_t),
+// and the mask (s <= t <= q, t - s <= k_diff) never couples s with q, so the op is two chained
+// banded attentions (O(T^2 D) instead of O(T^3 D)):
+//   inner:  lse1[t] = logsumexp_s alpha K1_s.K2_t,  R[t] = softmax_s(.) @ U,  W[t] = R[t] * V2[t]
+//   outer:  O[q] = softmax_t(alpha Q_q.K2_t + lse1[t]) @ W,  LSE[q] = logsumexp_t(.)
+// and the backward is the two attention backwards chained through (dR, dlse1).
+//
+// Three kernels, each a generic "attention with a per-key bias" building block on 32x32x16 MFMA:
+//   attn_fwd_mfma_kernel       owner = 32 query-like rows;  out, out*mul, (out*mul)^T, lse
+//   attn_bwd_row_mfma_kernel   owner = 32 query-like rows;  dX
+//   attn_bwd_col_mfma_kernel   owner = 32 key-like rows;    dK, dV, dbias (+ the element-wise link
+//                              between the two passes when it runs the outer pass)
+// A workgroup is 4 waves that share one owner tile and split the streamed 32-row tiles between
+// them round-robin (their partial results meet in LDS), so T = 1024 already gives 4096 waves.
+// Every tile is computed transposed where needed so that the owner index sits on the MFMA column
+// (= lane) axis: softmax statistics, LSE and Delta stay lane-local, and with the permuted row order
+// of mfma.hpp the probabilities leave one MFMA in exactly the operand layout of the next.
+// Operands are read straight from global memory in MFMA layout (16 B per lane); contraction over
+// a row index reads the [D][Tp] transposed copies that the prep kernel / the producing epilogue
+// writes.  Every output element has one owner: no atomics, bitwise reproducible.
+#include "kernels.hpp"
+#include "mfma.hpp"
+
+namespace tritt {
+namespace {
+
+constexpr int kW = 4;     // waves per workgroup
+constexpr int kLdr = 33;  // LDS row stride (floats) of the cross-wave reduction tiles
+
+template <typename E>
+__device__ __forceinline__ typename Mma<E>::v8 ld8(const E* p) {
+    return *reinterpret_cast<const typename Mma<E>::v8*>(p);
+}
+
+// 16 fp32 values of one lane (registers of a C tile) -> the two 8-wide 16-bit operands they form
+template <typename E>
+__device__ __forceinline__ void pack16(const float (&x)[16], typename Mma<E>::v8 (&out)[2]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            const typename Mma<E>::v2 t = Mma<E>::pack(x[8 * h + e], x[8 * h + e + 1]);
+            out[h][e] = t[0];
+            out[h][e + 1] = t[1];
+        }
+}
+
+// pair (query-like row r, key-like row a) takes part
+__device__ __forceinline__ bool pair_ok(int T, int causal, int k_diff, int r, int a) {
+    return (r < T) & (a < T) & ((!causal) | ((a <= r) & (r - a <= k_diff)));
+}
+
+template <int D>
+__device__ __forceinline__ void spill_tiles(float* sO, int wave, const f32x16 (&acc)[D / 32], int n, int g) {
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sO[(wave * D + 32 * dt + c_row(g, i)) * kLdr + n] = acc[dt][i];
+}
+
+// ------------------------------------------------------------------------------------ forward
+template <typename E>
+struct AttnFwdP {
+    const E* x;         // [BH][T][D]   query-like rows
+    const E* k;         // [BH][T][D]   key-like rows
+    const E* vt;        // [BH][D][Tp]  values, transposed, zero padded
+    const float* bias;  // [BH][Tp] per-key bias in log2 units, or null
+    const E* mul;       // [BH][T][D] or null
+    E* out;             // [BH][T][D] or null
+    float* out_f32;     // [BH][T][D] or null
+    E* outm;            // out * mul, [BH][T][D] or null
+    E* outm_t;          // out * mul, [BH][D][Tp] or null
+    float* lse;         // [BH][lse_stride]
+    int lse_stride;
+    float lse_scale;    // lse = lse_scale * log2-sum-exp2
+    int T, Tp;
+    float scale_log2;
+    int causal, k_diff;
+};
+
+template <typename E, int D>
+__global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
+    using M = Mma<E>;
+    using v8 = typename M::v8;
+    constexpr int KS = D / 16, DT = D / 32;
+    extern __shared__ __align__(16) char smem_raw[];
+    float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
+    float* sM = sO + kW * D * kLdr;                  // [kW][32]
+    float* sL = sM + kW * 32;                        // [kW][32]
+
+    const int bh = blockIdx.y, r0 = (gridDim.x - 1 - blockIdx.x) * 32;  // longest rows first
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int T = p.T, Tp = p.Tp;
+    const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
+    const E* __restrict__ X = p.x + base;
+    const E* __restrict__ K = p.k + base;
+    const E* __restrict__ VT = p.vt + tb;
+    const float* __restrict__ bias = p.bias ? p.bias + vb : nullptr;
+    const int r = r0 + n;
+
+    v8 xb[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) xb[ks] = ld8<E>(X + (size_t)min(r, T - 1) * D + 16 * ks + 8 * g);
+
+    const int a_lo = p.causal ? max(0, r0 - p.k_diff) : 0;
+    const int a_hi = p.causal ? min(T - 1, r0 + 31) : T - 1;
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    for (int t = a_lo / 32 + wave; t <= a_hi / 32; t += kW) {
+        const int a0 = t * 32;
+        f32x16 s;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = 0.f;
+        const E* krow = K + (size_t)min(a0 + key_of_row(n), T - 1) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = M::mma(ld8<E>(krow + 16 * ks), xb[ks], s);
+        float b[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) b[i] = 0.f;
+        if (bias) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const float4 v = *reinterpret_cast<const float4*>(bias + a0 + 16 * h + 8 * g + 4 * c);
+                    b[8 * h + 4 * c] = v.x; b[8 * h + 4 * c + 1] = v.y; b[8 * h + 4 * c + 2] = v.z; b[8 * h + 4 * c + 3] = v.w;
+                }
+        }
+        float sv[16], tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int a = a0 + key_of(g, i);
+            const bool ok = (a < T) & ((!p.causal) | ((a <= r) & (r - a <= p.k_diff)));
+            sv[i] = ok ? fmaf(s[i], p.scale_log2, b[i]) : -INFINITY;
+            tmax = fmaxf(tmax, sv[i]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m, tmax);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float f = fast_exp2(m - m_use);
+        m = m_new;
+        l *= f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[dt][i] *= f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            sv[i] = fast_exp2(sv[i] - m_use);
+            l += sv[i];
+        }
+        v8 pb[2];
+        pack16<E>(sv, pb);
+        // O^T[d][r] += V^T[d][a] P^T[a][r]
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+                acc[dt] = M::mma(ld8<E>(VT + (size_t)(32 * dt + n) * Tp + a0 + 16 * kk + 8 * g), pb[kk], acc[dt]);
+    }
+    l += __shfl_xor(l, 32, 64);
+
+    // merge the waves' partial softmaxes
+    if (g == 0) {
+        sM[wave * 32 + n] = m;
+        sL[wave * 32 + n] = l;
+    }
+    spill_tiles<D>(sO, wave, acc, n, g);
+    __syncthreads();
+    const int rr = tid & 31, dg = tid >> 5, row = r0 + rr;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kW; ++w) mm = fmaxf(mm, sM[w * 32 + rr]);
+    float e[kW], ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < kW; ++w) {
+        const float mw = sM[w * 32 + rr];
+        e[w] = mw == -INFINITY ? 0.f : fast_exp2(mw - mm);
+        ll += e[w] * sL[w * 32 + rr];
+    }
+    const float inv = 1.0f / ll;
+    if (dg == 0 && row < T) p.lse[(size_t)bh * p.lse_stride + row] = (mm + fast_log2(ll)) * p.lse_scale;
+#pragma unroll
+    for (int c = 0; c < D / 64; ++c) {
+        const int d0 = dg * (D / 8) + 8 * c;
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < kW; ++w) v += e[w] * sO[(w * D + d0 + j) * kLdr + rr];
+            o[j] = v * inv;
+        }
+        const size_t off = base + (size_t)row * D + d0;
+        if (row < T) {
+            if (p.out) {
+                v8 ov;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ov[j] = (E)o[j];
+                *reinterpret_cast<v8*>(p.out + off) = ov;
+            }
+            if (p.out_f32) {
+                *reinterpret_cast<float4*>(p.out_f32 + off) = make_float4(o[0], o[1], o[2], o[3]);
+                *reinterpret_cast<float4*>(p.out_f32 + off + 4) = make_float4(o[4], o[5], o[6], o[7]);
+            }
+        }
+        if (p.mul) {
+            v8 mv;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) mv[j] = (E)0.f;
+            if (row < T) mv = ld8<E>(p.mul + off);
+            v8 wv;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) wv[j] = (E)(row < T ? o[j] * (float)mv[j] : 0.f);
+            if (p.outm && row < T) *reinterpret_cast<v8*>(p.outm + off) = wv;
+            if (p.outm_t)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) p.outm_t[tb + (size_t)(d0 + j) * Tp + row] = wv[j];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------ backward, rows
+template <typename E>
+struct AttnBwdP {
+    const E *x, *g, *k, *v;  // [BH][T][D] row-major: query-like rows, their upstream gradient, keys, values
+    const E *kt;             // K^T [BH][D][Tp]   (row kernel)
+    const E *xt, *gt;        // X^T, G^T [BH][D][Tp]  (column kernel)
+    const float* bias;       // [BH][Tp] log2 units or null
+    const float* lse2;       // [BH][Tp] log2 units
+    const float* delta;      // [BH][Tp]
+    int T, Tp;
+    float alpha;
+    int causal, k_diff;
+    // row kernel output: dx = alpha * sum + addend
+    const float* addend;     // fp32 [BH][T][D] or null
+    E* dx;
+    // column kernel outputs
+    float* dk_f32;           // alpha * sum  (fp32) or null
+    E* dk;                   // alpha * sum  (16 bit) or null
+    // LINK == false: dv = sum * SiLU'(v1)
+    const E* v1;
+    E* dv;
+    // LINK == true: dW = sum;  dV2 = dW R;  dR = dW V2;  delta1 = rowsum(dR R) - dbias
+    const float* r_f32;
+    const E* v2;
+    E *dv2, *dr, *dr_t;
+    float* delta1;           // [BH][Tp]
+};
+
+template <typename E, int D>
+__global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> p) {
+    using M = Mma<E>;
+    using v8 = typename M::v8;
+    constexpr int KS = D / 16, DT = D / 32;
+    extern __shared__ __align__(16) char smem_raw[];
+    float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
+
+    const int bh = blockIdx.y, r0 = (gridDim.x - 1 - blockIdx.x) * 32;
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int T = p.T, Tp = p.Tp;
+    const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
+    const E* __restrict__ K = p.k + base;
+    const E* __restrict__ V = p.v + base;
+    const E* __restrict__ KT = p.kt + tb;
+    const float* __restrict__ bias = p.bias ? p.bias + vb : nullptr;
+    const int r = r0 + n, rc = min(r, T - 1);
+    const float scale_log2 = p.alpha * kLog2e;
+
+    v8 xb[KS], gb[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        xb[ks] = ld8<E>(p.x + base + (size_t)rc * D + 16 * ks + 8 * g);
+        gb[ks] = ld8<E>(p.g + base + (size_t)rc * D + 16 * ks + 8 * g);
+    }
+    const float lse2 = p.lse2[vb + rc], dl = p.delta[vb + rc];
+
+    const int a_lo = p.causal ? max(0, r0 - p.k_diff) : 0;
+    const int a_hi = p.causal ? min(T - 1, r0 + 31) : T - 1;
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
+
+    for (int t = a_lo / 32 + wave; t <= a_hi / 32; t += kW) {
+        const int a0 = t * 32;
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s[i] = 0.f;
+            dp[i] = 0.f;
+        }
+        const size_t ro = (size_t)min(a0 + key_of_row(n), T - 1) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = M::mma(ld8<E>(K + ro + 16 * ks), xb[ks], s);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dp = M::mma(ld8<E>(V + ro + 16 * ks), gb[ks], dp);
+        float b[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) b[i] = 0.f;
+        if (bias) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const float4 v = *reinterpret_cast<const float4*>(bias + a0 + 16 * h + 8 * g + 4 * c);
+                    b[8 * h + 4 * c] = v.x; b[8 * h + 4 * c + 1] = v.y; b[8 * h + 4 * c + 2] = v.z; b[8 * h + 4 * c + 3] = v.w;
+                }
+        }
+        float ds[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int a = a0 + key_of(g, i);
+            const bool ok = pair_ok(T, p.causal, p.k_diff, r, a);
+            const float pr = ok ? fast_exp2(fmaf(s[i], scale_log2, b[i] - lse2)) : 0.f;
+            ds[i] = pr * (dp[i] - dl);
+        }
+        v8 dsb[2];
+        pack16<E>(ds, dsb);
+        // dX^T[d][r] += K^T[d][a] dS^T[a][r]
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+                acc[dt] = M::mma(ld8<E>(KT + (size_t)(32 * dt + n) * Tp + a0 + 16 * kk + 8 * g), dsb[kk], acc[dt]);
+    }
+
+    spill_tiles<D>(sO, wave, acc, n, g);
+    __syncthreads();
+    const int rr = tid & 31, dg = tid >> 5, row = r0 + rr;
+    if (row >= T) return;
+#pragma unroll
+    for (int c = 0; c < D / 64; ++c) {
+        const int d0 = dg * (D / 8) + 8 * c;
+        const size_t off = base + (size_t)row * D + d0;
+        v8 ov;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < kW; ++w) v += sO[(w * D + d0 + j) * kLdr + rr];
+            v *= p.alpha;
+            if (p.addend) v += p.addend[off + j];
+            ov[j] = (E)v;
+        }
+        *reinterpret_cast<v8*>(p.dx + off) = ov;
+    }
+}
+
+// --------------------------------------------------------------------------- backward, columns
+template <typename E, int D, bool LINK>
+__global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> p) {
+    using M = Mma<E>;
+    using v8 = typename M::v8;
+    constexpr int KS = D / 16, DT = D / 32;
+    extern __shared__ __align__(16) char smem_raw[];
+    float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
+    float* sB = sO + kW * D * kLdr;                  // [kW][32]  dbias partials
+    float* sR = sB + kW * 32;                        // [8][32]   delta1 partials
+
+    const int bh = blockIdx.y, c0 = blockIdx.x * 32;  // lowest key rows are the longest
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int T = p.T, Tp = p.Tp;
+    const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
+    const E* __restrict__ X = p.x + base;
+    const E* __restrict__ G = p.g + base;
+    const E* __restrict__ XT = p.xt + tb;
+    const E* __restrict__ GT = p.gt + tb;
+    const float* __restrict__ lse2 = p.lse2 + vb;
+    const float* __restrict__ delta = p.delta + vb;
+    const int a = c0 + n, ac = min(a, T - 1);
+    const float scale_log2 = p.alpha * kLog2e;
+
+    v8 kb[KS], vbv[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        kb[ks] = ld8<E>(p.k + base + (size_t)ac * D + 16 * ks + 8 * g);
+        vbv[ks] = ld8<E>(p.v + base + (size_t)ac * D + 16 * ks + 8 * g);
+    }
+    const float ba = p.bias ? p.bias[vb + ac] : 0.f;
+
+    const int r_lo = p.causal ? c0 : 0;
+    const int r_hi = p.causal ? (int)min((long)T - 1, (long)c0 + 31 + p.k_diff) : T - 1;
+    f32x16 acck[DT], accv[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acck[dt][i] = 0.f;
+            accv[dt][i] = 0.f;
+        }
+    float db = 0.f;
+
+    for (int t = r_lo / 32 + wave; t <= r_hi / 32; t += kW) {
+        const int r0 = t * 32;
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s[i] = 0.f;
+            dp[i] = 0.f;
+        }
+        const size_t ro = (size_t)min(r0 + key_of_row(n), T - 1) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = M::mma(ld8<E>(X + ro + 16 * ks), kb[ks], s);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dp = M::mma(ld8<E>(G + ro + 16 * ks), vbv[ks], dp);
+        float ls[16], dl[16];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const float4 v = *reinterpret_cast<const float4*>(lse2 + r0 + 16 * h + 8 * g + 4 * c);
+                const float4 w = *reinterpret_cast<const float4*>(delta + r0 + 16 * h + 8 * g + 4 * c);
+                ls[8 * h + 4 * c] = v.x; ls[8 * h + 4 * c + 1] = v.y; ls[8 * h + 4 * c + 2] = v.z; ls[8 * h + 4 * c + 3] = v.w;
+                dl[8 * h + 4 * c] = w.x; dl[8 * h + 4 * c + 1] = w.y; dl[8 * h + 4 * c + 2] = w.z; dl[8 * h + 4 * c + 3] = w.w;
+            }
+        float pr[16], ds[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int r = r0 + key_of(g, i);
+            const bool ok = pair_ok(T, p.causal, p.k_diff, r, a);
+            pr[i] = ok ? fast_exp2(fmaf(s[i], scale_log2, ba - ls[i])) : 0.f;
+            ds[i] = ok ? pr[i] * (dp[i] - dl[i]) : 0.f;
+            db += ds[i];
+        }
+        v8 pb[2], dsb[2];
+        pack16<E>(pr, pb);
+        pack16<E>(ds, dsb);
+        // dK^T[d][a] += X^T[d][r] dS[r][a];  dV^T[d][a] += G^T[d][r] P[r][a]
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                const size_t to = (size_t)(32 * dt + n) * Tp + r0 + 16 * kk + 8 * g;
+                acck[dt] = M::mma(ld8<E>(XT + to), dsb[kk], acck[dt]);
+                accv[dt] = M::mma(ld8<E>(GT + to), pb[kk], accv[dt]);
+            }
+    }
+    db += __shfl_xor(db, 32, 64);
+
+    const int aa = tid & 31, dg = tid >> 5, row = c0 + aa;
+    // ---- dK
+    if (g == 0) sB[wave * 32 + n] = db;
+    spill_tiles<D>(sO, wave, acck, n, g);
+    __syncthreads();
+    if (row < T) {
+#pragma unroll
+        for (int c = 0; c < D / 64; ++c) {
+            const int d0 = dg * (D / 8) + 8 * c;
+            const size_t off = base + (size_t)row * D + d0;
+            float o[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float v = 0.f;
+#pragma unroll
+                for (int w = 0; w < kW; ++w) v += sO[(w * D + d0 + j) * kLdr + aa];
+                o[j] = v * p.alpha;
+            }
+            if (p.dk_f32) {
+                *reinterpret_cast<float4*>(p.dk_f32 + off) = make_float4(o[0], o[1], o[2], o[3]);
+                *reinterpret_cast<float4*>(p.dk_f32 + off + 4) = make_float4(o[4], o[5], o[6], o[7]);
+            }
+            if (p.dk) {
+                v8 ov;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ov[j] = (E)o[j];
+                *reinterpret_cast<v8*>(p.dk + off) = ov;
+            }
+        }
+    }
+    __syncthreads();
+    // ---- dV
+    spill_tiles<D>(sO, wave, accv, n, g);
+    __syncthreads();
+    float part = 0.f;
+#pragma unroll
+    for (int c = 0; c < D / 64; ++c) {
+        const int d0 = dg * (D / 8) + 8 * c;
+        const size_t off = base + (size_t)row * D + d0;
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < kW; ++w) v += sO[(w * D + d0 + j) * kLdr + aa];
+            o[j] = v;
+        }
+        if constexpr (!LINK) {
+            if (row < T) {
+                const v8 x = ld8<E>(p.v1 + off);
+                v8 ov;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ov[j] = (E)(o[j] * silu_grad_f((float)x[j]));
+                *reinterpret_cast<v8*>(p.dv + off) = ov;
+            }
+        } else {
+            v8 dv2, dr;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                dv2[j] = (E)0.f;
+                dr[j] = (E)0.f;
+            }
+            if (row < T) {
+                const v8 x = ld8<E>(p.v2 + off);
+                const float4 ra = *reinterpret_cast<const float4*>(p.r_f32 + off);
+                const float4 rb = *reinterpret_cast<const float4*>(p.r_f32 + off + 4);
+                const float rv[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float drj = o[j] * (float)x[j];
+                    dv2[j] = (E)(o[j] * rv[j]);
+                    dr[j] = (E)drj;
+                    part += drj * rv[j];
+                }
+                *reinterpret_cast<v8*>(p.dv2 + off) = dv2;
+                *reinterpret_cast<v8*>(p.dr + off) = dr;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) p.dr_t[tb + (size_t)(d0 + j) * Tp + row] = dr[j];
+        }
+    }
+    if constexpr (LINK) {
+        sR[dg * 32 + aa] = part;
+        __syncthreads();
+        if (tid < 32) {
+            float d1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) d1 += sR[j * 32 + tid];
+#pragma unroll
+            for (int w = 0; w < kW; ++w) d1 -= sB[w * 32 + tid];
+            p.delta1[vb + c0 + tid] = (c0 + tid < T) ? d1 : 0.f;
+        }
+    }
+}
+
+// --------------------------------------------------------------------------------------- prep
+// Transposed, zero padded [D][Tp] copies (U = SiLU(V1)), U row-major, and the padded per-row
+// vectors of the backward (LSE in log2 units, Delta = rowsum(dO * O)).  Null pointers are skipped.
+template <typename E>
+struct PrepP {
+    const E *v1, *k1, *k2, *q, *o, *d_o;
+    const float* lse;
+    E *u, *ut, *k1t, *k2t, *qt, *dot;
+    float *lse2, *delta;
+    int T, Tp, D;
+};
+
+template <typename E>
+__global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
+    const int bh = blockIdx.y, j0 = blockIdx.x * 32, T = p.T, Tp = p.Tp, D = p.D;
+    const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp;
+    for (int idx = threadIdx.x; idx < D * 32; idx += 256) {
+        const int d = idx >> 5, j = j0 + (idx & 31);
+        const bool in = j < T;
+        const size_t off = base + (size_t)(in ? j : 0) * D + d, to = tb + (size_t)d * Tp + j;
+        if (p.ut) p.ut[to] = (E)(in ? silu_f((float)p.v1[off]) : 0.f);
+        if (p.k1t) p.k1t[to] = in ? p.k1[off] : (E)0.f;
+        if (p.k2t) p.k2t[to] = in ? p.k2[off] : (E)0.f;
+        if (p.qt) p.qt[to] = in ? p.q[off] : (E)0.f;
+        if (p.dot) p.dot[to] = in ? p.d_o[off] : (E)0.f;
+    }
+    if (p.u)
+        for (int idx = threadIdx.x; idx < D * 32; idx += 256) {
+            const int j = j0 + idx / D;
+            if (j < T) {
+                const size_t off = base + (size_t)j * D + idx % D;
+                p.u[off] = (E)silu_f((float)p.v1[off]);
+            }
+        }
+    if (p.delta) {
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        for (int jj = wave; jj < 32; jj += 4) {
+            const int j = j0 + jj;
+            float part = 0.f;
+            if (j < T)
+                for (int d = lane; d < D; d += 64)
+                    part += (float)p.o[base + (size_t)j * D + d] * (float)p.d_o[base + (size_t)j * D + d];
+            part = wave_sum(part);
+            if (lane == 0) {
+                p.delta[(size_t)bh * Tp + j] = part;
+                p.lse2[(size_t)bh * Tp + j] = j < T ? p.lse[(size_t)bh * T + j] * kLog2e : 0.f;
+            }
+        }
+    }
+}
+
+struct Layout {
+    size_t u, ut, k1t, k2t, qt, dot, w, wt, dr, drt, r, dk2p, lse1, lse2, delta, delta1, total;
+};
+Layout layout(int BH, int T, int D, bool bwd) {
+    const size_t Tp = (size_t)(T + 31) / 32 * 32, n = (size_t)BH * T * D, nt = (size_t)BH * D * Tp, nv = (size_t)BH * Tp;
+    Layout l{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        off = (off + 255) & ~size_t(255);
+        const size_t r = off;
+        off += bytes;
+        return r;
+    };
+    l.ut = take(nt * 2);
+    l.wt = take(nt * 2);
+    l.lse1 = take(nv * 4);
+    if (bwd) {
+        l.u = take(n * 2);
+        l.k1t = take(nt * 2);
+        l.k2t = take(nt * 2);
+        l.qt = take(nt * 2);
+        l.dot = take(nt * 2);
+        l.w = take(n * 2);
+        l.dr = take(n * 2);
+        l.drt = take(nt * 2);
+        l.r = take(n * 4);
+        l.dk2p = take(n * 4);
+        l.lse2 = take(nv * 4);
+        l.delta = take(nv * 4);
+        l.delta1 = take(nv * 4);
+    }
+    l.total = (off + 255) & ~size_t(255);
+    return l;
+}
+
+template <int D>
+constexpr size_t fwd_smem() { return 4 * (size_t)(kW * D * kLdr + 2 * kW * 32); }
+template <int D>
+constexpr size_t col_smem() { return 4 * (size_t)(kW * D * kLdr + kW * 32 + 8 * 32); }
+template <int D>
+constexpr size_t row_smem() { return 4 * (size_t)(kW * D * kLdr); }
+
+template <typename F>
+hipError_t allow_smem(F kern, size_t bytes) {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+template <typename E, int D>
+hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
+    const int Tp = (a.T + 31) / 32 * 32;
+    const Layout l = layout(a.BH, a.T, D, for_bwd);
+    char* ws = static_cast<char*>(a.workspace);
+    const dim3 grid(Tp / 32, a.BH);
+    auto kern = attn_fwd_mfma_kernel<E, D>;
+    hipError_t e = allow_smem(kern, fwd_smem<D>());
+    if (e != hipSuccess) return e;
+    const float sl2 = a.alpha * kLog2e;
+
+    if (!for_bwd) {  // the backward's prep kernel has already written U^T
+        PrepP<E> pp{};
+        pp.v1 = (const E*)a.v1; pp.ut = (E*)(ws + l.ut);
+        pp.T = a.T; pp.Tp = Tp; pp.D = D;
+        hipLaunchKernelGGL(dps_prep_kernel<E>, grid, dim3(256), 0, st, pp);
+    }
+    // inner: rows K2[t], keys K1, values U; R (fp32, backward only), W = R * V2 and W^T, lse1 (log2)
+    AttnFwdP<E> p{};
+    p.x = (const E*)a.k2; p.k = (const E*)a.k1; p.vt = (const E*)(ws + l.ut); p.mul = (const E*)a.v2;
+    p.out_f32 = for_bwd ? (float*)(ws + l.r) : nullptr;
+    p.outm = for_bwd ? (E*)(ws + l.w) : nullptr;
+    p.outm_t = (E*)(ws + l.wt);
+    p.lse = (float*)(ws + l.lse1); p.lse_stride = Tp; p.lse_scale = 1.0f;
+    p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff;
+    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, p);
+    if (for_bwd) return hipGetLastError();
+    // outer: rows Q[q], keys K2 with bias lse1, values W; O and LSE (natural log)
+    AttnFwdP<E> o{};
+    o.x = (const E*)a.q; o.k = (const E*)a.k2; o.vt = (const E*)(ws + l.wt); o.bias = (const float*)(ws + l.lse1);
+    o.out = (E*)a.o_out; o.lse = a.lse_out; o.lse_stride = a.T; o.lse_scale = kLn2;
+    o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T;
+    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, o);
+    return hipGetLastError();
+}
+
+template <typename E, int D>
+hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
+    const int Tp = (a.T + 31) / 32 * 32;
+    const Layout l = layout(a.BH, a.T, D, true);
+    char* ws = static_cast<char*>(a.workspace);
+    const dim3 grid(Tp / 32, a.BH);
+    auto krow = attn_bwd_row_mfma_kernel<E, D>;
+    auto kcol_link = attn_bwd_col_mfma_kernel<E, D, true>;
+    auto kcol = attn_bwd_col_mfma_kernel<E, D, false>;
+    hipError_t e = allow_smem(krow, row_smem<D>());
+    if (e == hipSuccess) e = allow_smem(kcol_link, col_smem<D>());
+    if (e == hipSuccess) e = allow_smem(kcol, col_smem<D>());
+    if (e != hipSuccess) return e;
+
+    PrepP<E> pp{};
+    pp.v1 = (const E*)a.v1; pp.k1 = (const E*)a.k1; pp.k2 = (const E*)a.k2; pp.q = (const E*)a.q;
+    pp.o = (const E*)a.o; pp.d_o = (const E*)a.d_o; pp.lse = a.lse_in;
+    pp.u = (E*)(ws + l.u); pp.ut = (E*)(ws + l.ut); pp.k1t = (E*)(ws + l.k1t); pp.k2t = (E*)(ws + l.k2t);
+    pp.qt = (E*)(ws + l.qt); pp.dot = (E*)(ws + l.dot);
+    pp.lse2 = (float*)(ws + l.lse2); pp.delta = (float*)(ws + l.delta);
+    pp.T = a.T; pp.Tp = Tp; pp.D = D;
+    hipLaunchKernelGGL(dps_prep_kernel<E>, grid, dim3(256), 0, st, pp);
+    // recompute the inner pass: R, W, W^T, lse1
+    e = run_fwd<E, D>(a, st, true);
+    if (e != hipSuccess) return e;
+
+    // outer pass: X = Q, G = dO, K = K2 (bias lse1), V = W
+    AttnBwdP<E> o{};
+    o.x = (const E*)a.q; o.g = (const E*)a.d_o; o.k = (const E*)a.k2; o.v = (const E*)(ws + l.w);
+    o.kt = (const E*)(ws + l.k2t); o.xt = (const E*)(ws + l.qt); o.gt = (const E*)(ws + l.dot);
+    o.bias = (const float*)(ws + l.lse1); o.lse2 = (const float*)(ws + l.lse2); o.delta = (const float*)(ws + l.delta);
+    o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T;
+    o.dx = (E*)a.dq;
+    o.dk_f32 = (float*)(ws + l.dk2p);
+    o.r_f32 = (const float*)(ws + l.r); o.v2 = (const E*)a.v2; o.dv2 = (E*)a.dv2;
+    o.dr = (E*)(ws + l.dr); o.dr_t = (E*)(ws + l.drt); o.delta1 = (float*)(ws + l.delta1);
+    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), row_smem<D>(), st, o);
+    hipLaunchKernelGGL(kcol_link, grid, dim3(64 * kW), col_smem<D>(), st, o);
+
+    // inner pass: X = K2, G = dR, K = K1, V = U
+    AttnBwdP<E> i{};
+    i.x = (const E*)a.k2; i.g = (const E*)(ws + l.dr); i.k = (const E*)a.k1; i.v = (const E*)(ws + l.u);
+    i.kt = (const E*)(ws + l.k1t); i.xt = (const E*)(ws + l.k2t); i.gt = (const E*)(ws + l.drt);
+    i.lse2 = (const float*)(ws + l.lse1); i.delta = (const float*)(ws + l.delta1);
+    i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff;
+    i.addend = (const float*)(ws + l.dk2p); i.dx = (E*)a.dk2;
+    i.dk = (E*)a.dk1; i.v1 = (const E*)a.v1; i.dv = (E*)a.dv1;
+    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), row_smem<D>(), st, i);
+    hipLaunchKernelGGL(kcol, grid, dim3(64 * kW), col_smem<D>(), st, i);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool mfma_dps_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
+size_t mfma_dps_fwd_workspace(int BH, int T, int D) { return layout(BH, T, D, false).total; }
+size_t mfma_dps_bwd_workspace(int BH, int T, int D) { return layout(BH, T, D, true).total; }
+
+hipError_t mfma_dps_fwd(const MfmaDpsArgs& a, hipStream_t st) {
+    if (a.D == 64) return a.is_bf16 ? run_fwd<__bf16, 64>(a, st, false) : run_fwd<_Float16, 64>(a, st, false);
+    if (a.D == 128) return a.is_bf16 ? run_fwd<__bf16, 128>(a, st, false) : run_fwd<_Float16, 128>(a, st, false);
+    return hipErrorInvalidValue;
+}
+
+hipError_t mfma_dps_bwd(const MfmaDpsArgs& a, hipStream_t st) {
+    if (a.D == 64) return a.is_bf16 ? run_bwd<__bf16, 64>(a, st) : run_bwd<_Float16, 64>(a, st);
+    if (a.D == 128) return a.is_bf16 ? run_bwd<__bf16, 128>(a, st) : run_bwd<_Float16, 128>(a, st);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace tritt

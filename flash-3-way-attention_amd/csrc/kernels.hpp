@@ -68,4 +68,24 @@ size_t mfma_tdp_bwd_workspace(int BH, int T, int D);
 bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st);
 
+// 16-bit MFMA dot-product-sum (two chained banded attentions; D = 64 or 128).
+struct MfmaDpsArgs {
+    const void *q, *k1, *k2, *v1, *v2;
+    void* o_out;          // forward output
+    float* lse_out;       // forward output [BH, T] (natural log)
+    const void *o, *d_o;  // backward inputs
+    const float* lse_in;  // backward input
+    void *dq, *dk1, *dk2, *dv1, *dv2;
+    void* workspace;      // mfma_dps_{fwd,bwd}_workspace() bytes
+    int BH, T, D;
+    float alpha;
+    int causal, k_diff;
+    int is_bf16;
+};
+size_t mfma_dps_fwd_workspace(int BH, int T, int D);
+size_t mfma_dps_bwd_workspace(int BH, int T, int D);
+bool mfma_dps_supported(int D, int dtype_is_16bit);
+hipError_t mfma_dps_fwd(const MfmaDpsArgs& a, hipStream_t st);
+hipError_t mfma_dps_bwd(const MfmaDpsArgs& a, hipStream_t st);
+
 }  // namespace tritt

@@ -92,6 +92,64 @@ def test_config4_bf16_T1024():
             util.assert_close(name, a[b:b + 1, h:h + 1], ref, **LOWP)
 
 
+@pytest.mark.parametrize("seq_len", [1, 33, 100, 257])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("D", [64, 128])
+def test_mfma_ragged_lengths(seq_len, causal, D):
+    """16-bit tensors take the MFMA kernels (forced, so a silent fall-back would fail)."""
+    inputs = orc.make_inputs(1, 2, seq_len, D, torch.bfloat16, seed=20 + seq_len)
+    alpha = 1 / math.sqrt(D)
+    z, lse, grads = util.oracle_dps(inputs, alpha, causal, seq_len)
+    out, m, g = util.run_dps(inputs, alpha, causal, seq_len, flags=2)
+    util.assert_close("out", out, z, **LOWP)
+    util.assert_close("m", m, lse, rtol=1e-3, atol=2e-2)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+        if seq_len > 1:
+            assert util.rel_err(a, b) <= 3e-2, (name, util.rel_err(a, b))
+
+
+@pytest.mark.parametrize("k_diff", [0, 3, 40, 1000])
+def test_mfma_k_diff_band(k_diff):
+    inputs = orc.make_inputs(2, 2, 150, 64, torch.float16, seed=31)
+    z, lse, grads = util.oracle_dps(inputs, 1 / 8, True, k_diff)
+    out, m, g = util.run_dps(inputs, 1 / 8, True, k_diff, flags=2)
+    util.assert_close("out", out, z, **LOWP)
+    util.assert_close("m", m, lse, rtol=1e-3, atol=2e-2)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+
+
+def test_mfma_matches_generic_kernels():
+    inputs = orc.make_inputs(1, 3, 200, 64, torch.bfloat16, seed=32)
+    a = util.run_dps(inputs, 1 / 8, True, 50, flags=2)
+    b = util.run_dps(inputs, 1 / 8, True, 50, flags=1)
+    util.assert_close("out", a[0], b[0], **LOWP)
+    util.assert_close("m", a[1], b[1], rtol=1e-3, atol=2e-2)
+    for name, x, y in zip(util.NAMES, a[2], b[2]):
+        util.assert_mostly_close(name, x, y, **LOWP)
+
+
+def test_mfma_large_logits():
+    """Logits of a few hundred: the online softmax and the chained lse1 bias must not overflow."""
+    inputs = [t * (6.0 if i < 3 else 1.0) for i, t in enumerate(orc.make_inputs(1, 2, 128, 64, torch.bfloat16, seed=33))]
+    out, m, g = util.run_dps(inputs, 1 / 8, True, 128, flags=2)
+    assert torch.isfinite(out).all() and torch.isfinite(m).all()
+    assert all(torch.isfinite(x).all() for x in g)
+    z, lse, _ = util.oracle_dps(inputs, 1 / 8, True, 128)
+    util.assert_close("m", m, lse, rtol=2e-3, atol=5e-2)
+    bad = ((out - z).abs() > 5e-2 + 5e-2 * z.abs()).float().mean().item()
+    assert bad < 0.01, bad
+
+
+def test_force_mfma_refused_for_fp32():
+    from flash_trittention import _lib
+
+    inputs = orc.make_inputs(1, 1, 32, 64, torch.float32, seed=34)
+    with pytest.raises(RuntimeError):
+        util.run_dps(inputs, 1 / 8, True, 32, flags=_lib.FLAG_FORCE_MFMA)
+
+
 def test_bitwise_reproducible():
     inputs = orc.make_inputs(1, 2, 200, 64, torch.bfloat16, seed=16)
     a = util.run_dps(inputs, 1 / 8, True, 200)

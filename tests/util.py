@@ -65,7 +65,17 @@ def _run_tdp(flash_trittention, inputs, alpha, causal, windows, backward, device
     return out.detach().float().cpu(), grads
 
 
-def run_dps(inputs, alpha, causal, k_diff, backward=True, device="cuda"):
+def run_dps(inputs, alpha, causal, k_diff, backward=True, device="cuda", flags=0):
+    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTritonFunction
+
+    TrittentionTritonFunction.impl_flags = flags
+    try:
+        return _run_dps(inputs, alpha, causal, k_diff, backward, device)
+    finally:
+        TrittentionTritonFunction.impl_flags = 0
+
+
+def _run_dps(inputs, alpha, causal, k_diff, backward, device):
     from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
 
     q, k1, k2, v1, v2, do = (t.to(device) for t in inputs)
