@@ -238,7 +238,7 @@ def main():
                      "achieved": bwd_tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": bwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BWD_ROWS,
                      "flops_per_launch": f_bwd // 2, "ms_per_launch": ms_bwd / 2},
-        "roofline_fwd": {"bound": "mfma", "kernel": "tdp_fwd_mfma_kernel<bf16,64,NT=1,16 waves>",
+        "roofline_fwd": {"bound": "mfma", "kernel": "tdp_fwd_mfma_kernel<bf16,64,NT=2,8 waves>",
                          "achieved": fwd_tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                          "frac": fwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_FWD,
                          "flops_per_launch": f_fwd, "ms_per_launch": ms_fwd},

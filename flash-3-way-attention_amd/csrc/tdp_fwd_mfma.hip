@@ -8,7 +8,7 @@
 // merged once per k-tile:  O[q] = sum_k w_k * V2[k] (.) Tv[(q,k)],  w_k = exp2(m_qk - M_q).
 //
 // Work decomposition.  One workgroup = WAVES waves = BQ = WAVES*NT queries of one (batch, head)
-// (D=64: 16 waves x 1 query at 4 waves per SIMD; D=128: 8 waves x 1 query).  A wave owns NT
+// (D=64: 8 waves x 2 queries at 2 waves per SIMD; D=128: 8 waves x 1 query).  A wave owns NT
 // queries; a 32x32 MFMA tile is 32 consecutive k (columns) of ONE query, so the causal bound
 // j <= q is uniform over a tile and the k-merge stays inside the wave.
 // Outer loop: k-tiles of 32.  Inner loop: JS-row stages of K1 and U^T, staged through LDS and
@@ -102,32 +102,50 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     }
 
     // ---- staging helpers ------------------------------------------------------------------
-    uint4 rs[CS], rkv[CK];
+    // one stage = K1 [JS][D] then U^T [D][JS], 16-byte chunks dealt out to the threads: either one
+    // chunk per thread (ra[0]) or CH from each (ra from K1, rb from U^T)
+    constexpr int CH = K1_CHUNKS >= NTH ? K1_CHUNKS / NTH : 1;
+    static_assert(CS == 1 || K1_CHUNKS % NTH == 0, "stage chunks per thread");
+    uint4 ra[CH], rb[CH], rkv[CK];
+    auto k1_chunk = [&](int item, int jb) {
+        const int r = item / (D / 8), ch = item % (D / 8);
+        return reinterpret_cast<const uint4*>(K1 + (size_t)min(jb + r, T - 1) * D + ch * 8);
+    };
+    auto ut_chunk = [&](int i2, int jb) {
+        const int d = i2 / (JS / 8), cj = i2 % (JS / 8);
+        return reinterpret_cast<const uint4*>(UT + (size_t)d * p.Tp + jb + cj * 8);
+    };
+    auto k1_slot = [&](int item, int buf) {
+        const int r = item / (D / 8), ch = item % (D / 8);
+        return reinterpret_cast<uint4*>(sK1 + (buf * JS + r) * LDK + ch * 8);
+    };
+    auto ut_slot = [&](int i2, int buf) {
+        const int d = i2 / (JS / 8), cj = i2 % (JS / 8);
+        return reinterpret_cast<uint4*>(sUT + (buf * D + d) * LDU + cj * 8);
+    };
     auto issue_stage = [&](int st) {
         const int jb = st * JS;
+        if constexpr (CS > 1) {
 #pragma unroll
-        for (int c = 0; c < CS; ++c) {
-            const int item = tid + c * NTH;
-            if (item < K1_CHUNKS) {
-                const int r = item / (D / 8), ch = item % (D / 8);
-                rs[c] = *reinterpret_cast<const uint4*>(K1 + (size_t)min(jb + r, T - 1) * D + ch * 8);
-            } else if (item < STAGE_CHUNKS) {
-                const int i2 = item - K1_CHUNKS, d = i2 / (JS / 8), cj = i2 % (JS / 8);
-                rs[c] = *reinterpret_cast<const uint4*>(UT + (size_t)d * p.Tp + jb + cj * 8);
+            for (int c = 0; c < CH; ++c) {
+                ra[c] = *k1_chunk(tid + c * NTH, jb);
+                rb[c] = *ut_chunk(tid + c * NTH, jb);
             }
+        } else {
+            if (tid < K1_CHUNKS) ra[0] = *k1_chunk(tid, jb);
+            else if (tid < STAGE_CHUNKS) ra[0] = *ut_chunk(tid - K1_CHUNKS, jb);
         }
     };
     auto commit_stage = [&](int buf) {
+        if constexpr (CS > 1) {
 #pragma unroll
-        for (int c = 0; c < CS; ++c) {
-            const int item = tid + c * NTH;
-            if (item < K1_CHUNKS) {
-                const int r = item / (D / 8), ch = item % (D / 8);
-                *reinterpret_cast<uint4*>(sK1 + (buf * JS + r) * LDK + ch * 8) = rs[c];
-            } else if (item < STAGE_CHUNKS) {
-                const int i2 = item - K1_CHUNKS, d = i2 / (JS / 8), cj = i2 % (JS / 8);
-                *reinterpret_cast<uint4*>(sUT + (buf * D + d) * LDU + cj * 8) = rs[c];
+            for (int c = 0; c < CH; ++c) {
+                *k1_slot(tid + c * NTH, buf) = ra[c];
+                *ut_slot(tid + c * NTH, buf) = rb[c];
             }
+        } else {
+            if (tid < K1_CHUNKS) *k1_slot(tid, buf) = ra[0];
+            else if (tid < STAGE_CHUNKS) *ut_slot(tid - K1_CHUNKS, buf) = ra[0];
         }
     };
     auto issue_ktile = [&](int kt) {
@@ -233,7 +251,93 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[t][dt][i] = 0.f;
             }
-            for (int st = 0; st < nst; ++st, ++gstage) {
+            int st = 0;
+            if constexpr (NT == 2 && !CAREFUL) {
+                // Stages whose 64 keys lie inside the causal bound of both tiles of this wave: a loop
+                // without branches on tile validity, so the accumulators stay in place (no copies
+                // at control-flow joins) and the wave itself overlaps matrix and vector work.  The
+                // arbiter serves the oldest wave first and all waves of a workgroup reach the same
+                // phase together, so overlap between waves cannot be relied on: the second tile's
+                // score product is issued in between the exp2/pack work of the first, and the first
+                // tile's value product in between that of the second.  K1 and U^T operands are
+                // read once for both tiles; the K1 operands of a block are fetched during the
+                // previous block of the same stage.
+                const int nfull = min(nst, (min(jmax[0], jmax[1]) + 1) / JS);
+                auto fused = [&](const E* utp, const E* k1_next, v8 (&kn)[KS]) {
+                v8 ka[KS], ua[DT][2];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) ka[ks] = kn[ks];
+                f32x16 s0, s1;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s0[i] = 0.f;
+                    s1[i] = 0.f;
+                }
+                v8 pa0[2], pa1[2];
+                // quarter r of a tile's exp2 / pack / row-sum work: 4 exp2, 2 packs, 2 dot2
+                auto quarter = [&](const f32x16& sc, v8 (&pa)[2], float& ls, int r) {
+                    const int h = r >> 1, e0 = 4 * (r & 1);
+#pragma unroll
+                    for (int e = e0; e < e0 + 4; e += 2) {
+                        const v2 pr = M::pack(fast_exp2(sc[h * 8 + e]), fast_exp2(sc[h * 8 + e + 1]));
+                        ls = M::add_pair(pr, ls);
+                        pa[h][e] = pr[0];
+                        pa[h][e + 1] = pr[1];
+                    }
+                };
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) s0 = M::mma(ka[ks], bq[0][ks], s0);
+                __builtin_amdgcn_sched_barrier(0);
+                // U^T operands are first needed two MFMA groups from here
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        ua[dt][h] = *reinterpret_cast<const v8*>(utp + dt * 32 * LDU + h * 16);
+                __builtin_amdgcn_sched_barrier(0);
+                static_assert(KS == 4 && DT == 2, "the interleave below is written for D = 64");
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    s1 = M::mma(ka[r], bq[1][r], s1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    quarter(s0, pa0, lsum[0], r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // the K1 operands are dead now: fetch those of the next block (null: none in reach)
+                if (k1_next) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1_next + ks * 16);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    acc[0][r & 1] = M::mma(pa0[r >> 1], ua[r & 1][r >> 1], acc[0][r & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    quarter(s1, pa1, lsum[1], r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[1][r & 1] = M::mma(pa1[r >> 1], ua[r & 1][r >> 1], acc[1][r & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                };
+                for (; st < nfull; ++st, ++gstage) {
+                    const int sb = gstage & 1;
+                    issue_stage(st + 1 < nst ? st + 1 : 0);
+                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
+                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
+                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
+                    v8 kn[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
+                    static_assert(JS == 64 || NT != 2, "two blocks per stage");
+                    fused(utp, k1p + 32 * LDK, kn);
+                    fused(utp + 32, nullptr, kn);
+                    commit_stage(sb ^ 1);
+                    __syncthreads();
+                }
+            }
+            for (; st < nst; ++st, ++gstage) {
                 const int sb = gstage & 1;
                 // stage 0 is fetched again after the last stage: the next k-tile, or a CAREFUL repeat
                 // of this one, starts from it
@@ -444,15 +548,15 @@ size_t mfma_tdp_fwd_workspace(int BH, int T, int D) {
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
 
 // Tile shape used for D = 64.  TRITT_FWD_VARIANT (read once) selects another instantiation for
-// tuning sweeps: "nt1w16", "nt2w8", "nt1w8", "nt1w16j128", "nt1w8j128", "nt2w8j128", "nt2w16j128".
+// tuning sweeps: "nt2w8" (default), "nt1w16", "nt1w8".
 static int fwd_variant() {
     static int v = -1;
     if (v < 0) {
         const char* e = getenv("TRITT_FWD_VARIANT");
         v = 0;
         if (e) {
-            const char* names[] = {"nt1w16", "nt2w8", "nt1w8", "nt1w16j128", "nt1w8j128", "nt2w8j128", "nt2w16j128"};
-            for (int i = 0; i < 7; ++i)
+            const char* names[] = {"nt2w8", "nt1w16", "nt1w8"};
+            for (int i = 0; i < 3; ++i)
                 if (!strcmp(e, names[i])) v = i;
         }
     }
@@ -462,13 +566,9 @@ static int fwd_variant() {
 template <typename E>
 static hipError_t launch_d64(const MfmaFwdArgs& a, hipStream_t st) {
     switch (fwd_variant()) {
-        case 1: return launch<E, 64, 2, 8, 2, 64>(a, st);
+        case 1: return launch<E, 64, 1, 16, 4, 64>(a, st);
         case 2: return launch<E, 64, 1, 8, 4, 64>(a, st);
-        case 3: return launch<E, 64, 1, 16, 4, 128>(a, st);
-        case 4: return launch<E, 64, 1, 8, 4, 128>(a, st);
-        case 5: return launch<E, 64, 2, 8, 2, 128>(a, st);
-        case 6: return launch<E, 64, 2, 16, 2, 128>(a, st);
-        default: return launch<E, 64, 1, 16, 4, 64>(a, st);
+        default: return launch<E, 64, 2, 8, 2, 64>(a, st);
     }
 }
 
