@@ -40,21 +40,35 @@ struct BwdParams {
 // Owner = 32 consecutive queries (the columns of every MFMA tile of the workgroup).  The eight
 // waves take eight consecutive K2/V2 rows k per "round" (one k per wave), so a tile is
 // (32 q) x (1 k), and sweep j in 64-row stages of K1 / U (and their transposes) shared by the
-// workgroup, fetched direct-to-LDS three stages deep.  Per round and wave, over the whole j sweep:
+// workgroup.  Per round and wave, over the whole j sweep:
 //   Yq[(q,k), :] = sum_j dS K1[j, :]        Tv[(q,k), :] = sum_j P U[j, :]
 // and then
 //   dQ[q]  += Yq (.) K2[k]                      (WITH_DQ: registers, all rounds; reduced over waves at the end)
 //   dK2[k] += alpha * sum_q Yq (.) Q[q]         (sum over the tile's 32 rows in registers, then ONE
 //   dV2[k] += sum_q Tv (.) dO[q]                 returnless fp32 atomic per element per (q-tile, k))
+//
+// The inner loop is laid out for latency: a wave that reads each MFMA operand from LDS just before
+// the MFMA that uses it spends most of a step waiting for sixteen LDS round trips, and two waves
+// per SIMD cannot hide that.  Here
+//  * the eight row operands (K1 / U rows) of a step are read one step ahead, the eight transposed
+//    operands (K1^T / U^T) right after the score products, under the exp2 / pack work;
+//  * the gradient products of the first half of the registers are issued between the exp2 / pack
+//    work of the second half;
+//  * an invalid (q, j, k) gets -3e4 as C operand of the first score k-step, so its P is exactly 0
+//    and interior and diagonal steps share one loop body: no branch around accumulator updates,
+//    the accumulators stay in place;
+//  * stages are fetched direct-to-LDS three ahead into four buffers and the workgroup barrier
+//    sits in the middle of a stage: by then the next stage has landed for every wave, so its
+//    first row operands are read during the second half and nothing waits at the stage boundary.
 template <typename E, int D, bool WITH_DQ>
 __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using v2 = typename M::v2;
-    constexpr int KS = D / 16, DT = D / 32, BQ = 32;
+    constexpr int KS = D / 16, DT = D / 32, BQ = 32, NW = 8, NTH = 64 * NW;
     constexpr int LDK = D + 8, LDF = D + 4;
-    constexpr int TILE = 64 * 64;  // elements of one dense, swizzled 64x64 stage tile (see direct_lds.hpp)
-    constexpr int NBUF = 3, LW = 4;  // stages in flight; direct loads per wave per stage
+    constexpr int TILE = 64 * 64;
+    constexpr int NBUF = 4, LW = 4;  // stage buffers; direct loads per wave per stage
     static_assert(D == 64, "stages are four 64x64 tiles = 32 blocks of 1 KB, four per wave");
 
     extern __shared__ __align__(16) char smem[];
@@ -62,9 +76,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     E* sKr = sStage + NBUF * 4 * TILE;       // [2][8][D]  K2 rows of a round (one per wave), dense
     E* sVr = sKr + 2 * 8 * D;                // [2][8][D]  V2 rows
     E* sQb = sVr + 2 * 8 * D;                // [BQ][LDK]  Q tile (operand build)
-    E* sOb = sQb + BQ * LDK;               // [BQ][LDK]    dO tile
-    float* sQf = reinterpret_cast<float*>(sOb + BQ * LDK);  // [BQ][LDF]  alpha * Q, fp32 (epilogue)
-    float* sOf = sQf + BQ * LDF;                            // [BQ][LDF]  dO, fp32
+    E* sOb = sQb + BQ * LDK;                 // [BQ][LDK]  dO tile
 
     const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -86,6 +98,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     const int q0 = qt * BQ;
     const int qlast = min(T - 1, q0 + BQ - 1);
     const int jend = p.causal ? qlast : T - 1;  // last j (and last k) any query of the tile needs
+    const int jfull = p.causal ? q0 : T - 1;    // keys / rows 0 .. jfull are valid for every column
     const int nst = jend / 64 + 1, nrounds = jend / 8 + 1;
     const int q = q0 + n;                        // this lane's column
     const bool q_ok = q < T;
@@ -96,18 +109,33 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     const int tensor = wave >> 1;
     const bool rowmajor = tensor < 2;  // K1 / U: row = key j (read with permuted rows); else row = d
     const E* gsrc = uniform_ptr(tensor == 0 ? K1 : tensor == 1 ? U : tensor == 2 ? K1T : UT);
-    auto issue_stage = [&](int st, int buf) {
-        const int jb = st * 64;
-        int ln = lane;
-        asm volatile("" : "+v"(ln));  // keep this address arithmetic inside the loops (no spilled invariants)
-        const int pos = ln & 7, rr = ln >> 3;
-        E* dst = sStage + (buf * 4 + tensor) * TILE;
+    // Per-lane byte offsets of the wave's four blocks inside a stage; the stage itself only moves
+    // the (scalar) base.  Row-major tensors clamp rows past the end of the sequence (last stage of
+    // a ragged T only): that path recomputes the offsets.
+    unsigned soff[LW];
+    {
+        const int pos = lane & 7, rr = lane >> 3;
 #pragma unroll
         for (int c = 0; c < LW; ++c) {
-            const int blk = (wave & 1) * 4 + c, r = blk * 8 + rr;
-            const unsigned off = rowmajor ? (unsigned)min(jb + r, T - 1) * (D * 2) + ((pos ^ swz_perm(r)) * 16)
-                                          : ((unsigned)r * p.Tp + jb) * 2 + ((pos ^ swz_seq(r)) * 16);
-            direct_load_16(gsrc, off, dst + blk * 512);
+            const int r = ((wave & 1) * 4 + c) * 8 + rr;
+            soff[c] = rowmajor ? (unsigned)r * (D * 2) + ((pos ^ swz_perm(r)) * 16)
+                               : (unsigned)r * p.Tp * 2 + ((pos ^ swz_seq(r)) * 16);
+        }
+    }
+    auto issue_stage = [&](int st, int buf) {
+        const int jb = st * 64;
+        E* dst = sStage + (buf * 4 + tensor) * TILE + (wave & 1) * 4 * 512;
+        if (rowmajor && jb + 63 > T - 1) {
+            const int pos = lane & 7, rr = lane >> 3;
+#pragma unroll
+            for (int c = 0; c < LW; ++c) {
+                const int r = ((wave & 1) * 4 + c) * 8 + rr;
+                direct_load_16(gsrc, (unsigned)min(jb + r, T - 1) * (D * 2) + ((pos ^ swz_perm(r)) * 16), dst + c * 512);
+            }
+        } else {
+            const E* sbase = gsrc + (size_t)jb * (rowmajor ? D : 1);
+#pragma unroll
+            for (int c = 0; c < LW; ++c) direct_load_16(sbase, soff[c], dst + c * 512);
         }
     };
     auto issue_round = [&](int m, int buf) {  // waves 0, 1: K2 / V2 rows 8m .. 8m+7 (1 KB each)
@@ -119,21 +147,20 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         }
     };
 
-    // prologue: Q / dO tiles in both forms, first round, first stage
-    for (int idx = tid; idx < BQ * D; idx += 512) {
+    // prologue: Q / dO tiles in both forms, first round, first three stages (the j sweep repeats
+    // every round, so stage numbers simply cycle: stage of running index x is x mod nst)
+    for (int idx = tid; idx < BQ * D; idx += NTH) {
         const int r = idx / D, d = idx % D;
         const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
         const E qv = p.q[off], ov = p.d_o[off];
         sQb[r * LDK + d] = qv;
         sOb[r * LDK + d] = ov;
-        sQf[r * LDF + d] = (float)qv * p.alpha;
-        sOf[r * LDF + d] = (float)ov;
     }
-    issue_stage(0, 0);
-    issue_stage(nst > 1 ? 1 : 0, 1);
     issue_round(0, 0);
-    wait_vmcnt<0>();
-    __syncthreads();
+    issue_stage(0, 0);
+    issue_stage(1 % nst, 1);
+    issue_stage(2 % nst, 2);
+    barrier_keep_loads<LW>();  // stages 0 and 1 and the first round have landed for every wave
 
     // per-column constants folded into the score products (see offset_operand); a column past the
     // end of the sequence gets a huge LSE so that its P underflows to exactly 0
@@ -151,13 +178,25 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
             for (int i = 0; i < 16; ++i) dQacc[dt][i] = 0.f;
     }
 
-    int gstage = 0;
+    // row operands (K1 / U rows in MFMA A layout) of the step about to run
+    v8 ak[KS], au[KS];
+    auto load_rows = [&](int buf, int half) {
+        const E* sK1 = sStage + (buf * 4 + 0) * TILE;
+        const E* sU = sStage + (buf * 4 + 1) * TILE;
+        const int rowoff = (half * 32 + krow_off) * 64;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            ak[ks] = *reinterpret_cast<const v8*>(sK1 + rowoff + (((ks * 2 + g) ^ fperm) * 8));
+            au[ks] = *reinterpret_cast<const v8*>(sU + rowoff + (((ks * 2 + g) ^ fperm) * 8));
+        }
+    };
+    load_rows(0, 0);
+
+    int gstage = 0;          // running stage index; buffer = gstage % NBUF
+    int st_ahead = 3 % nst;  // stage number of running index gstage + 3
     for (int m = 0; m < nrounds; ++m) {
         const int mb = m & 1;
-        const int k = m * 8 + wave;                 // this wave's K2/V2 row
-        const bool k_active = k <= jend;            // wave-uniform
-        const bool k_diag = p.causal && k > q0;     // some columns of the tile have q < k
-        const bool kv_ok = !p.causal || k <= jq;    // per lane
+        const int k = m * 8 + wave;  // this wave's K2/V2 row
 
         v8 bq[KS], bg[KS];
 #pragma unroll
@@ -191,81 +230,99 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
 
         for (int st = 0; st < nst; ++st, ++gstage) {
             const int sb = gstage % NBUF;
-            // this stage has landed for every wave and the buffer two stages ahead is free; the j
-            // sweep repeats every round, so the stages fetched ahead simply cycle
-            barrier_keep_loads<LW>();
-            if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads below
-            int st2 = st + 2;
-            if (st2 >= nst) st2 -= nst;
-            if (st2 >= nst) st2 = 0;
-            issue_stage(st2, (gstage + 2) % NBUF);
-            const E* sK1 = sStage + (sb * 4 + 0) * TILE;
-            const E* sU = sStage + (sb * 4 + 1) * TILE;
             const E* sK1T = sStage + (sb * 4 + 2) * TILE;
             const E* sUT = sStage + (sb * 4 + 3) * TILE;
-            if (k_active) {
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int jb = st * 64 + half * 32;
-                    if (jb > jend) break;
-                    f32x16 s, dp;
+            for (int half = 0; half < 2; ++half) {
+                const int jb = st * 64 + half * 32;
+                // wave-uniform: some (q, j, k) of this step is invalid
+                const bool need_mask = (k > jfull) || (jb + 31 > jfull);
+                f32x16 s, dp;
+                __builtin_amdgcn_sched_barrier(0);
+                // the extra k-step subtracts LSE2[q] from S and Delta[q] from dP inside the MFMA; its C
+                // operand is 0, or -3e4 where (q, j, k) is invalid.  Element i of a lane is key
+                // jb + key_of(0, i) + 8 g.
+                if (need_mask) {
+                    const int lim = (k <= jq) ? jq - jb - 8 * g : -1;
+                    f32x16 c;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        s[i] = 0.f;
-                        dp[i] = 0.f;
-                    }
-                    const int rowoff = (half * 32 + krow_off) * 64;
-                    // the extra k-step subtracts LSE2[q] from S and Delta[q] from dP inside the MFMA
+                    for (int i = 0; i < 16; ++i) c[i] = key_of(0, i) <= lim ? 0.f : -3.0e4f;
+                    s = M::mma(ones, off_lse, c);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) s[i] = 0.f;
                     s = M::mma(ones, off_lse, s);
+                }
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks)
-                        s = M::mma(*reinterpret_cast<const v8*>(sK1 + rowoff + (((ks * 2 + g) ^ fperm) * 8)), bq[ks], s);
-                    dp = M::mma(ones, off_delta, dp);
+                for (int i = 0; i < 16; ++i) dp[i] = 0.f;
+                dp = M::mma(ones, off_delta, dp);
+                __builtin_amdgcn_sched_barrier(0);
+                if (half == 1) {
+                    // mid-stage: the buffer three stages ahead was last read in the previous stage, and
+                    // every wave is past that (the barrier below was crossed): fetch it now
+                    if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
+                    issue_stage(st_ahead, (gstage + 3) % NBUF);
+                    st_ahead = st_ahead + 1 < nst ? st_ahead + 1 : 0;
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks)
-                        dp = M::mma(*reinterpret_cast<const v8*>(sU + rowoff + (((ks * 2 + g) ^ fperm) * 8)), bg[ks], dp);
-                    v8 pa[2], da[2];
-                    // P = exp2(S - LSE2), dS = P (dP - Delta), packed as A operands of the next products.
-                    // The masked variant is a separate (wave-uniform) branch: interior steps carry no
-                    // predication.
-                    auto softmax_grad = [&](auto masked_tag) {
-                        constexpr bool MASKED = decltype(masked_tag)::value;
+                for (int ks = 0; ks < KS; ++ks) {
+                    s = M::mma(ak[ks], bq[ks], s);
+                    dp = M::mma(au[ks], bg[ks], dp);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                // transposed operands of the gradient products: they land under the exp2 / pack work
+                v8 bt[DT][2], bk[DT][2];
 #pragma unroll
-                        for (int h = 0; h < 2; ++h) {
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                            for (int e = 0; e < 8; e += 2) {
-                                const int i = h * 8 + e;
-                                float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
-                                if constexpr (MASKED) {
-                                    p0 = (kv_ok && jb + key_of(g, i) <= jq) ? p0 : 0.f;
-                                    p1 = (kv_ok && jb + key_of(g, i + 1) <= jq) ? p1 : 0.f;
-                                }
-                                const v2 pp = M::pack(p0, p1);
-                                const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
-                                pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
-                                da[h][e] = dd[0]; da[h][e + 1] = dd[1];
-                            }
-                        }
-                    };
-                    if (__builtin_amdgcn_readfirstlane(k_diag || (p.causal && jb + 31 > q0) || jb + 31 > T - 1))
-                        softmax_grad(std::true_type{});
-                    else
-                        softmax_grad(std::false_type{});
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-                        for (int h = 0; h < 2; ++h) {
-                            const int toff = (dt * 32 + n) * 64 + (((half * 4 + h * 2 + g) ^ fseq) * 8);
-                            accT[dt] = M::mma(pa[h], *reinterpret_cast<const v8*>(sUT + toff), accT[dt]);
-                            accQ[dt] = M::mma(da[h], *reinterpret_cast<const v8*>(sK1T + toff), accQ[dt]);
-                        }
+                    for (int h = 0; h < 2; ++h) {
+                        const int toff = (dt * 32 + n) * 64 + (((half * 4 + h * 2 + g) ^ fseq) * 8);
+                        bt[dt][h] = *reinterpret_cast<const v8*>(sUT + toff);
+                        bk[dt][h] = *reinterpret_cast<const v8*>(sK1T + toff);
                     }
+                __builtin_amdgcn_sched_barrier(0);
+                v8 pa[2], da[2];
+                // register pair r (0..7):  P = exp2(S), dS = P dP, both packed to 16 bit
+                auto softmax_pair = [&](int r) {
+                    const int h = r >> 2, e = 2 * (r & 3), i = h * 8 + e;
+                    const float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
+                    const v2 pp = M::pack(p0, p1);
+                    const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
+                    pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
+                    da[h][e] = dd[0]; da[h][e + 1] = dd[1];
+                };
+#pragma unroll
+                for (int r = 0; r < 4; ++r) softmax_pair(r);
+                __builtin_amdgcn_sched_barrier(0);
+                static_assert(DT == 2, "interleave written for D = 64");
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[0], bt[r >> 1][0], accT[r >> 1]);
+                    else accQ[r >> 1] = M::mma(da[0], bk[r >> 1][0], accQ[r >> 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    softmax_pair(4 + r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // the row operands are dead: read those of the next step (second half of this stage,
+                // or first half of the next one, which has landed for everyone since the barrier)
+                load_rows(half == 0 ? sb : (gstage + 1) % NBUF, half ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[1], bt[r >> 1][1], accT[r >> 1]);
+                    else accQ[r >> 1] = M::mma(da[1], bk[r >> 1][1], accQ[r >> 1]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (half == 0) {
+                    // the next stage has landed for every wave; everyone is done with the previous one
+                    barrier_keep_loads<LW>();
                 }
             }
         }
 
         // ---- round epilogue (rows of the accumulators = the 32 queries, column = d) ---------------
-        if (k_active) {
+        if (k <= jend) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const int d = dt * 32 + n;
@@ -275,36 +332,36 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 for (int i = 0; i < 16; ++i) {
                     const int r = c_row(g, i);
                     if constexpr (WITH_DQ) dQacc[dt][i] += accQ[dt][i] * kd;
-                    sk += accQ[dt][i] * sQf[r * LDF + d];
-                    sv += accT[dt][i] * sOf[r * LDF + d];
+                    sk += accQ[dt][i] * (float)sQb[r * LDK + d];
+                    sv += accT[dt][i] * (float)sOb[r * LDK + d];
                 }
                 sk += __shfl_xor(sk, 32, 64);
                 sv += __shfl_xor(sv, 32, 64);
                 if (g == 0) {
-                    unsafeAtomicAdd(p.acc_k + base + (size_t)k * D + d, sk);
+                    unsafeAtomicAdd(p.acc_k + base + (size_t)k * D + d, sk * p.alpha);
                     unsafeAtomicAdd(p.acc_v + base + (size_t)k * D + d, sv);
                 }
             }
         }
-        // all waves are done with this round's K2/V2 rows and with the last stage
-        barrier_keep_loads<LW>();
+        // all waves are done with this round's K2/V2 rows; the next round's have landed
+        barrier_keep_loads<LW + 4>();
     }
     wait_vmcnt<0>();  // the stages fetched ahead land in the buffers reused below
     __syncthreads();
 
     if constexpr (WITH_DQ) {
-        // ---- dQ: sum the eight waves' partial tiles through LDS (the stage buffers are free now) --
-        float* red = reinterpret_cast<float*>(smem);  // [8][32][LDF]
+        // ---- dQ: sum the waves' partial tiles through LDS (the stage buffers are free now) -------
+        float* red = reinterpret_cast<float*>(smem);  // [NW][32][LDF]
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) red[(wave * 32 + c_row(g, i)) * LDF + dt * 32 + n] = dQacc[dt][i];
         __syncthreads();
-        for (int idx = tid; idx < BQ * D; idx += 512) {
+        for (int idx = tid; idx < BQ * D; idx += NTH) {
             const int r = idx / D, d = idx % D;
             float v = 0.f;
 #pragma unroll
-            for (int w = 0; w < 8; ++w) v += red[(w * 32 + r) * LDF + d];
+            for (int w = 0; w < NW; ++w) v += red[(w * 32 + r) * LDF + d];
             if (q0 + r < T) p.dq[base + (size_t)(q0 + r) * D + d] = (E)(v * p.alpha);
         }
     }
@@ -428,10 +485,12 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
 
-    constexpr size_t smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8)) + 4 * (size_t)(2 * 32 * (D + 4));
+    // four stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles
+    constexpr size_t smem = 2 * (size_t)(4 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8));
     static_assert(smem >= 4 * 8 * 32 * (D + 4), "dQ reduction reuses the stage buffers");
     auto kern_dq = tdp_bwd_rows_kernel<E, D, true>;
     auto kern_nodq = tdp_bwd_rows_kernel<E, D, false>;
+    const int nthreads = 512;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq),
@@ -448,12 +507,12 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
     p.acc_k = dk2acc; p.acc_v = dv2acc;
-    hipLaunchKernelGGL(kern_dq, grid, dim3(512), smem, st, p);
+    hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU
     p.row_k = (const E*)a.k1; p.row_v = u;
     p.st_k = (const E*)a.k2; p.st_v = (const E*)a.v2; p.st_kt = k2t; p.st_vt = v2t;
     p.acc_k = dk1acc; p.acc_v = duacc;
-    hipLaunchKernelGGL(kern_nodq, grid, dim3(512), smem, st, p);
+    hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
 
     const size_t n = (size_t)a.BH * a.T * D;
     size_t gridf = (n + 255) / 256;
