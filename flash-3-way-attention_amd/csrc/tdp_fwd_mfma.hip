@@ -103,10 +103,11 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 
     // ---- staging helpers ------------------------------------------------------------------
     // one stage = K1 [JS][D] then U^T [D][JS], 16-byte chunks dealt out to the threads: either one
-    // chunk per thread (ra[0]) or CH from each (ra from K1, rb from U^T)
+    // chunk per thread (ra0) or CH from each (ra* from K1, rb* from U^T)
     constexpr int CH = K1_CHUNKS >= NTH ? K1_CHUNKS / NTH : 1;
     static_assert(CS == 1 || K1_CHUNKS % NTH == 0, "stage chunks per thread");
-    uint4 ra[CH], rb[CH], rkv[CK];
+    static_assert(CH <= 2 && CK <= 2, "staging registers are named, not indexed (indexed ones end up in scratch memory)");
+    uint4 ra0, ra1, rb0, rb1, rkv0, rkv1;
     auto k1_chunk = [&](int item, int jb) {
         const int r = item / (D / 8), ch = item % (D / 8);
         return reinterpret_cast<const uint4*>(K1 + (size_t)min(jb + r, T - 1) * D + ch * 8);
@@ -126,50 +127,53 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     auto issue_stage = [&](int st) {
         const int jb = st * JS;
         if constexpr (CS > 1) {
-#pragma unroll
-            for (int c = 0; c < CH; ++c) {
-                ra[c] = *k1_chunk(tid + c * NTH, jb);
-                rb[c] = *ut_chunk(tid + c * NTH, jb);
+            ra0 = *k1_chunk(tid, jb);
+            rb0 = *ut_chunk(tid, jb);
+            if constexpr (CH == 2) {
+                ra1 = *k1_chunk(tid + NTH, jb);
+                rb1 = *ut_chunk(tid + NTH, jb);
             }
         } else {
-            if (tid < K1_CHUNKS) ra[0] = *k1_chunk(tid, jb);
-            else if (tid < STAGE_CHUNKS) ra[0] = *ut_chunk(tid - K1_CHUNKS, jb);
+            if (tid < K1_CHUNKS) ra0 = *k1_chunk(tid, jb);
+            else if (tid < STAGE_CHUNKS) ra0 = *ut_chunk(tid - K1_CHUNKS, jb);
         }
     };
     auto commit_stage = [&](int buf) {
         if constexpr (CS > 1) {
-#pragma unroll
-            for (int c = 0; c < CH; ++c) {
-                *k1_slot(tid + c * NTH, buf) = ra[c];
-                *ut_slot(tid + c * NTH, buf) = rb[c];
+            *k1_slot(tid, buf) = ra0;
+            *ut_slot(tid, buf) = rb0;
+            if constexpr (CH == 2) {
+                *k1_slot(tid + NTH, buf) = ra1;
+                *ut_slot(tid + NTH, buf) = rb1;
             }
         } else {
-            if (tid < K1_CHUNKS) *k1_slot(tid, buf) = ra[0];
-            else if (tid < STAGE_CHUNKS) *ut_slot(tid - K1_CHUNKS, buf) = ra[0];
+            if (tid < K1_CHUNKS) *k1_slot(tid, buf) = ra0;
+            else if (tid < STAGE_CHUNKS) *ut_slot(tid - K1_CHUNKS, buf) = ra0;
         }
     };
+    // K2 [32][D] then V2 [32][D]: the guard is compiled in only when the chunks do not divide evenly
+    // (a guarded, indexed register array ends up in scratch memory)
+    constexpr bool KT_EVEN = KTILE_CHUNKS % NTH == 0;
+    auto kt_src = [&](int item, int kt) {
+        const int which = item / (4 * D), rem = item % (4 * D);
+        const int r = rem / (D / 8), ch = rem % (D / 8);
+        return reinterpret_cast<const uint4*>((which ? V2 : K2) + (size_t)min(kt * 32 + r, T - 1) * D + ch * 8);
+    };
+    auto kt_dst = [&](int item, int buf) {
+        const int which = item / (4 * D), rem = item % (4 * D);
+        const int r = rem / (D / 8), ch = rem % (D / 8);
+        return reinterpret_cast<uint4*>((which ? sV2 : sK2) + (buf * 32 + r) * LDK + ch * 8);
+    };
     auto issue_ktile = [&](int kt) {
-#pragma unroll
-        for (int c = 0; c < CK; ++c) {
-            const int item = tid + c * NTH;
-            if (item < KTILE_CHUNKS) {
-                const int which = item / (4 * D), rem = item % (4 * D);
-                const int r = rem / (D / 8), ch = rem % (D / 8);
-                const E* src = which ? V2 : K2;
-                rkv[c] = *reinterpret_cast<const uint4*>(src + (size_t)min(kt * 32 + r, T - 1) * D + ch * 8);
-            }
+        if (KT_EVEN || tid < KTILE_CHUNKS) rkv0 = *kt_src(tid, kt);
+        if constexpr (CK == 2) {
+            if (KT_EVEN || tid + NTH < KTILE_CHUNKS) rkv1 = *kt_src(tid + NTH, kt);
         }
     };
     auto commit_ktile = [&](int buf) {
-#pragma unroll
-        for (int c = 0; c < CK; ++c) {
-            const int item = tid + c * NTH;
-            if (item < KTILE_CHUNKS) {
-                const int which = item / (4 * D), rem = item % (4 * D);
-                const int r = rem / (D / 8), ch = rem % (D / 8);
-                E* dst = which ? sV2 : sK2;
-                *reinterpret_cast<uint4*>(dst + (buf * 32 + r) * LDK + ch * 8) = rkv[c];
-            }
+        if (KT_EVEN || tid < KTILE_CHUNKS) *kt_dst(tid, buf) = rkv0;
+        if constexpr (CK == 2) {
+            if (KT_EVEN || tid + NTH < KTILE_CHUNKS) *kt_dst(tid + NTH, buf) = rkv1;
         }
     };
     // broadcast a per-virtual-row scalar (held by lane n) to the C/D layout (rows in registers):
@@ -333,6 +337,83 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     static_assert(JS == 64 || NT != 2, "two blocks per stage");
                     fused(utp, k1p + 32 * LDK, kn);
                     fused(utp + 32, nullptr, kn);
+                    commit_stage(sb ^ 1);
+                    __syncthreads();
+                }
+            }
+            if constexpr (NT == 1 && !CAREFUL) {
+                // The same for one tile per wave (D = 128: two tiles do not fit the register file).
+                // The two 32-key steps of a stage play the part of the two tiles: the score product
+                // of the second step is issued between the exp2 / pack work of the first, the value
+                // product of the first between that of the second.  No branch on validity inside
+                // the loop; every operand is read ahead of its use.
+                static_assert(JS == 64, "two steps per stage");
+                const int nfull = min(nst, (jmax[0] + 1) / JS);
+                for (; st < nfull; ++st, ++gstage) {
+                    const int sb = gstage & 1;
+                    issue_stage(st + 1 < nst ? st + 1 : 0);
+                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
+                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
+                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
+                    v8 ka[KS], ua[DT][2], pa[2][2];
+                    f32x16 sc[2];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        sc[0][i] = 0.f;
+                        sc[1][i] = 0.f;
+                    }
+                    auto load_k = [&](int half) {
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks)
+                            ka[ks] = *reinterpret_cast<const v8*>(k1p + half * 32 * LDK + ks * 16);
+                    };
+                    auto load_u = [&](int half) {
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                            for (int h = 0; h < 2; ++h)
+                                ua[dt][h] = *reinterpret_cast<const v8*>(utp + half * 32 + dt * 32 * LDU + h * 16);
+                    };
+                    auto pair = [&](int half, int r) {  // register pair r (0..7): 2 exp2, 1 pack, 1 row-sum step
+                        const int h = r >> 2, e = 2 * (r & 3);
+                        const v2 pr = M::pack(fast_exp2(sc[half][h * 8 + e]), fast_exp2(sc[half][h * 8 + e + 1]));
+                        lsum[0] = M::add_pair(pr, lsum[0]);
+                        pa[half][h][e] = pr[0];
+                        pa[half][h][e + 1] = pr[1];
+                    };
+                    auto value_mma = [&](int half, int r) {  // r = 0 .. 2 DT - 1; dependent ones are DT apart
+                        const int h = r / DT, dt = r % DT;
+                        acc[0][dt] = M::mma(pa[half][h], ua[dt][h], acc[0][dt]);
+                    };
+                    load_k(0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) sc[0] = M::mma(ka[ks], bq[0][ks], sc[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_k(1);
+                    load_u(0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        sc[1] = M::mma(ka[ks], bq[0][ks], sc[1]);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int r = ks * 8 / KS; r < (ks + 1) * 8 / KS; ++r) pair(0, r);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 2 * DT; ++r) {
+                        value_mma(0, r);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int q2 = r * 8 / (2 * DT); q2 < (r + 1) * 8 / (2 * DT); ++q2) pair(1, q2);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    load_u(1);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int r = 0; r < 2 * DT; ++r) value_mma(1, r);
+                    __builtin_amdgcn_sched_barrier(0);
                     commit_stage(sb ^ 1);
                     __syncthreads();
                 }
