@@ -19,6 +19,8 @@
 
 namespace tritt {
 
+__device__ __forceinline__ int wave_of(unsigned tid) { return __builtin_amdgcn_readfirstlane(tid >> 6); }
+
 template <typename E>
 struct BwdParams {
     const E *q, *d_o;
@@ -68,7 +70,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     constexpr int KS = D / 16, DT = D / 32, BQ = 32, NW = 8, NTH = 64 * NW;
     constexpr int LDK = D + 8, LDF = D + 4;
     constexpr int TILE = 64 * 64;
-    constexpr int NBUF = 4, LW = 4;  // stage buffers; direct loads per wave per stage
+    constexpr int NBUF = 3, LW = 4;  // stage buffers; direct loads per wave per stage
     static_assert(D == 64, "stages are four 64x64 tiles = 32 blocks of 1 KB, four per wave");
 
     extern __shared__ __align__(16) char smem[];
@@ -77,6 +79,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     E* sVr = sKr + 2 * 8 * D;                // [2][8][D]  V2 rows
     E* sQb = sVr + 2 * 8 * D;                // [BQ][LDK]  Q tile (operand build)
     E* sOb = sQb + BQ * LDK;                 // [BQ][LDK]  dO tile
+    // dQ / alpha of the tile, summed over rounds: one slice per pair of waves, element (dt, i) of a
+    // lane at [((dt * 4 + i / 4) * 64 + lane) * 4 + i % 4] (the accumulator layout, 16 bytes per access)
+    float* sDQ = reinterpret_cast<float*>(sOb + BQ * LDK) + (wave_of(threadIdx.x) >> 1) * (BQ * D);
 
     const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -156,11 +161,14 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         sQb[r * LDK + d] = qv;
         sOb[r * LDK + d] = ov;
     }
+    if constexpr (WITH_DQ) {
+        float* all = reinterpret_cast<float*>(sOb + BQ * LDK);
+        for (int idx = tid; idx < (NW / 2) * BQ * D; idx += NTH) all[idx] = 0.f;
+    }
     issue_round(0, 0);
     issue_stage(0, 0);
     issue_stage(1 % nst, 1);
-    issue_stage(2 % nst, 2);
-    barrier_keep_loads<LW>();  // stages 0 and 1 and the first round have landed for every wave
+    barrier_keep_loads<0>();  // stages 0 and 1 and the first round have landed for every wave
 
     // per-column constants folded into the score products (see offset_operand); a column past the
     // end of the sequence gets a huge LSE so that its P underflows to exactly 0
@@ -170,14 +178,10 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     const int krow_off = key_of_row(n);
     const int fperm = swz_perm(krow_off), fseq = swz_seq(n);
 
-    f32x16 dQacc[WITH_DQ ? DT : 1];
-    if constexpr (WITH_DQ) {
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) dQacc[dt][i] = 0.f;
-    }
-
+    // dQ[q] += Yq (.) K2[k] once per round.  A register tile per wave would cost 32 registers in a
+    // loop that has none to spare, so the running sum lives in LDS: the two waves of a pair add
+    // their round's tile to the pair's slice one after the other, the even wave before the
+    // round-end barrier, the odd wave after it.
     // row operands (K1 / U rows in MFMA A layout) of the step about to run
     v8 ak[KS], au[KS];
     auto load_rows = [&](int buf, int half) {
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     load_rows(0, 0);
 
     int gstage = 0;          // running stage index; buffer = gstage % NBUF
-    int st_ahead = 3 % nst;  // stage number of running index gstage + 3
+    int st_ahead = 2 % nst;  // stage number of running index gstage + 2
     for (int m = 0; m < nrounds; ++m) {
         const int mb = m & 1;
         const int k = m * 8 + wave;  // this wave's K2/V2 row
@@ -261,7 +265,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                     // mid-stage: the buffer three stages ahead was last read in the previous stage, and
                     // every wave is past that (the barrier below was crossed): fetch it now
                     if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
-                    issue_stage(st_ahead, (gstage + 3) % NBUF);
+                    issue_stage(st_ahead, (gstage + 2) % NBUF);
                     st_ahead = st_ahead + 1 < nst ? st_ahead + 1 : 0;
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -316,22 +320,35 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 __builtin_amdgcn_sched_barrier(0);
                 if (half == 0) {
                     // the next stage has landed for every wave; everyone is done with the previous one
-                    barrier_keep_loads<LW>();
+                    barrier_keep_loads<0>();
                 }
             }
         }
 
         // ---- round epilogue (rows of the accumulators = the 32 queries, column = d) ---------------
+        [[maybe_unused]] auto add_dq = [&]() {  // slice += Yq (.) K2[k]
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const float kd = (float)sKr[(mb * 8 + wave) * D + dt * 32 + n];
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    float4* slot = reinterpret_cast<float4*>(sDQ + ((dt * 4 + i4) * 64 + lane) * 4);
+                    float4 v = *slot;
+                    v.x += accQ[dt][i4 * 4] * kd; v.y += accQ[dt][i4 * 4 + 1] * kd;
+                    v.z += accQ[dt][i4 * 4 + 2] * kd; v.w += accQ[dt][i4 * 4 + 3] * kd;
+                    *slot = v;
+                }
+            }
+        };
         if (k <= jend) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const int d = dt * 32 + n;
-                const float kd = (float)sKr[(mb * 8 + wave) * D + d];
+                [[maybe_unused]] const float kd = (float)sKr[(mb * 8 + wave) * D + d];
                 float sk = 0.f, sv = 0.f;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int r = c_row(g, i);
-                    if constexpr (WITH_DQ) dQacc[dt][i] += accQ[dt][i] * kd;
                     sk += accQ[dt][i] * (float)sQb[r * LDK + d];
                     sv += accT[dt][i] * (float)sOb[r * LDK + d];
                 }
@@ -343,27 +360,33 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 }
             }
         }
+        if constexpr (WITH_DQ) {
+            if (k <= jend && (wave & 1) == 0) add_dq();
+        }
         // all waves are done with this round's K2/V2 rows; the next round's have landed
         barrier_keep_loads<LW + 4>();
+        if constexpr (WITH_DQ) {
+            if (k <= jend && (wave & 1) == 1) add_dq();
+        }
     }
     wait_vmcnt<0>();  // the stages fetched ahead land in the buffers reused below
     __syncthreads();
 
     if constexpr (WITH_DQ) {
-        // ---- dQ: sum the waves' partial tiles through LDS (the stage buffers are free now) -------
-        float* red = reinterpret_cast<float*>(smem);  // [NW][32][LDF]
+        // ---- dQ: sum the pairs' slices; thread (wave, lane) owns accumulator registers 4*(wave%4) .. +3
+        // of d-tile wave/4, i.e. four consecutive query rows of column d
+        const float* all = reinterpret_cast<const float*>(sOb + BQ * LDK);
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) red[(wave * 32 + c_row(g, i)) * LDF + dt * 32 + n] = dQacc[dt][i];
-        __syncthreads();
-        for (int idx = tid; idx < BQ * D; idx += NTH) {
-            const int r = idx / D, d = idx % D;
-            float v = 0.f;
-#pragma unroll
-            for (int w = 0; w < NW; ++w) v += red[(w * 32 + r) * LDF + d];
-            if (q0 + r < T) p.dq[base + (size_t)(q0 + r) * D + d] = (E)(v * p.alpha);
+        for (int sl = 0; sl < NW / 2; ++sl) {
+            const float4 x = *reinterpret_cast<const float4*>(all + sl * (BQ * D) + (wave * 64 + lane) * 4);
+            v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
         }
+        const int d = (wave >> 2) * 32 + n, r0 = c_row(g, (wave & 3) * 4);
+        const float out[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (q0 + r0 + e < T) p.dq[base + (size_t)(q0 + r0 + e) * D + d] = (E)(out[e] * p.alpha);
     }
 }
 
@@ -485,9 +508,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
 
-    // four stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles
-    constexpr size_t smem = 2 * (size_t)(4 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8));
-    static_assert(smem >= 4 * 8 * 32 * (D + 4), "dQ reduction reuses the stage buffers");
+    // three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles, four dQ slices
+    constexpr size_t smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8)) + 4 * (size_t)(4 * 32 * D);
     auto kern_dq = tdp_bwd_rows_kernel<E, D, true>;
     auto kern_nodq = tdp_bwd_rows_kernel<E, D, false>;
     const int nthreads = 512;
