@@ -82,6 +82,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     // dQ / alpha of the tile, summed over rounds: one slice per pair of waves, element (dt, i) of a
     // lane at [((dt * 4 + i / 4) * 64 + lane) * 4 + i % 4] (the accumulator layout, 16 bytes per access)
     float* sDQ = reinterpret_cast<float*>(sOb + BQ * LDK) + (wave_of(threadIdx.x) >> 1) * (BQ * D);
+    // Q and dO once more, in accumulator layout for the round epilogue: [dt][lane][i] = X[c_row(lane / 32, i)][32 dt + lane % 32]
+    E* sQe = reinterpret_cast<E*>(reinterpret_cast<float*>(sOb + BQ * LDK) + (NW / 2) * (BQ * D));
+    E* sOe = sQe + DT * 64 * 16;
 
     const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -160,6 +163,12 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         const E qv = p.q[off], ov = p.d_o[off];
         sQb[r * LDK + d] = qv;
         sOb[r * LDK + d] = ov;
+    }
+    for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
+        const int i = idx & 15, ln = (idx >> 4) & 63, dt = idx >> 10;
+        const size_t off = base + (size_t)min(q0 + c_row(ln >> 5, i), T - 1) * D + dt * 32 + (ln & 31);
+        sQe[idx] = p.q[off];
+        sOe[idx] = p.d_o[off];
     }
     if constexpr (WITH_DQ) {
         float* all = reinterpret_cast<float*>(sOb + BQ * LDK);
@@ -347,10 +356,14 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 [[maybe_unused]] const float kd = (float)sKr[(mb * 8 + wave) * D + d];
                 float sk = 0.f, sv = 0.f;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int r = c_row(g, i);
-                    sk += accQ[dt][i] * (float)sQb[r * LDK + d];
-                    sv += accT[dt][i] * (float)sOb[r * LDK + d];
+                for (int h = 0; h < 2; ++h) {
+                    const v8 qv = *reinterpret_cast<const v8*>(sQe + (dt * 64 + lane) * 16 + h * 8);
+                    const v8 ov = *reinterpret_cast<const v8*>(sOe + (dt * 64 + lane) * 16 + h * 8);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        sk += accQ[dt][h * 8 + e] * (float)qv[e];
+                        sv += accT[dt][h * 8 + e] * (float)ov[e];
+                    }
                 }
                 sk += __shfl_xor(sk, 32, 64);
                 sv += __shfl_xor(sv, 32, 64);
@@ -508,8 +521,9 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
 
-    // three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles, four dQ slices
-    constexpr size_t smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8)) + 4 * (size_t)(4 * 32 * D);
+    // three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles (twice: operand and epilogue layout), four dQ slices
+    constexpr size_t smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8) + 2 * (D / 32) * 64 * 16) +
+                            4 * (size_t)(4 * 32 * D);
     auto kern_dq = tdp_bwd_rows_kernel<E, D, true>;
     auto kern_nodq = tdp_bwd_rows_kernel<E, D, false>;
     const int nthreads = 512;
