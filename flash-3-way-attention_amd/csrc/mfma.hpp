@@ -54,35 +54,6 @@ struct Mma<_Float16> {
     }
 };
 
-// Folding "minus a per-column constant" into a score product.  An extra k-step whose A operand
-// is `ones_operand` (1 in k-slots 0..2 of every row) and whose B operand is `offset_operand(x)`
-// (the three 16-bit pieces of -x in the same slots of every column that should be shifted) adds
-// -x to the fp32 accumulator exactly to ~24 bits, at the price of one more MFMA and no VALU work.
-template <typename E>
-__device__ __forceinline__ typename Mma<E>::v8 ones_operand(int g) {
-    typename Mma<E>::v8 r;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) r[e] = (E)((g == 0 && e < 3) ? 1.0f : 0.0f);
-    return r;
-}
-template <typename E>
-__device__ __forceinline__ typename Mma<E>::v8 offset_operand(float x, int g) {
-    const float neg = -x;
-    const E hi = (E)neg;
-    const float r1 = neg - (float)hi;
-    const E mid = (E)r1;
-    const E lo = (E)(r1 - (float)mid);
-    typename Mma<E>::v8 r;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) r[e] = (E)0.0f;
-    if (g == 0) {
-        r[0] = hi;
-        r[1] = mid;
-        r[2] = lo;
-    }
-    return r;
-}
-
 // row of the 32x32 C/D tile held in register i of a lane in half g = lane/32
 __device__ __forceinline__ constexpr int c_row(int g, int i) { return 8 * (i / 4) + 4 * g + (i % 4); }
 

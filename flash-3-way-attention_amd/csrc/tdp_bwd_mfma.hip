@@ -179,11 +179,19 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     issue_stage(1 % nst, 1);
     barrier_keep_loads<0>();  // stages 0 and 1 and the first round have landed for every wave
 
-    // per-column constants folded into the score products (see offset_operand); a column past the
-    // end of the sequence gets a huge LSE so that its P underflows to exactly 0
+    // per-column constants that enter the score products as C operands; a column past the end of
+    // the sequence gets a huge LSE so that its P underflows to exactly 0
     const float lse2 = q_ok ? p.lse[(size_t)bh * T + q] * kLog2e : 3.0e4f;  // representable in fp16 too
     const float delta = q_ok ? p.delta[(size_t)bh * T + q] : 0.f;
-    const v8 ones = ones_operand<E>(g), off_lse = offset_operand<E>(lse2, g), off_delta = offset_operand<E>(delta, g);
+    // C operands of the first k-step of S and dP: -LSE2[q] / -Delta[q] in every register of the lane
+    // (the columns of a tile are the queries).  Opaque, so that they stay in registers.
+    f32x16 init_s, init_dp;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        init_s[i] = -lse2;
+        init_dp[i] = -delta;
+    }
+    asm volatile("" : "+v"(init_s), "+v"(init_dp));
     const int krow_off = key_of_row(n);
     const int fperm = swz_perm(krow_off), fseq = swz_seq(n);
 
@@ -252,23 +260,19 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 const bool need_mask = (k > jfull) || (jb + 31 > jfull);
                 f32x16 s, dp;
                 __builtin_amdgcn_sched_barrier(0);
-                // the extra k-step subtracts LSE2[q] from S and Delta[q] from dP inside the MFMA; its C
-                // operand is 0, or -3e4 where (q, j, k) is invalid.  Element i of a lane is key
+                // S starts from -LSE2[q] and dP from -Delta[q] (C operand of the first k-step); where
+                // (q, j, k) is invalid S starts from -3e4 instead.  Element i of a lane is key
                 // jb + key_of(0, i) + 8 g.
                 if (need_mask) {
                     const int lim = (k <= jq) ? jq - jb - 8 * g : -1;
                     f32x16 c;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) c[i] = key_of(0, i) <= lim ? 0.f : -3.0e4f;
-                    s = M::mma(ones, off_lse, c);
+                    for (int i = 0; i < 16; ++i) c[i] = key_of(0, i) <= lim ? -lse2 : -3.0e4f;
+                    s = M::mma(ak[0], bq[0], c);
                 } else {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) s[i] = 0.f;
-                    s = M::mma(ones, off_lse, s);
+                    s = M::mma(ak[0], bq[0], init_s);
                 }
-#pragma unroll
-                for (int i = 0; i < 16; ++i) dp[i] = 0.f;
-                dp = M::mma(ones, off_delta, dp);
+                dp = M::mma(au[0], bg[0], init_dp);
                 __builtin_amdgcn_sched_barrier(0);
                 if (half == 1) {
                     // mid-stage: the buffer three stages ahead was last read in the previous stage, and
@@ -280,8 +284,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    s = M::mma(ak[ks], bq[ks], s);
-                    dp = M::mma(au[ks], bg[ks], dp);
+                    if (ks > 0) s = M::mma(ak[ks], bq[ks], s);
+                    if (ks > 0) dp = M::mma(au[ks], bg[ks], dp);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 // transposed operands of the gradient products: they land under the exp2 / pack work
