@@ -267,15 +267,19 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 // read once for both tiles; the K1 operands of a block are fetched during the
                 // previous block of the same stage.
                 const int nfull = min(nst, (min(jmax[0], jmax[1]) + 1) / JS);
-                auto fused = [&](const E* utp, const E* k1_next, v8 (&kn)[KS]) {
+                // MASKED (the stages that straddle the causal bound): a key past the bound of its tile
+                // starts its score at -3e4 (C operand of the first k-step), so its P is exactly 0.
+                // Element i of a lane is key jb + key_of(0, i) + 8 g.
+                auto fused = [&](auto masked_tag, const E* utp, const E* k1_next, v8 (&kn)[KS], int jb) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
                 v8 ka[KS], ua[DT][2];
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) ka[ks] = kn[ks];
                 f32x16 s0, s1;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    s0[i] = 0.f;
-                    s1[i] = 0.f;
+                    s0[i] = (MASKED && key_of(0, i) > jmax[0] - jb - 8 * g) ? -3.0e4f : 0.f;
+                    s1[i] = (MASKED && key_of(0, i) > jmax[1] - jb - 8 * g) ? -3.0e4f : 0.f;
                 }
                 v8 pa0[2], pa1[2];
                 // quarter r of a tile's exp2 / pack / row-sum work: 4 exp2, 2 packs, 2 dot2
@@ -335,8 +339,22 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
                     static_assert(JS == 64 || NT != 2, "two blocks per stage");
-                    fused(utp, k1p + 32 * LDK, kn);
-                    fused(utp + 32, nullptr, kn);
+                    fused(std::false_type{}, utp, k1p + 32 * LDK, kn, 0);
+                    fused(std::false_type{}, utp + 32, nullptr, kn, 0);
+                    commit_stage(sb ^ 1);
+                    __syncthreads();
+                }
+                for (; st < nst; ++st, ++gstage) {  // the one or two stages on the diagonal
+                    const int sb = gstage & 1;
+                    issue_stage(st + 1 < nst ? st + 1 : 0);
+                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
+                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
+                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
+                    v8 kn[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
+                    fused(std::true_type{}, utp, k1p + 32 * LDK, kn, st * JS);
+                    if (st * JS + 32 <= jend) fused(std::true_type{}, utp + 32, nullptr, kn, st * JS + 32);
                     commit_stage(sb ^ 1);
                     __syncthreads();
                 }
