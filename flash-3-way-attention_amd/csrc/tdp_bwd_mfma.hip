@@ -213,6 +213,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     };
     load_rows(0, 0);
 
+    const bool late = (wave >> 2) & 1;  // second wave of its SIMD (waves w and w + 4 share one)
     int gstage = 0;          // running stage index; buffer = gstage % NBUF
     int st_ahead = 2 % nst;  // stage number of running index gstage + 2
     for (int m = 0; m < nrounds; ++m) {
@@ -299,6 +300,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                         bk[dt][h] = *reinterpret_cast<const v8*>(sK1T + toff);
                     }
                 __builtin_amdgcn_sched_barrier(0);
+                if (half == 0 && late) barrier_keep_loads<0>();  // see below
+                __builtin_amdgcn_sched_barrier(0);
                 v8 pa[2], da[2];
                 // register pair r (0..7):  P = exp2(S), dS = P dP, both packed to 16 bit
                 auto softmax_pair = [&](int r) {
@@ -331,10 +334,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                     else accQ[r >> 1] = M::mma(da[1], bk[r >> 1][1], accQ[r >> 1]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (half == 0) {
-                    // the next stage has landed for every wave; everyone is done with the previous one
-                    barrier_keep_loads<0>();
-                }
+                // The stage's one workgroup barrier: the next stage has landed for every wave, everyone is
+                // done with the previous one.  The two waves of a SIMD cross it at different points of
+                // their step (the first after its first step, the second in the middle of it, above):
+                // waves that leave a barrier in the same phase run score products together and exp2
+                // work together, with the other pipe idle; half a step apart, one wave's matrix phase
+                // runs under the other's vector phase.
+                if (half == 0 && !late) barrier_keep_loads<0>();
             }
         }
 
