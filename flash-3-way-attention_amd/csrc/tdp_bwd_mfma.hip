@@ -59,7 +59,7 @@ struct BwdParams {
 //  * an invalid (q, j, k) gets -3e4 as C operand of the first score k-step, so its P is exactly 0
 //    and interior and diagonal steps share one loop body: no branch around accumulator updates,
 //    the accumulators stay in place;
-//  * stages are fetched direct-to-LDS three ahead into four buffers and the workgroup barrier
+//  * stages are fetched direct-to-LDS two ahead into three buffers and the workgroup barrier
 //    sits in the middle of a stage: by then the next stage has landed for every wave, so its
 //    first row operands are read during the second half and nothing waits at the stage boundary.
 template <typename E, int D, bool WITH_DQ>
@@ -276,8 +276,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 dp = M::mma(au[0], bg[0], init_dp);
                 __builtin_amdgcn_sched_barrier(0);
                 if (half == 1) {
-                    // mid-stage: the buffer three stages ahead was last read in the previous stage, and
-                    // every wave is past that (the barrier below was crossed): fetch it now
+                    // the buffer two stages ahead was last read in the previous stage, and every wave is
+                    // past that (this stage's barrier was crossed in the first half): fetch it now
                     if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
                     issue_stage(st_ahead, (gstage + 2) % NBUF);
                     st_ahead = st_ahead + 1 < nst ? st_ahead + 1 : 0;
