@@ -35,6 +35,12 @@ struct BwdParams {
     int causal;
 };
 
+}  // namespace tritt
+
+#include "tdp_bwd_rows128.hpp"
+
+namespace tritt {
+
 // ------------------------------------------------------------------------------------------
 // Written for launch 1 (rows = K2/V2 indexed by k, streamed = K1/U indexed by j); launch 2 is the
 // same code with the two roles exchanged.
@@ -71,7 +77,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     constexpr int LDK = D + 8, LDF = D + 4;
     constexpr int TILE = 64 * 64;
     constexpr int NBUF = 3, LW = 4;  // stage buffers; direct loads per wave per stage
-    static_assert(D == 64, "stages are four 64x64 tiles = 32 blocks of 1 KB, four per wave");
+    static_assert(D == 64, "stages are four 64x64 tiles = 32 blocks of 1 KB, four per wave (D = 128: tdp_bwd_rows128_kernel)");
 
     extern __shared__ __align__(16) char smem[];
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][4 tensors: K1, U, K1^T, U^T][TILE]
@@ -531,11 +537,21 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
 
-    // three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles (twice: operand and epilogue layout), four dQ slices
-    constexpr size_t smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8) + 2 * (D / 32) * 64 * 16) +
-                            4 * (size_t)(4 * 32 * D);
-    auto kern_dq = tdp_bwd_rows_kernel<E, D, true>;
-    auto kern_nodq = tdp_bwd_rows_kernel<E, D, false>;
+    // D = 64: three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles (twice:
+    // operand and epilogue layout), four dQ slices.  D = 128: a workgroup per column half, see tdp_bwd_rows128.hpp
+    size_t smem;
+    void (*kern_dq)(BwdParams<E>);
+    void (*kern_nodq)(BwdParams<E>);
+    if constexpr (D == 128) {
+        smem = kBwd128Smem;
+        kern_dq = tdp_bwd_rows128_kernel<E, true>;
+        kern_nodq = tdp_bwd_rows128_kernel<E, false>;
+    } else {
+        smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8) + 2 * (D / 32) * 64 * 16) +
+               4 * (size_t)(4 * 32 * D);
+        kern_dq = tdp_bwd_rows_kernel<E, D, true>;
+        kern_nodq = tdp_bwd_rows_kernel<E, D, false>;
+    }
     const int nthreads = 512;
     static bool attr_set = false;
     if (!attr_set) {
@@ -548,7 +564,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         attr_set = true;
     }
     const int groups = (a.BH + 7) / 8;
-    const dim3 grid(8 * groups * p.nqt);
+    const dim3 grid(8 * groups * p.nqt * (D == 128 ? 2 : 1));
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
@@ -570,11 +586,12 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
 }
 
 size_t mfma_tdp_bwd_workspace(int BH, int T, int D) { return bwd_layout(BH, T, D).total; }
-bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && D == 64; }
+bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
 
 hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st) {
-    if (a.D != 64) return hipErrorInvalidValue;
-    return a.is_bf16 ? launch_bwd<__bf16, 64>(a, st) : launch_bwd<_Float16, 64>(a, st);
+    if (a.D == 64) return a.is_bf16 ? launch_bwd<__bf16, 64>(a, st) : launch_bwd<_Float16, 64>(a, st);
+    if (a.D == 128) return a.is_bf16 ? launch_bwd<__bf16, 128>(a, st) : launch_bwd<_Float16, 128>(a, st);
+    return hipErrorInvalidValue;
 }
 
 }  // namespace tritt

@@ -1,0 +1,375 @@
+// Triple-dot-product trittention backward on MFMA, head dimension 128 (included by
+// tdp_bwd_mfma.hip after BwdParams).
+//
+// Same decomposition as tdp_bwd_rows_kernel (rows = one K2/V2 row k per wave and round, K1 / U
+// streamed over j, the columns of every tile = 32 queries), with two differences forced by the
+// register file (two waves per SIMD, 256 registers):
+//  * a workgroup produces 64 of the 128 gradient columns (blockIdx carries the column half), so
+//    the accumulators Yq / Tv stay at 64 registers; the score products S and dP still contract
+//    over all 128 and are recomputed by both halves;
+//  * -LSE2[q] and -Delta[q] enter S and dP through one extra k-step (A = ones_operand, B =
+//    offset_operand) instead of two resident 16-register C tiles.
+// A tile-step (32 keys) is 18 + 8 MFMAs.  Stages are 32 keys: K1 and U rows as 64 x 64 tiles
+// (tile row = 32 * (d / 64) + key, the swizzle of direct_lds.hpp), K1^T and U^T of the column half
+// as compact [64 d][32 keys] tiles; three buffers, fetched direct-to-LDS two steps ahead, one
+// workgroup barrier per step.
+#pragma once
+
+namespace tritt {
+
+// An extra k-step whose A operand is `ones_operand` (1 in k-slots 0..2 of every row) and whose B
+// operand is `offset_operand(x)` (the three 16-bit pieces of -x in the same slots of the lane's
+// column) adds -x to the fp32 accumulator to ~24 bits.
+template <typename E>
+__device__ __forceinline__ typename Mma<E>::v8 ones_operand(int g) {
+    typename Mma<E>::v8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (E)((g == 0 && e < 3) ? 1.0f : 0.0f);
+    return r;
+}
+template <typename E>
+__device__ __forceinline__ typename Mma<E>::v8 offset_operand(float x, int g) {
+    const float neg = -x;
+    const E hi = (E)neg;
+    const float r1 = neg - (float)hi;
+    const E mid = (E)r1;
+    const E lo = (E)(r1 - (float)mid);
+    typename Mma<E>::v8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (E)0.0f;
+    if (g == 0) {
+        r[0] = hi;
+        r[1] = mid;
+        r[2] = lo;
+    }
+    return r;
+}
+
+// chunk swizzle of the compact transposed tiles: rows are 64 bytes, so rows r, r+4, r+8, r+12
+// share banks; 16-byte chunk c of row r sits at position c ^ swz_t(r)
+__device__ __forceinline__ constexpr int swz_t(int r) { return (r >> 2) & 3; }
+
+constexpr int kBwd128StageBytes = 24 * 1024;
+constexpr size_t kBwd128Smem = 3 * (size_t)kBwd128StageBytes      // stage buffers
+                               + 2 * (2 * 8 * 128 * 2)             // K2 / V2 rows of two rounds
+                               + 2 * (32 * (128 + 8) * 2)          // Q and dO tiles (operand build)
+                               + 4 * (32 * 64 * 4)                 // dQ slices (one per pair of waves)
+                               + 2 * (2 * 64 * 16 * 2);            // Q and dO, accumulator layout, column half
+
+template <typename E, bool WITH_DQ>
+__global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
+    using M = Mma<E>;
+    using v8 = typename M::v8;
+    using v2 = typename M::v2;
+    constexpr int D = 128, KS = 8, DT = 2, DH = 64, BQ = 32, NW = 8, NTH = 64 * NW;
+    constexpr int LDK = D + 8;
+    constexpr int NBUF = 3, LW = 3;  // stage buffers; direct loads per wave per stage
+    constexpr int STAGE = kBwd128StageBytes / 2;  // elements
+
+    extern __shared__ __align__(16) char smem[];
+    E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows 4096 | U rows 4096 | K1^T 2048 | U^T 2048]
+    E* sKr = sStage + NBUF * STAGE;          // [2][8][D]
+    E* sVr = sKr + 2 * 8 * D;
+    E* sQb = sVr + 2 * 8 * D;                // [BQ][LDK]
+    E* sOb = sQb + BQ * LDK;
+    float* sDQall = reinterpret_cast<float*>(sOb + BQ * LDK);  // [4][BQ * DH], accumulator layout
+    float* sDQ = sDQall + (wave_of(threadIdx.x) >> 1) * (BQ * DH);
+    E* sQe = reinterpret_cast<E*>(sDQall + (NW / 2) * (BQ * DH));  // [DT][64][16]
+    E* sOe = sQe + DT * 64 * 16;
+
+    const int groups = (p.BH + 7) / 8;
+    const int xcd = blockIdx.x & 7;
+    int slot = blockIdx.x >> 3;
+    const int c0 = (slot & 1) * DH;  // first gradient column of this workgroup
+    slot >>= 1;
+    const int bh = (slot % groups) * 8 + xcd;
+    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
+    if (bh >= p.BH) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int T = p.T;
+    const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
+    const E* __restrict__ K2 = p.row_k + base;
+    const E* __restrict__ V2 = p.row_v + base;
+
+    const int q0 = qt * BQ;
+    const int qlast = min(T - 1, q0 + BQ - 1);
+    const int jend = p.causal ? qlast : T - 1;
+    const int jfull = p.causal ? q0 : T - 1;
+    const int nsteps = jend / 32 + 1, nrounds = jend / 8 + 1;
+    const int q = q0 + n;
+    const bool q_ok = q < T;
+    const int jq = p.causal ? min(q, T - 1) : T - 1;
+    const float scale_log2 = p.alpha * kLog2e;
+
+    // ---- stage loader: 24 blocks of 1 KB, wave w fetches blocks 3w .. 3w+2
+    //   blocks 0..7 K1 rows, 8..15 U rows (tile rows 8b .. 8b+7), 16..19 K1^T, 20..23 U^T (16 d-rows each)
+    const E* gsrc[LW];
+    unsigned goff[LW];     // per-lane byte offset at key 0
+    unsigned gstep[LW];    // bytes per key
+    int rowkey[LW];        // row-major blocks: key offset of this lane's row inside the stage; else -1
+    unsigned rowrest[LW];  // row-major blocks: byte offset inside the row
+#pragma unroll
+    for (int c = 0; c < LW; ++c) {
+        const int b = wave * LW + c;
+        if (b < 16) {
+            const int R = (b & 7) * 8 + (lane >> 3), hh = R >> 5, r = R & 31;
+            const int chunk = (lane & 7) ^ swz_perm(r);
+            gsrc[c] = uniform_ptr((b < 8 ? p.st_k : p.st_v) + base);
+            rowkey[c] = r;
+            rowrest[c] = (unsigned)(hh * 64 + chunk * 8) * 2;
+            goff[c] = (unsigned)r * (D * 2) + rowrest[c];
+            gstep[c] = D * 2;
+        } else {
+            const int dl = ((b - 16) & 3) * 16 + (lane >> 2);
+            const int chunk = (lane & 3) ^ swz_t(dl);
+            gsrc[c] = uniform_ptr((b < 20 ? p.st_kt : p.st_vt) + tbase);
+            rowkey[c] = -1;
+            rowrest[c] = 0;
+            goff[c] = ((unsigned)(c0 + dl) * p.Tp + chunk * 8) * 2;
+            gstep[c] = 2;
+        }
+    }
+    auto issue_stage = [&](int st, int buf) {
+        const int jb = st * 32;
+        char* dst = reinterpret_cast<char*>(sStage + buf * STAGE) + wave * LW * 1024;
+        const bool ragged = jb + 31 > T - 1;  // row-major rows past the end of the sequence: clamp
+#pragma unroll
+        for (int c = 0; c < LW; ++c) {
+            unsigned off = goff[c] + (unsigned)jb * gstep[c];
+            if (ragged && rowkey[c] >= 0) off = (unsigned)min(jb + rowkey[c], T - 1) * (D * 2) + rowrest[c];
+            direct_load_16(gsrc[c], off, dst + c * 1024);
+        }
+    };
+    auto issue_round = [&](int m, int buf) {  // waves 0..3: K2 / V2 rows 8m .. 8m+7 (2 KB each = two loads)
+        if (wave < 4) {
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const int half = wave & 1;
+            const unsigned off = (unsigned)min(m * 8 + half * 4 + (ln >> 4), T - 1) * (D * 2) + (ln & 15) * 16;
+            direct_load_16(uniform_ptr(wave >= 2 ? V2 : K2), off, (wave >= 2 ? sVr : sKr) + buf * 8 * D + half * 4 * D);
+        }
+    };
+
+    // ---- prologue
+    for (int idx = tid; idx < BQ * D; idx += NTH) {
+        const int r = idx / D, d = idx % D;
+        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
+        sQb[r * LDK + d] = p.q[off];
+        sOb[r * LDK + d] = p.d_o[off];
+    }
+    for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
+        const int i = idx & 15, ln = (idx >> 4) & 63, dt = idx >> 10;
+        const size_t off = base + (size_t)min(q0 + c_row(ln >> 5, i), T - 1) * D + c0 + dt * 32 + (ln & 31);
+        sQe[idx] = p.q[off];
+        sOe[idx] = p.d_o[off];
+    }
+    if constexpr (WITH_DQ) {
+        for (int idx = tid; idx < (NW / 2) * BQ * DH; idx += NTH) sDQall[idx] = 0.f;
+    }
+    issue_round(0, 0);
+    issue_stage(0, 0);
+    issue_stage(1 % nsteps, 1);
+    int st_ahead = 2 % nsteps;  // stage number of running index gstage + 2 (the j sweep repeats every round)
+    int gstage = 0;
+
+    const float lse2 = q_ok ? p.lse[(size_t)bh * T + q] * kLog2e : 3.0e4f;
+    const float delta = q_ok ? p.delta[(size_t)bh * T + q] : 0.f;
+    const v8 a_ones = ones_operand<E>(g);
+    const v8 b_lse = offset_operand<E>(lse2, g), b_delta = offset_operand<E>(delta, g);
+    const int krow_off = key_of_row(n);
+    const int fperm = swz_perm(krow_off);
+
+    for (int m = 0; m < nrounds; ++m) {
+        const int mb = m & 1;
+        const int k = m * 8 + wave;
+
+        v8 bq[KS], bg[KS];
+        bool built = false;
+        f32x16 accQ[DT], accT[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                accQ[dt][i] = 0.f;
+                accT[dt][i] = 0.f;
+            }
+
+        for (int st = 0; st < nsteps; ++st, ++gstage) {
+            // this wave's part of stage gstage (and, at a round's first step, its part of the round's
+            // rows) has landed; after the barrier that holds for every wave's part, and every wave is
+            // done with the buffer the next fetch overwrites
+            barrier_keep_loads<LW>();
+            if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
+            issue_stage(st_ahead, (gstage + 2) % NBUF);
+            st_ahead = st_ahead + 1 < nsteps ? st_ahead + 1 : 0;
+            if (!built) {
+                // B operands of the score products of this round: alpha log2e Q (.) K2[k] and dO (.) V2[k]
+                built = true;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int off = ks * 16 + g * 8;
+                    const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * 8 + wave) * D + off);
+                    const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * 8 + wave) * D + off);
+                    const v8 qv = *reinterpret_cast<const v8*>(sQb + n * LDK + off);
+                    const v8 dv = *reinterpret_cast<const v8*>(sOb + n * LDK + off);
+                    v8 a, b;
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2) {
+                        const v2 pa = M::pack((float)kv[e] * (float)qv[e] * scale_log2,
+                                              (float)kv[e + 1] * (float)qv[e + 1] * scale_log2);
+                        const v2 pb = M::pack((float)vv[e] * (float)dv[e], (float)vv[e + 1] * (float)dv[e + 1]);
+                        a[e] = pa[0]; a[e + 1] = pa[1];
+                        b[e] = pb[0]; b[e + 1] = pb[1];
+                    }
+                    bq[ks] = a;
+                    bg[ks] = b;
+                }
+            }
+
+            const E* sb = sStage + (gstage % NBUF) * STAGE;
+            const E* sK1 = sb;
+            const E* sU = sb + 4096;
+            const E* sK1T = sb + 8192;
+            const E* sUT = sb + 8192 + 2048;
+            const int jb = st * 32;
+            const bool need_mask = (k > jfull) || (jb + 31 > jfull);
+
+            v8 ak[KS], au[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int roff = ((ks >> 2) * 32 + krow_off) * 64 + ((((ks & 3) * 2 + g) ^ fperm) * 8);
+                ak[ks] = *reinterpret_cast<const v8*>(sK1 + roff);
+                au[ks] = *reinterpret_cast<const v8*>(sU + roff);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // S starts from 0, or from -3e4 where (q, j, k) is invalid; element i of a lane is key
+            // jb + key_of(0, i) + 8 g.  The extra k-step subtracts LSE2[q] / Delta[q].
+            f32x16 s, dp;
+            {
+                f32x16 c;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) c[i] = 0.f;
+                dp = M::mma(a_ones, b_delta, c);
+                if (need_mask) {
+                    const int lim = (k <= jq) ? jq - jb - 8 * g : -1;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) c[i] = key_of(0, i) <= lim ? 0.f : -3.0e4f;
+                }
+                s = M::mma(a_ones, b_lse, c);
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                s = M::mma(ak[ks], bq[ks], s);
+                dp = M::mma(au[ks], bg[ks], dp);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            v8 bt[DT][2], bk[DT][2];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int dl = dt * 32 + n;
+                    const int toff = dl * 32 + (((h * 2 + g) ^ swz_t(dl)) * 8);
+                    bt[dt][h] = *reinterpret_cast<const v8*>(sUT + toff);
+                    bk[dt][h] = *reinterpret_cast<const v8*>(sK1T + toff);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+            v8 pa[2], da[2];
+            auto softmax_pair = [&](int r) {  // register pair r (0..7): P = exp2(S), dS = P dP, packed
+                const int h = r >> 2, e = 2 * (r & 3), i = h * 8 + e;
+                const float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
+                const v2 pp = M::pack(p0, p1);
+                const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
+                pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
+                da[h][e] = dd[0]; da[h][e + 1] = dd[1];
+            };
+#pragma unroll
+            for (int r = 0; r < 4; ++r) softmax_pair(r);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[0], bt[r >> 1][0], accT[r >> 1]);
+                else accQ[r >> 1] = M::mma(da[0], bk[r >> 1][0], accQ[r >> 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                softmax_pair(4 + r);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[1], bt[r >> 1][1], accT[r >> 1]);
+                else accQ[r >> 1] = M::mma(da[1], bk[r >> 1][1], accQ[r >> 1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // ---- round epilogue (rows of the accumulators = the 32 queries, column = c0 + 32 dt + n)
+        [[maybe_unused]] auto add_dq = [&]() {  // slice += Yq (.) K2[k]
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const float kd = (float)sKr[(mb * 8 + wave) * D + c0 + dt * 32 + n];
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    float4* slot4 = reinterpret_cast<float4*>(sDQ + ((dt * 4 + i4) * 64 + lane) * 4);
+                    float4 v = *slot4;
+                    v.x += accQ[dt][i4 * 4] * kd; v.y += accQ[dt][i4 * 4 + 1] * kd;
+                    v.z += accQ[dt][i4 * 4 + 2] * kd; v.w += accQ[dt][i4 * 4 + 3] * kd;
+                    *slot4 = v;
+                }
+            }
+        };
+        if (k <= jend) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = c0 + dt * 32 + n;
+                float sk = 0.f, sv = 0.f;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const v8 qv = *reinterpret_cast<const v8*>(sQe + (dt * 64 + lane) * 16 + h * 8);
+                    const v8 ov = *reinterpret_cast<const v8*>(sOe + (dt * 64 + lane) * 16 + h * 8);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        sk += accQ[dt][h * 8 + e] * (float)qv[e];
+                        sv += accT[dt][h * 8 + e] * (float)ov[e];
+                    }
+                }
+                sk += __shfl_xor(sk, 32, 64);
+                sv += __shfl_xor(sv, 32, 64);
+                if (g == 0) {
+                    unsafeAtomicAdd(p.acc_k + base + (size_t)k * D + d, sk * p.alpha);
+                    unsafeAtomicAdd(p.acc_v + base + (size_t)k * D + d, sv);
+                }
+            }
+        }
+        if constexpr (WITH_DQ) {
+            if (k <= jend && (wave & 1) == 0) add_dq();
+        }
+        // all waves are done with this round's K2/V2 rows; the next round's have landed (they are older
+        // than the stage loads kept in flight)
+        barrier_keep_loads<2 * LW>();
+        if constexpr (WITH_DQ) {
+            if (k <= jend && (wave & 1) == 1) add_dq();
+        }
+    }
+    wait_vmcnt<0>();  // the stages fetched ahead land in LDS before the workgroup ends
+    __syncthreads();
+
+    if constexpr (WITH_DQ) {
+        // dQ: sum the pairs' slices; thread (wave, lane) owns accumulator registers 4*(wave%4) .. +3 of
+        // d-tile wave/4, i.e. four consecutive query rows of column d
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int sl = 0; sl < NW / 2; ++sl) {
+            const float4 x = *reinterpret_cast<const float4*>(sDQall + sl * (BQ * DH) + (wave * 64 + lane) * 4);
+            v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
+        }
+        const int d = c0 + (wave >> 2) * 32 + n, r0 = c_row(g, (wave & 3) * 4);
+        const float out[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (q0 + r0 + e < T) p.dq[base + (size_t)(q0 + r0 + e) * D + d] = (E)(out[e] * p.alpha);
+    }
+}
+
+}  // namespace tritt

@@ -231,6 +231,33 @@ def test_mfma_backward_bf16(seq_len, causal):
             assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("seq_len", [1, 33, 100, 256, 300])
+def test_mfma_backward_d128_bf16(seq_len, causal):
+    """Head dimension 128: the backward kernel that produces the gradient columns in two halves."""
+    print(f"case mfma bwd D=128 T={seq_len} causal={causal}", flush=True)
+    inputs = orc.make_inputs(1, 3, seq_len, 128, torch.bfloat16, seed=seq_len + 7)
+    alpha = 1 / math.sqrt(128)
+    z, _, grads = util.oracle_tdp(inputs, alpha, causal)
+    out, g = util.run_tdp(inputs, alpha, causal, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+        if seq_len > 1:
+            assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
+
+
+def test_mfma_backward_d128_fp16_matches_generic():
+    """Head dimension 128, fp16, several batch entries and heads: MFMA kernels against the fp32 kernels."""
+    inputs = orc.make_inputs(2, 5, 150, 128, torch.float16, seed=33)
+    alpha = 1 / math.sqrt(128)
+    _, ga = util.run_tdp(inputs, alpha, True, flags=FORCE_MFMA)
+    _, gb = util.run_tdp(inputs, alpha, True, flags=FORCE_GENERIC)
+    for name, a, b in zip(util.NAMES, ga, gb):
+        util.assert_mostly_close(name, a, b, **LOWP)
+        assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
+
+
 def test_mfma_backward_fp16():
     inputs = orc.make_inputs(2, 2, 130, 64, torch.float16, seed=31)
     z, _, grads = util.oracle_tdp(inputs, 1 / 8, True)
