@@ -11,6 +11,8 @@
 //   launch 1: rows = (K2, V2), streamed = (K1, U):  dQ (owner-computes), dK2, dV2
 //   launch 2: rows = (K1, U),  streamed = (K2, V2): dK1, dU
 // See the comment above the kernel.
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 #include "direct_lds.hpp"
@@ -542,29 +544,43 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     size_t smem;
     void (*kern_dq)(BwdParams<E>);
     void (*kern_nodq)(BwdParams<E>);
+    int nthreads = 512, col_parts = 1;
     if constexpr (D == 128) {
-        smem = kBwd128Smem;
-        kern_dq = tdp_bwd_rows128_kernel<E, true>;
-        kern_nodq = tdp_bwd_rows128_kernel<E, false>;
+        // One wave per SIMD with all 128 columns is ~10 % faster once the grid fills the chip several times
+        // over; below that the smaller workgroups of the two-waves-per-SIMD shape balance better.
+        // TRITT_BWD128_VARIANT=w8 / w4 overrides the choice (read at every call).
+        bool w8 = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32) < 1024;
+        if (const char* v = getenv("TRITT_BWD128_VARIANT")) {
+            if (strcmp(v, "w8") == 0) w8 = true;
+            if (strcmp(v, "w4") == 0) w8 = false;
+        }
+        if (w8) {
+            smem = bwd128_smem(8, 64, true);
+            kern_dq = tdp_bwd_rows128_kernel<E, true, 8, 64>;
+            kern_nodq = tdp_bwd_rows128_kernel<E, false, 8, 64>;
+            col_parts = 2;
+        } else {
+            smem = bwd128_smem(4, 128, true);
+            kern_dq = tdp_bwd_rows128_kernel<E, true, 4, 128>;
+            kern_nodq = tdp_bwd_rows128_kernel<E, false, 4, 128>;
+            nthreads = 256;
+        }
     } else {
         smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8) + 2 * (D / 32) * 64 * 16) +
                4 * (size_t)(4 * 32 * D);
         kern_dq = tdp_bwd_rows_kernel<E, D, true>;
         kern_nodq = tdp_bwd_rows_kernel<E, D, false>;
     }
-    const int nthreads = 512;
-    static bool attr_set = false;
-    if (!attr_set) {
+    {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return e;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_nodq),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return e;
-        attr_set = true;
     }
     const int groups = (a.BH + 7) / 8;
-    const dim3 grid(8 * groups * p.nqt * (D == 128 ? 2 : 1));
+    const dim3 grid(8 * groups * p.nqt * col_parts);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;

@@ -2,17 +2,18 @@
 // tdp_bwd_mfma.hip after BwdParams).
 //
 // Same decomposition as tdp_bwd_rows_kernel (rows = one K2/V2 row k per wave and round, K1 / U
-// streamed over j, the columns of every tile = 32 queries), with two differences forced by the
-// register file (two waves per SIMD, 256 registers):
-//  * a workgroup produces 64 of the 128 gradient columns (blockIdx carries the column half), so
-//    the accumulators Yq / Tv stay at 64 registers; the score products S and dP still contract
-//    over all 128 and are recomputed by both halves;
-//  * -LSE2[q] and -Delta[q] enter S and dP through one extra k-step (A = ones_operand, B =
-//    offset_operand) instead of two resident 16-register C tiles.
-// A tile-step (32 keys) is 18 + 8 MFMAs.  Stages are 32 keys: K1 and U rows as 64 x 64 tiles
-// (tile row = 32 * (d / 64) + key, the swizzle of direct_lds.hpp), K1^T and U^T of the column half
-// as compact [64 d][32 keys] tiles; three buffers, fetched direct-to-LDS two steps ahead, one
-// workgroup barrier per step.
+// streamed over j, the columns of every tile = 32 queries).  The accumulators Yq / Tv of all 128
+// gradient columns are 128 registers, so there are two shapes:
+//  * NW = 4 waves, NCOL = 128: one wave per SIMD with the whole 512-entry register file; a
+//    tile-step (32 keys) is 18 + 16 MFMAs;
+//  * NW = 8 waves, NCOL = 64: two waves per SIMD, a workgroup produces one half of the gradient
+//    columns (blockIdx carries the half) and both halves recompute S and dP, which still
+//    contract over all 128: 18 + 8 MFMAs per tile-step and half.
+// -LSE2[q] and -Delta[q] enter S and dP through one extra k-step (A = ones_operand, B =
+// offset_operand) instead of two resident 16-register C tiles.  Stages are 32 keys: K1 and U rows
+// as 64 x 64 tiles (tile row = 32 * (d / 64) + key, the swizzle of direct_lds.hpp), K1^T and U^T
+// of the workgroup's columns as compact [NCOL d][32 keys] tiles; three buffers, fetched
+// direct-to-LDS two steps ahead, one workgroup barrier per step.
 #pragma once
 
 namespace tritt {
@@ -49,39 +50,48 @@ __device__ __forceinline__ typename Mma<E>::v8 offset_operand(float x, int g) {
 // share banks; 16-byte chunk c of row r sits at position c ^ swz_t(r)
 __device__ __forceinline__ constexpr int swz_t(int r) { return (r >> 2) & 3; }
 
-constexpr int kBwd128StageBytes = 24 * 1024;
-constexpr size_t kBwd128Smem = 3 * (size_t)kBwd128StageBytes      // stage buffers
-                               + 2 * (2 * 8 * 128 * 2)             // K2 / V2 rows of two rounds
-                               + 2 * (32 * (128 + 8) * 2)          // Q and dO tiles (operand build)
-                               + 4 * (32 * 64 * 4)                 // dQ slices (one per pair of waves)
-                               + 2 * (2 * 64 * 16 * 2);            // Q and dO, accumulator layout, column half
+constexpr int bwd128_stage_bytes(int ncol) { return 16 * 1024 + 2 * ncol * 64; }
+constexpr size_t bwd128_smem(int nw, int ncol, bool with_dq) {
+    return 3 * (size_t)bwd128_stage_bytes(ncol)               // stage buffers
+           + 2 * (2 * nw * 128 * 2)                            // K2 / V2 rows of two rounds
+           + 2 * (32 * (128 + 8) * 2)                          // Q and dO tiles
+           + (with_dq ? (nw / 2) * (32 * ncol * 4) : 0)        // dQ slices (one per pair of waves)
+           + (ncol == 64 ? 2 * (2 * 64 * 16 * 2) : 0);         // Q and dO in accumulator layout (NCOL = 64)
+}
 
-template <typename E, bool WITH_DQ>
-__global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
+template <typename E, bool WITH_DQ, int NW, int NCOL>
+__global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using v2 = typename M::v2;
-    constexpr int D = 128, KS = 8, DT = 2, DH = 64, BQ = 32, NW = 8, NTH = 64 * NW;
+    constexpr int D = 128, KS = 8, DT = NCOL / 32, DH = NCOL, BQ = 32, NTH = 64 * NW;
     constexpr int LDK = D + 8;
-    constexpr int NBUF = 3, LW = 3;  // stage buffers; direct loads per wave per stage
-    constexpr int STAGE = kBwd128StageBytes / 2;  // elements
+    constexpr int NBLK = 16 + NCOL / 8;      // 1 KB blocks of a stage: 8 + 8 row-major, NCOL/16 + NCOL/16 transposed
+    constexpr int NBUF = 3, LW = NBLK / NW;  // stage buffers; direct loads per wave per stage
+    constexpr int STAGE = bwd128_stage_bytes(NCOL) / 2;  // elements
+    constexpr bool EPI_TILES = NCOL == 64;   // Q / dO kept a second time in accumulator layout
+    static_assert((NW == 8 && NCOL == 64) || (NW == 4 && NCOL == 128), "two shapes");
+    static_assert(NBLK % NW == 0, "whole blocks per wave");
 
     extern __shared__ __align__(16) char smem[];
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows 4096 | U rows 4096 | K1^T 2048 | U^T 2048]
-    E* sKr = sStage + NBUF * STAGE;          // [2][8][D]
-    E* sVr = sKr + 2 * 8 * D;
-    E* sQb = sVr + 2 * 8 * D;                // [BQ][LDK]
+    E* sKr = sStage + NBUF * STAGE;          // [2][NW][D]
+    E* sVr = sKr + 2 * NW * D;
+    E* sQb = sVr + 2 * NW * D;               // [BQ][LDK]
     E* sOb = sQb + BQ * LDK;
-    float* sDQall = reinterpret_cast<float*>(sOb + BQ * LDK);  // [4][BQ * DH], accumulator layout
+    float* sDQall = reinterpret_cast<float*>(sOb + BQ * LDK);  // [NW/2][BQ * DH], accumulator layout (WITH_DQ)
     float* sDQ = sDQall + (wave_of(threadIdx.x) >> 1) * (BQ * DH);
-    E* sQe = reinterpret_cast<E*>(sDQall + (NW / 2) * (BQ * DH));  // [DT][64][16]
+    E* sQe = reinterpret_cast<E*>(sDQall + (WITH_DQ ? (NW / 2) * (BQ * DH) : 0));  // [DT][64][16] (EPI_TILES)
     E* sOe = sQe + DT * 64 * 16;
 
     const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7;
     int slot = blockIdx.x >> 3;
-    const int c0 = (slot & 1) * DH;  // first gradient column of this workgroup
-    slot >>= 1;
+    int c0 = 0;  // first gradient column of this workgroup
+    if constexpr (NCOL < D) {
+        c0 = (slot & 1) * DH;
+        slot >>= 1;
+    }
     const int bh = (slot % groups) * 8 + xcd;
     const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
     if (bh >= p.BH) return;
@@ -97,14 +107,15 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
     const int qlast = min(T - 1, q0 + BQ - 1);
     const int jend = p.causal ? qlast : T - 1;
     const int jfull = p.causal ? q0 : T - 1;
-    const int nsteps = jend / 32 + 1, nrounds = jend / 8 + 1;
+    const int nsteps = jend / 32 + 1, nrounds = jend / NW + 1;
     const int q = q0 + n;
     const bool q_ok = q < T;
     const int jq = p.causal ? min(q, T - 1) : T - 1;
     const float scale_log2 = p.alpha * kLog2e;
 
-    // ---- stage loader: 24 blocks of 1 KB, wave w fetches blocks 3w .. 3w+2
-    //   blocks 0..7 K1 rows, 8..15 U rows (tile rows 8b .. 8b+7), 16..19 K1^T, 20..23 U^T (16 d-rows each)
+    // ---- stage loader: NBLK blocks of 1 KB, wave w fetches blocks LW w .. LW w + LW - 1
+    //   blocks 0..7 K1 rows, 8..15 U rows (tile rows 8b .. 8b+7), then NCOL/16 blocks of K1^T and as many of
+    //   U^T (16 d-rows each)
     const E* gsrc[LW];
     unsigned goff[LW];     // per-lane byte offset at key 0
     unsigned gstep[LW];    // bytes per key
@@ -122,9 +133,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
             goff[c] = (unsigned)r * (D * 2) + rowrest[c];
             gstep[c] = D * 2;
         } else {
-            const int dl = ((b - 16) & 3) * 16 + (lane >> 2);
+            const int dl = ((b - 16) % (NCOL / 16)) * 16 + (lane >> 2);
             const int chunk = (lane & 3) ^ swz_t(dl);
-            gsrc[c] = uniform_ptr((b < 20 ? p.st_kt : p.st_vt) + tbase);
+            gsrc[c] = uniform_ptr((b < 16 + NCOL / 16 ? p.st_kt : p.st_vt) + tbase);
             rowkey[c] = -1;
             rowrest[c] = 0;
             goff[c] = ((unsigned)(c0 + dl) * p.Tp + chunk * 8) * 2;
@@ -142,13 +153,16 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
             direct_load_16(gsrc[c], off, dst + c * 1024);
         }
     };
-    auto issue_round = [&](int m, int buf) {  // waves 0..3: K2 / V2 rows 8m .. 8m+7 (2 KB each = two loads)
-        if (wave < 4) {
+    // the round's K2 / V2 rows NW m .. NW m + NW - 1: one load moves four rows (1 KB)
+    auto issue_round = [&](int m, int buf) {
+        constexpr int LR = NW / 4;  // loads per tensor
+        if (wave < 2 * LR) {
             int ln = lane;
             asm volatile("" : "+v"(ln));
-            const int half = wave & 1;
-            const unsigned off = (unsigned)min(m * 8 + half * 4 + (ln >> 4), T - 1) * (D * 2) + (ln & 15) * 16;
-            direct_load_16(uniform_ptr(wave >= 2 ? V2 : K2), off, (wave >= 2 ? sVr : sKr) + buf * 8 * D + half * 4 * D);
+            const int part = wave % LR;
+            const bool second = wave >= LR;
+            const unsigned off = (unsigned)min(m * NW + part * 4 + (ln >> 4), T - 1) * (D * 2) + (ln & 15) * 16;
+            direct_load_16(uniform_ptr(second ? V2 : K2), off, (second ? sVr : sKr) + buf * NW * D + part * 4 * D);
         }
     };
 
@@ -159,11 +173,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
         sQb[r * LDK + d] = p.q[off];
         sOb[r * LDK + d] = p.d_o[off];
     }
-    for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
-        const int i = idx & 15, ln = (idx >> 4) & 63, dt = idx >> 10;
-        const size_t off = base + (size_t)min(q0 + c_row(ln >> 5, i), T - 1) * D + c0 + dt * 32 + (ln & 31);
-        sQe[idx] = p.q[off];
-        sOe[idx] = p.d_o[off];
+    if constexpr (EPI_TILES) {
+        for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
+            const int i = idx & 15, ln = (idx >> 4) & 63, dt = idx >> 10;
+            const size_t off = base + (size_t)min(q0 + c_row(ln >> 5, i), T - 1) * D + c0 + dt * 32 + (ln & 31);
+            sQe[idx] = p.q[off];
+            sOe[idx] = p.d_o[off];
+        }
     }
     if constexpr (WITH_DQ) {
         for (int idx = tid; idx < (NW / 2) * BQ * DH; idx += NTH) sDQall[idx] = 0.f;
@@ -183,7 +199,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
 
     for (int m = 0; m < nrounds; ++m) {
         const int mb = m & 1;
-        const int k = m * 8 + wave;
+        const int k = m * NW + wave;
 
         v8 bq[KS], bg[KS];
         bool built = false;
@@ -210,8 +226,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const int off = ks * 16 + g * 8;
-                    const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * 8 + wave) * D + off);
-                    const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * 8 + wave) * D + off);
+                    const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * NW + wave) * D + off);
+                    const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * NW + wave) * D + off);
                     const v8 qv = *reinterpret_cast<const v8*>(sQb + n * LDK + off);
                     const v8 dv = *reinterpret_cast<const v8*>(sOb + n * LDK + off);
                     v8 a, b;
@@ -232,17 +248,21 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
             const E* sK1 = sb;
             const E* sU = sb + 4096;
             const E* sK1T = sb + 8192;
-            const E* sUT = sb + 8192 + 2048;
+            const E* sUT = sb + 8192 + NCOL * 32;
             const int jb = st * 32;
             const bool need_mask = (k > jfull) || (jb + 31 > jfull);
 
+            // row operands in two batches of four k-steps: the second is read under the first products
             v8 ak[KS], au[KS];
+            auto load_rows = [&](int first) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int roff = ((ks >> 2) * 32 + krow_off) * 64 + ((((ks & 3) * 2 + g) ^ fperm) * 8);
-                ak[ks] = *reinterpret_cast<const v8*>(sK1 + roff);
-                au[ks] = *reinterpret_cast<const v8*>(sU + roff);
-            }
+                for (int ks = first; ks < first + 4; ++ks) {
+                    const int roff = ((ks >> 2) * 32 + krow_off) * 64 + ((((ks & 3) * 2 + g) ^ fperm) * 8);
+                    ak[ks] = *reinterpret_cast<const v8*>(sK1 + roff);
+                    au[ks] = *reinterpret_cast<const v8*>(sU + roff);
+                }
+            };
+            load_rows(0);
             __builtin_amdgcn_sched_barrier(0);
             // S starts from 0, or from -3e4 where (q, j, k) is invalid; element i of a lane is key
             // jb + key_of(0, i) + 8 g.  The extra k-step subtracts LSE2[q] / Delta[q].
@@ -259,10 +279,14 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
                 }
                 s = M::mma(a_ones, b_lse, c);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            load_rows(4);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 s = M::mma(ak[ks], bq[ks], s);
                 dp = M::mma(au[ks], bg[ks], dp);
+                if (ks == 3) __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_sched_barrier(0);
             v8 bt[DT][2], bk[DT][2];
@@ -288,19 +312,22 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) softmax_pair(r);
             __builtin_amdgcn_sched_barrier(0);
+            // gradient product r of half h (0 .. 2 DT - 1): even -> Tv += P U, odd -> Yq += dS K1
+            auto grad = [&](int h, int r) {
+                if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[h], bt[r >> 1][h], accT[r >> 1]);
+                else accQ[r >> 1] = M::mma(da[h], bk[r >> 1][h], accQ[r >> 1]);
+            };
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[0], bt[r >> 1][0], accT[r >> 1]);
-                else accQ[r >> 1] = M::mma(da[0], bk[r >> 1][0], accQ[r >> 1]);
+                grad(0, r);
                 __builtin_amdgcn_sched_barrier(0);
                 softmax_pair(4 + r);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[1], bt[r >> 1][1], accT[r >> 1]);
-                else accQ[r >> 1] = M::mma(da[1], bk[r >> 1][1], accQ[r >> 1]);
-            }
+            for (int r = 4; r < 2 * DT; ++r) grad(0, r);
+#pragma unroll
+            for (int r = 0; r < 2 * DT; ++r) grad(1, r);
             __builtin_amdgcn_sched_barrier(0);
         }
 
@@ -308,7 +335,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
         [[maybe_unused]] auto add_dq = [&]() {  // slice += Yq (.) K2[k]
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const float kd = (float)sKr[(mb * 8 + wave) * D + c0 + dt * 32 + n];
+                const float kd = (float)sKr[(mb * NW + wave) * D + c0 + dt * 32 + n];
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
                     float4* slot4 = reinterpret_cast<float4*>(sDQ + ((dt * 4 + i4) * 64 + lane) * 4);
@@ -324,14 +351,22 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
             for (int dt = 0; dt < DT; ++dt) {
                 const int d = c0 + dt * 32 + n;
                 float sk = 0.f, sv = 0.f;
+                if constexpr (EPI_TILES) {
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const v8 qv = *reinterpret_cast<const v8*>(sQe + (dt * 64 + lane) * 16 + h * 8);
-                    const v8 ov = *reinterpret_cast<const v8*>(sOe + (dt * 64 + lane) * 16 + h * 8);
+                    for (int h = 0; h < 2; ++h) {
+                        const v8 qv = *reinterpret_cast<const v8*>(sQe + (dt * 64 + lane) * 16 + h * 8);
+                        const v8 ov = *reinterpret_cast<const v8*>(sOe + (dt * 64 + lane) * 16 + h * 8);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        sk += accQ[dt][h * 8 + e] * (float)qv[e];
-                        sv += accT[dt][h * 8 + e] * (float)ov[e];
+                        for (int e = 0; e < 8; ++e) {
+                            sk += accQ[dt][h * 8 + e] * (float)qv[e];
+                            sv += accT[dt][h * 8 + e] * (float)ov[e];
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        sk += accQ[dt][i] * (float)sQb[c_row(g, i) * LDK + d];
+                        sv += accT[dt][i] * (float)sOb[c_row(g, i) * LDK + d];
                     }
                 }
                 sk += __shfl_xor(sk, 32, 64);
@@ -356,19 +391,23 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
     __syncthreads();
 
     if constexpr (WITH_DQ) {
-        // dQ: sum the pairs' slices; thread (wave, lane) owns accumulator registers 4*(wave%4) .. +3 of
-        // d-tile wave/4, i.e. four consecutive query rows of column d
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        // dQ: sum the pairs' slices; a thread takes four consecutive accumulator registers (= four consecutive
+        // query rows of one column) at a time
 #pragma unroll
-        for (int sl = 0; sl < NW / 2; ++sl) {
-            const float4 x = *reinterpret_cast<const float4*>(sDQall + sl * (BQ * DH) + (wave * 64 + lane) * 4);
-            v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
+        for (int t = 0; t < BQ * DH / 4 / NTH; ++t) {
+            const int idx4 = t * NTH + tid, slot4 = idx4 >> 6, ln = idx4 & 63;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int sl = 0; sl < NW / 2; ++sl) {
+                const float4 x = *reinterpret_cast<const float4*>(sDQall + sl * (BQ * DH) + idx4 * 4);
+                v.x += x.x; v.y += x.y; v.z += x.z; v.w += x.w;
+            }
+            const int d = c0 + (slot4 >> 2) * 32 + (ln & 31), r0 = c_row(ln >> 5, (slot4 & 3) * 4);
+            const float out[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (q0 + r0 + e < T) p.dq[base + (size_t)(q0 + r0 + e) * D + d] = (E)(out[e] * p.alpha);
         }
-        const int d = c0 + (wave >> 2) * 32 + n, r0 = c_row(g, (wave & 3) * 4);
-        const float out[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (q0 + r0 + e < T) p.dq[base + (size_t)(q0 + r0 + e) * D + d] = (E)(out[e] * p.alpha);
     }
 }
 

@@ -233,9 +233,12 @@ def test_mfma_backward_bf16(seq_len, causal):
 
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("seq_len", [1, 33, 100, 256, 300])
-def test_mfma_backward_d128_bf16(seq_len, causal):
-    """Head dimension 128: the backward kernel that produces the gradient columns in two halves."""
-    print(f"case mfma bwd D=128 T={seq_len} causal={causal}", flush=True)
+@pytest.mark.parametrize("shape", ["w4", "w8"])
+def test_mfma_backward_d128_bf16(seq_len, causal, shape, monkeypatch):
+    """Head dimension 128, both workgroup shapes of the backward kernel (one wave per SIMD with all
+    128 gradient columns / two waves per SIMD with one half of them)."""
+    print(f"case mfma bwd D=128 T={seq_len} causal={causal} shape={shape}", flush=True)
+    monkeypatch.setenv("TRITT_BWD128_VARIANT", shape)
     inputs = orc.make_inputs(1, 3, seq_len, 128, torch.bfloat16, seed=seq_len + 7)
     alpha = 1 / math.sqrt(128)
     z, _, grads = util.oracle_tdp(inputs, alpha, causal)
