@@ -114,14 +114,36 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
         for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
     float m = -INFINITY, l = 0.f;
 
-    for (int t = a_lo / 32 + wave; t <= a_hi / 32; t += kW) {
+    // Operands of a streamed tile are fetched one tile ahead, into the registers the previous tile has
+    // just consumed (each wave runs only a handful of tiles, so two dependent global round trips per
+    // tile would be most of its time).
+    v8 kn[KS], vn[DT][2];
+    auto fetch_k = [&](int t) {
+        const E* krow = K + (size_t)min(t * 32 + key_of_row(n), T - 1) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kn[ks] = ld8<E>(krow + 16 * ks);
+    };
+    auto fetch_v = [&](int t) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+                vn[dt][kk] = ld8<E>(VT + (size_t)(32 * dt + n) * Tp + t * 32 + 16 * kk + 8 * g);
+    };
+    const int t_first = a_lo / 32 + wave, t_last = a_hi / 32;
+    if (t_first <= t_last) {
+        fetch_k(t_first);
+        fetch_v(t_first);
+    }
+    for (int t = t_first; t <= t_last; t += kW) {
         const int a0 = t * 32;
+        const bool more = t + kW <= t_last;
         f32x16 s;
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = 0.f;
-        const E* krow = K + (size_t)min(a0 + key_of_row(n), T - 1) * D + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = M::mma(ld8<E>(krow + 16 * ks), xb[ks], s);
+        for (int ks = 0; ks < KS; ++ks) s = M::mma(kn[ks], xb[ks], s);
+        if (more) fetch_k(t + kW);
         float b[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) b[i] = 0.f;
@@ -164,7 +186,8 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
-                acc[dt] = M::mma(ld8<E>(VT + (size_t)(32 * dt + n) * Tp + a0 + 16 * kk + 8 * g), pb[kk], acc[dt]);
+                acc[dt] = M::mma(vn[dt][kk], pb[kk], acc[dt]);
+        if (more) fetch_v(t + kW);
     }
     l += __shfl_xor(l, 32, 64);
 
