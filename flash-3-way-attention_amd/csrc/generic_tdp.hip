@@ -53,6 +53,30 @@ __device__ __forceinline__ void axpy_lds(float (&acc)[D], float p, const float* 
     }
 }
 
+// The backward kernels hold four D-vectors per virtual row; beyond D = 64 that no longer fits one
+// lane's registers, so a row is shared by LP = D/64 lanes, each owning DL = D/LP consecutive
+// columns: a wave then sweeps RPT = 64/LP rows at a time and the two partial dot products of a
+// row meet through one cross-lane add.
+template <int D>
+struct RowSplit {
+    static constexpr int LP = D > 64 ? D / 64 : 1;
+    static constexpr int DL = D / LP;
+    static constexpr int RPT = 64 / LP;
+    static_assert(LP <= 2, "one or two lanes per row");
+};
+// sum over the lanes that hold the same column part (all 64, or the 32 of one half)
+template <int LP>
+__device__ __forceinline__ float part_sum(float v) {
+#pragma unroll
+    for (int off = 32 / LP; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+template <int LP>
+__device__ __forceinline__ float join_parts(float v) {
+    if constexpr (LP == 2) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
 // ------------------------------------------------------------------------------------------
 // Forward.  grid = (ceil(T/4), BH), 256 threads: wave w owns query q = 4*blockIdx.x + w, its
 // lanes sweep the owner index b (K2/V2 rows) in tiles of 64; staged index a = K1/U rows.
@@ -165,15 +189,19 @@ __global__ __launch_bounds__(256) void tdp_bwd_q_generic_kernel(
     const float scale_log2 = alpha * kLog2e;
     const float lse2 = LSE[qc] * kLog2e, delta = Delta[qc];
 
-    float o0 = 0.f, o1 = 0.f;
-    for (int b0 = b_lo & ~63; b0 <= b_hi; b0 += 64) {
-        const int b = b0 + lane, bc = min(b, T - 1);
-        float qb[D], gb[D], acc[D];
+    using RS = RowSplit<D>;
+    constexpr int LP = RS::LP, DL = RS::DL, RPT = RS::RPT;
+    const int lrow = lane % RPT, c0 = (lane / RPT) * DL;  // this lane's row of a tile and its first column
+
+    float o0 = 0.f, o1 = 0.f;  // dQ[q][c0 + lrow] and dQ[q][c0 + lrow + RPT]
+    for (int b0 = b_lo & ~(RPT - 1); b0 <= b_hi; b0 += RPT) {
+        const int b = b0 + lrow, bc = min(b, T - 1);
+        float qb[DL], gb[DL], acc[DL];
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const float kb = KB[(size_t)bc * D + d];
-            qb[d] = Q[(size_t)qc * D + d] * kb * scale_log2;
-            gb[d] = dO[(size_t)qc * D + d] * VB[(size_t)bc * D + d];
+        for (int d = 0; d < DL; ++d) {
+            const float kb = KB[(size_t)bc * D + c0 + d];
+            qb[d] = Q[(size_t)qc * D + c0 + d] * kb * scale_log2;
+            gb[d] = dO[(size_t)qc * D + c0 + d] * VB[(size_t)bc * D + c0 + d];
             acc[d] = 0.f;
         }
         for (int a0 = a_lo & ~(kStageRows - 1); a0 <= a_hi; a0 += kStageRows) {
@@ -184,28 +212,28 @@ __global__ __launch_bounds__(256) void tdp_bwd_q_generic_kernel(
             const int n = min(kStageRows, a_hi - a0 + 1);
             for (int aa = 0; aa < n; ++aa) {
                 const int a = a0 + aa;
-                const bool ok = q_ok && b < T && tdp_valid(mask, q, a, b);
+                const bool ok = q_ok && b < T && tdp_valid(mask, q, a, b);  // the same for the lanes of a row
                 if (ok) {
-                    const float s = dot_lds<D>(qb, sK[aa]);
-                    const float dp = dot_lds<D>(gb, sV[aa]);
+                    const float s = join_parts<LP>(dot_lds<DL>(qb, sK[aa] + c0));
+                    const float dp = join_parts<LP>(dot_lds<DL>(gb, sV[aa] + c0));
                     const float ds = fast_exp2(s - lse2) * (dp - delta);
-                    axpy_lds<D>(acc, ds, sK[aa]);
+                    axpy_lds<DL>(acc, ds, sK[aa] + c0);
                 }
             }
         }
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const float t = wave_sum(acc[d] * KB[(size_t)bc * D + d]);
-            if (d < 64) {
-                o0 = (lane == d) ? o0 + t : o0;
+        for (int d = 0; d < DL; ++d) {
+            const float t = part_sum<LP>(acc[d] * KB[(size_t)bc * D + c0 + d]);
+            if (d < RPT) {
+                o0 = (lrow == d) ? o0 + t : o0;
             } else {
-                o1 = (lane == d - 64) ? o1 + t : o1;
+                o1 = (lrow == d - RPT) ? o1 + t : o1;
             }
         }
     }
     if (q_ok) {
-        if (lane < D) dQ[(size_t)q * D + lane] = o0 * alpha;
-        if (D > 64 && lane + 64 < D) dQ[(size_t)q * D + lane + 64] = o1 * alpha;
+        if (lrow < DL) dQ[(size_t)q * D + c0 + lrow] = o0 * alpha;
+        if (DL > RPT) dQ[(size_t)q * D + c0 + lrow + RPT] = o1 * alpha;
     }
 }
 
@@ -237,18 +265,22 @@ __global__ __launch_bounds__(256) void tdp_bwd_b_generic_kernel(
     const int q_hi = mask.causal ? min(T - 1, b_hi + mask.wb) : T - 1;
     const float scale_log2 = alpha * kLog2e;
 
-    float k0 = 0.f, k1 = 0.f, v0 = 0.f, v1 = 0.f;
-    for (int q0 = q_lo & ~63; q0 <= q_hi; q0 += 64) {
-        const int q = q0 + lane, qc = min(q, T - 1);
-        const int qt_hi = min(q_hi, q0 + 63);
+    using RS = RowSplit<D>;
+    constexpr int LP = RS::LP, DL = RS::DL, RPT = RS::RPT;
+    const int lrow = lane % RPT, c0 = (lane / RPT) * DL;
+
+    float k0 = 0.f, k1 = 0.f, v0 = 0.f, v1 = 0.f;  // columns c0 + lrow and c0 + lrow + RPT of dKB[b], dVB[b]
+    for (int q0 = q_lo & ~(RPT - 1); q0 <= q_hi; q0 += RPT) {
+        const int q = q0 + lrow, qc = min(q, T - 1);
+        const int qt_hi = min(q_hi, q0 + RPT - 1);
         const int a_lo = mask.causal ? max(0, max(q0, q_lo) - mask.wa) : 0;
         const int a_hi = mask.causal ? qt_hi : T - 1;
         const float lse2 = LSE[qc] * kLog2e, delta = Delta[qc];
-        float qb[D], gb[D], accK[D], accV[D];
+        float qb[DL], gb[DL], accK[DL], accV[DL];
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            qb[d] = Q[(size_t)qc * D + d] * KB[(size_t)bc * D + d] * scale_log2;
-            gb[d] = dO[(size_t)qc * D + d] * VB[(size_t)bc * D + d];
+        for (int d = 0; d < DL; ++d) {
+            qb[d] = Q[(size_t)qc * D + c0 + d] * KB[(size_t)bc * D + c0 + d] * scale_log2;
+            gb[d] = dO[(size_t)qc * D + c0 + d] * VB[(size_t)bc * D + c0 + d];
             accK[d] = 0.f;
             accV[d] = 0.f;
         }
@@ -260,37 +292,37 @@ __global__ __launch_bounds__(256) void tdp_bwd_b_generic_kernel(
             const int n = min(kStageRows, a_hi - a0 + 1);
             for (int aa = 0; aa < n; ++aa) {
                 const int a = a0 + aa;
-                const bool ok = b_ok && q < T && q >= q_lo && tdp_valid(mask, q, a, b);
+                const bool ok = b_ok && q < T && q >= q_lo && tdp_valid(mask, q, a, b);  // the same for the lanes of a row
                 if (ok) {
-                    const float s = dot_lds<D>(qb, sK[aa]);
-                    const float dp = dot_lds<D>(gb, sV[aa]);
+                    const float s = join_parts<LP>(dot_lds<DL>(qb, sK[aa] + c0));
+                    const float dp = join_parts<LP>(dot_lds<DL>(gb, sV[aa] + c0));
                     const float p = fast_exp2(s - lse2);
-                    axpy_lds<D>(accK, p * (dp - delta), sK[aa]);
-                    axpy_lds<D>(accV, p, sV[aa]);
+                    axpy_lds<DL>(accK, p * (dp - delta), sK[aa] + c0);
+                    axpy_lds<DL>(accV, p, sV[aa] + c0);
                 }
             }
         }
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const float tk = wave_sum(accK[d] * Q[(size_t)qc * D + d]);
-            const float tv = wave_sum(accV[d] * dO[(size_t)qc * D + d]);
-            if (d < 64) {
-                k0 = (lane == d) ? k0 + tk : k0;
-                v0 = (lane == d) ? v0 + tv : v0;
+        for (int d = 0; d < DL; ++d) {
+            const float tk = part_sum<LP>(accK[d] * Q[(size_t)qc * D + c0 + d]);
+            const float tv = part_sum<LP>(accV[d] * dO[(size_t)qc * D + c0 + d]);
+            if (d < RPT) {
+                k0 = (lrow == d) ? k0 + tk : k0;
+                v0 = (lrow == d) ? v0 + tv : v0;
             } else {
-                k1 = (lane == d - 64) ? k1 + tk : k1;
-                v1 = (lane == d - 64) ? v1 + tv : v1;
+                k1 = (lrow == d - RPT) ? k1 + tk : k1;
+                v1 = (lrow == d - RPT) ? v1 + tv : v1;
             }
         }
     }
     if (b_ok) {
-        if (lane < D) {
-            dKB[(size_t)b * D + lane] = k0 * alpha;
-            dVB[(size_t)b * D + lane] = v0;
+        if (lrow < DL) {
+            dKB[(size_t)b * D + c0 + lrow] = k0 * alpha;
+            dVB[(size_t)b * D + c0 + lrow] = v0;
         }
-        if (D > 64 && lane + 64 < D) {
-            dKB[(size_t)b * D + lane + 64] = k1 * alpha;
-            dVB[(size_t)b * D + lane + 64] = v1;
+        if (DL > RPT) {
+            dKB[(size_t)b * D + c0 + lrow + RPT] = k1 * alpha;
+            dVB[(size_t)b * D + c0 + lrow + RPT] = v1;
         }
     }
 }
