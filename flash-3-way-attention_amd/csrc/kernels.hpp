@@ -48,6 +48,8 @@ struct MfmaFwdArgs {
     float alpha;
     int causal;
     int is_bf16;  // else fp16
+    int windowed;  // some window can exclude a pair with j, k <= q: the banded instantiation
+    int k1_window, k2_window, kk_left, kk_right;
 };
 size_t mfma_tdp_fwd_workspace(int BH, int T, int D);
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit);

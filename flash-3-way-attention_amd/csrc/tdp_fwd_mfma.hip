@@ -39,12 +39,18 @@ struct FwdParams {
     int T, Tp, BH, nqt;
     float scale_log2;
     int causal;
+    // windowed instantiation only: (q, j, k) takes part iff j <= q, k <= q, q - j <= wa, q - k <= wb,
+    // k - j <= lab, j - k <= rab
+    int wa, wb, lab, rab;
 };
 
 constexpr float kLazyThreshold = 8.0f;
 
 // MINW (second launch-bounds argument): waves per SIMD the register allocator must leave room for
-template <typename E, int D, int NT, int WAVES, int MINW, int JS>
+// WIN: windowed causal masks.  The k-tile and stage loops run over the band only, every step goes
+// through the general (per tile, element-wise masked) loop, and the CAREFUL sweep tolerates rows whose
+// first valid key comes late.
+template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false>
 __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -93,6 +99,12 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     const int q0 = qt * BQ;
     const int jend = p.causal ? min(T - 1, q0 + BQ - 1) : T - 1;  // last key any query here needs
     const int nst = jend / JS + 1, nkt = jend / 32 + 1;
+    // WIN: the first k-tile any query here can use (k >= q - wb, and some j with q - wa <= j <= k + rab),
+    // and per k-tile the stages that hold keys j any (q, k) of it can use
+    const bool banded = WIN && p.causal;
+    const int kt_lo = banded ? max(0, max(q0 - p.wb, q0 - p.wa - p.rab)) / 32 : 0;
+    auto first_stage = [&](int kt) { return banded ? max(0, max(q0 - p.wa, kt * 32 - p.lab)) / JS : 0; };
+    auto last_stage = [&](int kt) { return banded ? min(jend, kt * 32 + 31 + p.rab) / JS : nst - 1; };
 
     int qrow[NT], jmax[NT];
 #pragma unroll
@@ -195,8 +207,8 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
         sQ[r * LDQ + d] = (float)Q[(size_t)min(q0 + r, T - 1) * D + d] * p.scale_log2;
     }
     if (tid == 0) *sFlag = 0;
-    issue_ktile(0);
-    issue_stage(0);
+    issue_ktile(kt_lo);
+    issue_stage(first_stage(kt_lo));
     commit_ktile(0);
     commit_stage(0);
     __syncthreads();
@@ -213,8 +225,23 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     const int krow_off = key_of_row(n);  // K1 row (within a 32-key step) this lane feeds to the MFMA
 
     int gstage = 0;  // running stage counter (buffer = gstage & 1)
-    for (int kt = 0; kt < nkt; ++kt) {
-        const int kb = kt & 1;
+    for (int kt = kt_lo; kt < nkt; ++kt) {
+        const int kb = (kt - kt_lo) & 1;
+        const int st_lo = first_stage(kt), st_hi = last_stage(kt);
+        // the stage fetched after the last one: the next k-tile starts from it (or a repeat of this one)
+        const int st_next = kt + 1 < nkt ? first_stage(kt + 1) : st_lo;
+        // per-lane window of keys j for the virtual row (q, k = 32 kt + n); hi < lo: the row is empty
+        [[maybe_unused]] int wlo[NT], whi[NT];
+        if constexpr (WIN) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int k = kt * 32 + n, q = qrow[t];
+                wlo[t] = banded ? max(q - p.wa, k - p.lab) : 0;
+                whi[t] = banded ? min(jmax[t], k + p.rab) : jmax[t];
+                if (k > jmax[t] || (banded && q > k + p.wb)) whi[t] = -1;
+                if (whi[t] < wlo[t]) { wlo[t] = 0; whi[t] = -1; }
+            }
+        }
 
         // B operands: QK2[(q, k), d] = Q[q,d] * K2[k,d] * alpha*log2(e), k = 32*kt + n
         v8 bq[NT][KS];
@@ -255,8 +282,11 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[t][dt][i] = 0.f;
             }
-            int st = 0;
-            if constexpr (NT == 2 && !CAREFUL) {
+            int st = st_lo;
+            [[maybe_unused]] bool started[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) started[t] = false;
+            if constexpr (NT == 2 && !CAREFUL && !WIN) {
                 // Stages whose 64 keys lie inside the causal bound of both tiles of this wave: a loop
                 // without branches on tile validity, so the accumulators stay in place (no copies
                 // at control-flow joins) and the wave itself overlaps matrix and vector work.  The
@@ -359,7 +389,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     __syncthreads();
                 }
             }
-            if constexpr (NT == 1 && !CAREFUL) {
+            if constexpr (NT == 1 && !CAREFUL && !WIN) {
                 // The same for one tile per wave (D = 128: two tiles do not fit the register file).
                 // The two 32-key steps of a stage play the part of the two tiles: the score product
                 // of the second step is issued between the exp2 / pack work of the first, the value
@@ -436,13 +466,13 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     __syncthreads();
                 }
             }
-            for (; st < nst; ++st, ++gstage) {
+            for (; st <= st_hi; ++st, ++gstage) {
                 const int sb = gstage & 1;
-                // stage 0 is fetched again after the last stage: the next k-tile, or a CAREFUL repeat
-                // of this one, starts from it
-                const bool more = (st + 1 < nst) || (kt + 1 < nkt) || !CAREFUL;
-                if (more) issue_stage(st + 1 < nst ? st + 1 : 0);
-                if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
+                // the first stage is fetched again after the last one: the next k-tile, or a CAREFUL
+                // repeat of this one, starts from it
+                const bool more = (st < st_hi) || (kt + 1 < nkt) || !CAREFUL;
+                if (more) issue_stage(st < st_hi ? st + 1 : st_next);
+                if (st == st_lo && kt + 1 < nkt) issue_ktile(kt + 1);
 
 #pragma unroll
                 for (int half = 0; half < JS / 32; ++half) {
@@ -455,17 +485,62 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
                     for (int t = 0; t < NT; ++t) {
                         if (jb > jmax[t]) continue;  // tile entirely above the causal bound (wave-uniform)
+                        bool inside = true;  // WIN: every (j, k) of this step is valid for the query
+                        if constexpr (WIN) {
+                            if (banded) {
+                                const int q = qrow[t], k0 = kt * 32;
+                                // no k of the tile, or no j of the step, is inside the band of this query
+                                if (k0 > jmax[t] || q > k0 + 31 + p.wb) continue;
+                                if (jb > min(jmax[t], k0 + 31 + p.rab) || jb + 31 < max(q - p.wa, k0 - p.lab)) continue;
+                                inside = (k0 + 31 <= jmax[t]) && (q <= k0 + p.wb) && (jb >= max(q - p.wa, k0 + 31 - p.lab)) &&
+                                         (jb + 31 <= min(jmax[t], k0 + p.rab));
+                            } else {
+                                inside = jb + 31 <= jmax[t];
+                            }
+                        }
                         f32x16 s;
 #pragma unroll
                         for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
                         for (int ks = 0; ks < KS; ++ks)
                             s = M::mma(*reinterpret_cast<const v8*>(k1p + ks * 16), bq[t][ks], s);
-                        if (jb + 31 > jmax[t]) {
+                        if constexpr (WIN) {
+                            if (!inside) {
+#pragma unroll
+                                for (int i = 0; i < 16; ++i) {
+                                    const int j = jb + key_of(g, i);
+                                    s[i] = (j >= wlo[t] && j <= whi[t]) ? s[i] : -INFINITY;
+                                }
+                            }
+                        } else if (jb + 31 > jmax[t]) {
 #pragma unroll
                             for (int i = 0; i < 16; ++i) s[i] = (jb + key_of(g, i) <= jmax[t]) ? s[i] : -INFINITY;
                         }
-                        if constexpr (CAREFUL) {
+                        if constexpr (CAREFUL && WIN) {
+                            // as below, but a row may have seen no valid key yet: its reference then sits at
+                            // a finite floor, and the reference is assigned, not incremented (floor + step
+                            // would round the step away)
+                            float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+                            for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
+                            const bool begin = !started[t];
+                            started[t] = true;
+                            if (begin || __any(mx - mref[t] > kLazyThreshold)) {
+                                const float rmax = fmaxf(fmaxf(mx, __shfl_xor(mx, 32, 64)), -1.0e30f);
+                                const float newref = begin ? rmax : fmaxf(rmax, mref[t]);
+                                const float f = fast_exp2(mref[t] - newref);
+                                mref[t] = newref;
+                                if (!begin) {
+                                    lsum[t] *= f;
+                                    float fr[16];
+                                    rows_of(f, fr);
+#pragma unroll
+                                    for (int i = 0; i < 16; ++i)
+#pragma unroll
+                                        for (int dt = 0; dt < DT; ++dt) acc[t][dt][i] *= fr[i];
+                                }
+                            }
+                        } else if constexpr (CAREFUL) {
                             float mx = fmaxf(s[0], s[1]);
 #pragma unroll
                             for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
@@ -529,7 +604,8 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) mag += fabsf(acc[t][dt][i]);
-                const bool kval = (kt * 32 + n) <= jmax[t];
+                bool kval = (kt * 32 + n) <= jmax[t];
+                if constexpr (WIN) kval = whi[t] >= 0;
                 bad |= (kval && !(lk > 1e-30f && lk < 1e30f)) || !(mag < 1e30f);
             }
             if (__any(bad) && lane == 0) *sFlag = 1;
@@ -538,6 +614,13 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
             __syncthreads();
             if (redo) {
                 if (tid == 0) *sFlag = 0;
+                if constexpr (WIN) {
+                    if (st_next != st_lo) {  // the stage fetched ahead belongs to the next k-tile: fetch this one's
+                        issue_stage(st_lo);
+                        commit_stage(gstage & 1);
+                        __syncthreads();
+                    }
+                }
                 sweep(std::true_type{});
             }
         }
@@ -546,12 +629,14 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const float lk = lsum[t] + __shfl_xor(lsum[t], 32, 64);
-            const bool kval = (kt * 32 + n) <= jmax[t];
+            bool kval = (kt * 32 + n) <= jmax[t];
+            if constexpr (WIN) kval = whi[t] >= 0;
             float mt = kval ? mref[t] : -INFINITY;
 #pragma unroll
             for (int off = 16; off > 0; off >>= 1) mt = fmaxf(mt, __shfl_xor(mt, off, 64));
             const float mnew = fmaxf(Mrun[t], mt);
-            const float f = fast_exp2(Mrun[t] - mnew);
+            // WIN: the first k-tiles of the band can hold no valid row for this query yet
+            const float f = (WIN && mnew == -INFINITY) ? 1.f : fast_exp2(Mrun[t] - mnew);
             const float w = kval ? fast_exp2(mref[t] - mnew) : 0.f;
             float wl = w * lk;
 #pragma unroll
@@ -613,7 +698,7 @@ constexpr size_t fwd_smem_bytes() {
 
 constexpr int kTpad = 128;  // U^T rows are padded to a multiple of the largest stage
 
-template <typename E, int D, int NT, int WAVES, int MINW, int JS>
+template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false>
 static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
@@ -625,8 +710,9 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + BQ - 1) / BQ;
     p.scale_log2 = a.alpha * kLog2e;
     p.causal = a.causal;
+    p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
     constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS>();
-    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS>;
+    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN>;
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -672,6 +758,17 @@ static hipError_t launch_d64(const MfmaFwdArgs& a, hipStream_t st) {
 }
 
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
+    if (a.windowed) {
+        // one tile per wave; D = 64 with four waves per SIMD (the general loop has no interleave of its own)
+        if (a.is_bf16) {
+            if (a.D == 64) return launch<__bf16, 64, 1, 16, 4, 64, true>(a, st);
+            if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64, true>(a, st);
+        } else {
+            if (a.D == 64) return launch<_Float16, 64, 1, 16, 4, 64, true>(a, st);
+            if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64, true>(a, st);
+        }
+        return hipErrorInvalidValue;
+    }
     if (a.is_bf16) {
         if (a.D == 64) return launch_d64<__bf16>(a, st);
         if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64>(a, st);
