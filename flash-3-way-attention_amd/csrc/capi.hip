@@ -261,7 +261,8 @@ bool use_mfma_fwd(int T, int D, int dtype, int causal, int w1, int w2, int kl, i
 
 bool use_mfma_bwd(int T, int D, int dtype, int causal, int w1, int w2, int kl, int kr, unsigned flags) {
     if (flags & TRITT_FLAG_FORCE_GENERIC) return false;
-    return mfma_tdp_bwd_supported(D, dtype != TRITT_F32) && full_windows(T, causal, w1, w2, kl, kr);
+    (void)T; (void)causal; (void)w1; (void)w2; (void)kl; (void)kr;  // any mask: windows take the banded kernels
+    return mfma_tdp_bwd_supported(D, dtype != TRITT_F32);
 }
 
 bool use_mfma_dps(int D, int dtype, unsigned flags) {
@@ -366,6 +367,8 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
         a.dq = dq; a.dk1 = dk1; a.dk2 = dk2; a.dv1 = dv1; a.dv2 = dv2; a.workspace = workspace;
         a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0;
         a.is_bf16 = dtype == TRITT_BF16;
+        a.windowed = full_windows(T, causal, w1, w2, kl, kr) ? 0 : 1;
+        a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
         return (int)mfma_tdp_bwd(a, (hipStream_t)stream);
     }
     Arena ar(workspace);

@@ -55,7 +55,7 @@ size_t mfma_tdp_fwd_workspace(int BH, int T, int D);
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st);
 
-// 16-bit MFMA triple-dot backward (full causal windows or no mask; D = 64).
+// 16-bit MFMA triple-dot backward (D = 64 or 128).
 struct MfmaBwdArgs {
     const void *q, *k1, *k2, *v1, *v2, *o, *d_o;
     const float* lse;
@@ -65,6 +65,8 @@ struct MfmaBwdArgs {
     float alpha;
     int causal;
     int is_bf16;
+    int windowed;  // some window can exclude a pair with j, k <= q: the banded kernels
+    int k1_window, k2_window, kk_left, kk_right;
 };
 size_t mfma_tdp_bwd_workspace(int BH, int T, int D);
 bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit);

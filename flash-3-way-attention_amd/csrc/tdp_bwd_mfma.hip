@@ -35,11 +35,14 @@ struct BwdParams {
     int T, Tp, BH, nqt;
     float alpha;
     int causal;
+    // windowed kernels only, in terms of the streamed index a and the row index b: (q, a, b) takes part
+    // iff a, b <= q, q - a <= wa, q - b <= wb, b - a <= lab, a - b <= rab
+    int wa, wb, lab, rab;
 };
 
 }  // namespace tritt
 
-#include "tdp_bwd_rows128.hpp"
+#include "tdp_bwd_rows_general.hpp"
 
 namespace tritt {
 
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     constexpr int LDK = D + 8, LDF = D + 4;
     constexpr int TILE = 64 * 64;
     constexpr int NBUF = 3, LW = 4;  // stage buffers; direct loads per wave per stage
-    static_assert(D == 64, "stages are four 64x64 tiles = 32 blocks of 1 KB, four per wave (D = 128: tdp_bwd_rows128_kernel)");
+    static_assert(D == 64, "stages are four 64x64 tiles = 32 blocks of 1 KB, four per wave (D = 128 and windowed masks: tdp_bwd_rows_general_kernel)");
 
     extern __shared__ __align__(16) char smem[];
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][4 tensors: K1, U, K1^T, U^T][TILE]
@@ -539,13 +542,18 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
 
-    // D = 64: three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO tiles (twice:
-    // operand and epilogue layout), four dQ slices.  D = 128: a workgroup per column half, see tdp_bwd_rows128.hpp
+    // D = 64, full windows: three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO
+    // tiles (twice: operand and epilogue layout), four dQ slices.  Otherwise: tdp_bwd_rows_general.hpp
     size_t smem;
     void (*kern_dq)(BwdParams<E>);
     void (*kern_nodq)(BwdParams<E>);
     int nthreads = 512, col_parts = 1;
-    if constexpr (D == 128) {
+    if (a.windowed) {
+        smem = bwdg_smem(D, 8, 64, true);
+        kern_dq = tdp_bwd_rows_general_kernel<E, D, true, 8, 64, true>;
+        kern_nodq = tdp_bwd_rows_general_kernel<E, D, false, 8, 64, true>;
+        col_parts = D / 64;
+    } else if constexpr (D == 128) {
         // One wave per SIMD with all 128 columns is ~10 % faster once the grid fills the chip several times
         // over; below that the smaller workgroups of the two-waves-per-SIMD shape balance better.
         // TRITT_BWD128_VARIANT=w8 / w4 overrides the choice (read at every call).
@@ -555,21 +563,21 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
             if (strcmp(v, "w4") == 0) w8 = false;
         }
         if (w8) {
-            smem = bwd128_smem(8, 64, true);
-            kern_dq = tdp_bwd_rows128_kernel<E, true, 8, 64>;
-            kern_nodq = tdp_bwd_rows128_kernel<E, false, 8, 64>;
+            smem = bwdg_smem(128, 8, 64, true);
+            kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 8, 64, false>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 128, false, 8, 64, false>;
             col_parts = 2;
         } else {
-            smem = bwd128_smem(4, 128, true);
-            kern_dq = tdp_bwd_rows128_kernel<E, true, 4, 128>;
-            kern_nodq = tdp_bwd_rows128_kernel<E, false, 4, 128>;
+            smem = bwdg_smem(128, 4, 128, true);
+            kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 4, 128, false>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 128, false, 4, 128, false>;
             nthreads = 256;
         }
     } else {
         smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8) + 2 * (D / 32) * 64 * 16) +
                4 * (size_t)(4 * 32 * D);
-        kern_dq = tdp_bwd_rows_kernel<E, D, true>;
-        kern_nodq = tdp_bwd_rows_kernel<E, D, false>;
+        kern_dq = tdp_bwd_rows_kernel<E, 64, true>;
+        kern_nodq = tdp_bwd_rows_kernel<E, 64, false>;
     }
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq),
@@ -585,11 +593,13 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
     p.acc_k = dk2acc; p.acc_v = dv2acc;
+    p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
     hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU
     p.row_k = (const E*)a.k1; p.row_v = u;
     p.st_k = (const E*)a.k2; p.st_v = (const E*)a.v2; p.st_kt = k2t; p.st_vt = v2t;
     p.acc_k = dk1acc; p.acc_v = duacc;
+    p.wa = a.k2_window; p.wb = a.k1_window; p.lab = a.kk_right; p.rab = a.kk_left;  // the mask with j and k exchanged
     hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
 
     const size_t n = (size_t)a.BH * a.T * D;

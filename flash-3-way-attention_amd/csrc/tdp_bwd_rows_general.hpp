@@ -1,9 +1,12 @@
-// Triple-dot-product trittention backward on MFMA, head dimension 128 (included by
-// tdp_bwd_mfma.hip after BwdParams).
+// Triple-dot-product trittention backward on MFMA: the general form of the rows kernel (included by
+// tdp_bwd_mfma.hip after BwdParams).  It serves head dimension 128 and, for head dimensions 64 and
+// 128, windowed causal masks (WIN): rounds and steps then cover the band only, and a key outside the
+// window of its (q, k) is masked like one past the causal bound.
 //
 // Same decomposition as tdp_bwd_rows_kernel (rows = one K2/V2 row k per wave and round, K1 / U
 // streamed over j, the columns of every tile = 32 queries).  The accumulators Yq / Tv of all 128
 // gradient columns are 128 registers, so there are two shapes:
+// For D = 128:
 //  * NW = 4 waves, NCOL = 128: one wave per SIMD with the whole 512-entry register file; a
 //    tile-step (32 keys) is 18 + 16 MFMAs;
 //  * NW = 8 waves, NCOL = 64: two waves per SIMD, a workgroup produces one half of the gradient
@@ -13,7 +16,8 @@
 // offset_operand) instead of two resident 16-register C tiles.  Stages are 32 keys: K1 and U rows
 // as 64 x 64 tiles (tile row = 32 * (d / 64) + key, the swizzle of direct_lds.hpp), K1^T and U^T
 // of the workgroup's columns as compact [NCOL d][32 keys] tiles; three buffers, fetched
-// direct-to-LDS two steps ahead, one workgroup barrier per step.
+// direct-to-LDS two steps ahead, one workgroup barrier per step.  D = 64 (WIN only; the full-window
+// case has its own kernel): NW = 8, NCOL = 64, the row tiles have 32 rows.
 #pragma once
 
 namespace tritt {
@@ -50,27 +54,29 @@ __device__ __forceinline__ typename Mma<E>::v8 offset_operand(float x, int g) {
 // share banks; 16-byte chunk c of row r sits at position c ^ swz_t(r)
 __device__ __forceinline__ constexpr int swz_t(int r) { return (r >> 2) & 3; }
 
-constexpr int bwd128_stage_bytes(int ncol) { return 16 * 1024 + 2 * ncol * 64; }
-constexpr size_t bwd128_smem(int nw, int ncol, bool with_dq) {
-    return 3 * (size_t)bwd128_stage_bytes(ncol)               // stage buffers
-           + 2 * (2 * nw * 128 * 2)                            // K2 / V2 rows of two rounds
-           + 2 * (32 * (128 + 8) * 2)                          // Q and dO tiles
-           + (with_dq ? (nw / 2) * (32 * ncol * 4) : 0)        // dQ slices (one per pair of waves)
-           + (ncol == 64 ? 2 * (2 * 64 * 16 * 2) : 0);         // Q and dO in accumulator layout (NCOL = 64)
+constexpr int bwdg_stage_bytes(int d, int ncol) { return 2 * d * 64 + 2 * ncol * 64; }
+constexpr size_t bwdg_smem(int d, int nw, int ncol, bool with_dq) {
+    return 3 * (size_t)bwdg_stage_bytes(d, ncol)               // stage buffers
+           + 2 * (2 * nw * d * 2)                               // K2 / V2 rows of two rounds
+           + 2 * (32 * (d + 8) * 2)                             // Q and dO tiles
+           + (with_dq ? (nw / 2) * (32 * ncol * 4) : 0)         // dQ slices (one per pair of waves)
+           + (ncol == 64 ? 2 * (2 * 64 * 16 * 2) : 0);          // Q and dO in accumulator layout (NCOL = 64)
 }
 
-template <typename E, bool WITH_DQ, int NW, int NCOL>
-__global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p) {
+template <typename E, int D, bool WITH_DQ, int NW, int NCOL, bool WIN>
+__global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using v2 = typename M::v2;
-    constexpr int D = 128, KS = 8, DT = NCOL / 32, DH = NCOL, BQ = 32, NTH = 64 * NW;
+    constexpr int KS = D / 16, DT = NCOL / 32, DH = NCOL, BQ = 32, NTH = 64 * NW;
     constexpr int LDK = D + 8;
-    constexpr int NBLK = 16 + NCOL / 8;      // 1 KB blocks of a stage: 8 + 8 row-major, NCOL/16 + NCOL/16 transposed
+    constexpr int RB = D / 16;               // 1 KB blocks of a row-major stage tile (32 keys x D)
+    constexpr int NBLK = 2 * RB + NCOL / 8;  // blocks of a stage: K1 rows, U rows, NCOL/16 + NCOL/16 transposed
     constexpr int NBUF = 3, LW = NBLK / NW;  // stage buffers; direct loads per wave per stage
-    constexpr int STAGE = bwd128_stage_bytes(NCOL) / 2;  // elements
+    constexpr int STAGE = bwdg_stage_bytes(D, NCOL) / 2;  // elements
     constexpr bool EPI_TILES = NCOL == 64;   // Q / dO kept a second time in accumulator layout
-    static_assert((NW == 8 && NCOL == 64) || (NW == 4 && NCOL == 128), "two shapes");
+    static_assert(D == 64 || D == 128, "head dimension");
+    static_assert((NW == 8 && NCOL == 64) || (D == 128 && NW == 4 && NCOL == 128), "workgroup shapes");
     static_assert(NBLK % NW == 0, "whole blocks per wave");
 
     extern __shared__ __align__(16) char smem[];
@@ -108,14 +114,21 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
     const int jend = p.causal ? qlast : T - 1;
     const int jfull = p.causal ? q0 : T - 1;
     const int nsteps = jend / 32 + 1, nrounds = jend / NW + 1;
+    // WIN, with a = streamed index (j), b = row index (k):  (q, a, b) takes part iff a, b <= q,
+    // q - a <= wa, q - b <= wb, b - a <= lab, a - b <= rab.  Rows below b_first are outside the band
+    // of every query here; a round's sweep over a covers step_lo(m) .. step_hi(m) (never empty).
+    const bool banded = WIN && p.causal;
+    const int m_first = banded ? max(0, max(q0 - p.wb, q0 - p.wa - p.rab)) / NW : 0;
+    auto step_lo = [&](int m) { return banded ? max(0, max(q0 - p.wa, m * NW - p.lab)) / 32 : 0; };
+    auto step_hi = [&](int m) { return banded ? min(jend, m * NW + NW - 1 + p.rab) / 32 : nsteps - 1; };
     const int q = q0 + n;
     const bool q_ok = q < T;
     const int jq = p.causal ? min(q, T - 1) : T - 1;
     const float scale_log2 = p.alpha * kLog2e;
 
     // ---- stage loader: NBLK blocks of 1 KB, wave w fetches blocks LW w .. LW w + LW - 1
-    //   blocks 0..7 K1 rows, 8..15 U rows (tile rows 8b .. 8b+7), then NCOL/16 blocks of K1^T and as many of
-    //   U^T (16 d-rows each)
+    //   RB blocks of K1 rows, RB of U rows (tile rows 8b .. 8b+7), then NCOL/16 blocks of K1^T and as many
+    //   of U^T (16 d-rows each)
     const E* gsrc[LW];
     unsigned goff[LW];     // per-lane byte offset at key 0
     unsigned gstep[LW];    // bytes per key
@@ -124,18 +137,18 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
 #pragma unroll
     for (int c = 0; c < LW; ++c) {
         const int b = wave * LW + c;
-        if (b < 16) {
-            const int R = (b & 7) * 8 + (lane >> 3), hh = R >> 5, r = R & 31;
+        if (b < 2 * RB) {
+            const int R = (b % RB) * 8 + (lane >> 3), hh = R >> 5, r = R & 31;
             const int chunk = (lane & 7) ^ swz_perm(r);
-            gsrc[c] = uniform_ptr((b < 8 ? p.st_k : p.st_v) + base);
+            gsrc[c] = uniform_ptr((b < RB ? p.st_k : p.st_v) + base);
             rowkey[c] = r;
             rowrest[c] = (unsigned)(hh * 64 + chunk * 8) * 2;
             goff[c] = (unsigned)r * (D * 2) + rowrest[c];
             gstep[c] = D * 2;
         } else {
-            const int dl = ((b - 16) % (NCOL / 16)) * 16 + (lane >> 2);
+            const int dl = ((b - 2 * RB) % (NCOL / 16)) * 16 + (lane >> 2);
             const int chunk = (lane & 3) ^ swz_t(dl);
-            gsrc[c] = uniform_ptr((b < 16 + NCOL / 16 ? p.st_kt : p.st_vt) + tbase);
+            gsrc[c] = uniform_ptr((b < 2 * RB + NCOL / 16 ? p.st_kt : p.st_vt) + tbase);
             rowkey[c] = -1;
             rowrest[c] = 0;
             goff[c] = ((unsigned)(c0 + dl) * p.Tp + chunk * 8) * 2;
@@ -153,16 +166,18 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
             direct_load_16(gsrc[c], off, dst + c * 1024);
         }
     };
-    // the round's K2 / V2 rows NW m .. NW m + NW - 1: one load moves four rows (1 KB)
+    // the round's K2 / V2 rows NW m .. NW m + NW - 1: one load moves 1 KB = RPL rows
     auto issue_round = [&](int m, int buf) {
-        constexpr int LR = NW / 4;  // loads per tensor
+        constexpr int RPL = 512 / D, LPR = D / 8;  // rows per load, lanes per row
+        constexpr int LR = NW / RPL;               // loads per tensor
+        static_assert(LR >= 1 && 2 * LR <= NW, "round loader");
         if (wave < 2 * LR) {
             int ln = lane;
             asm volatile("" : "+v"(ln));
             const int part = wave % LR;
             const bool second = wave >= LR;
-            const unsigned off = (unsigned)min(m * NW + part * 4 + (ln >> 4), T - 1) * (D * 2) + (ln & 15) * 16;
-            direct_load_16(uniform_ptr(second ? V2 : K2), off, (second ? sVr : sKr) + buf * NW * D + part * 4 * D);
+            const unsigned off = (unsigned)min(m * NW + part * RPL + ln / LPR, T - 1) * (D * 2) + (ln % LPR) * 16;
+            direct_load_16(uniform_ptr(second ? V2 : K2), off, (second ? sVr : sKr) + buf * NW * D + part * RPL * D);
         }
     };
 
@@ -184,10 +199,22 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
     if constexpr (WITH_DQ) {
         for (int idx = tid; idx < (NW / 2) * BQ * DH; idx += NTH) sDQall[idx] = 0.f;
     }
-    issue_round(0, 0);
-    issue_stage(0, 0);
-    issue_stage(1 % nsteps, 1);
-    int st_ahead = 2 % nsteps;  // stage number of running index gstage + 2 (the j sweep repeats every round)
+    // (round, step) of the stage fetched next: the sequence the main loop walks, wrapping to the first
+    // round after the last (those fetches are never used)
+    int m_ahead = m_first, st_ahead = step_lo(m_first);
+    auto advance = [&]() {
+        if (st_ahead < step_hi(m_ahead)) {
+            ++st_ahead;
+        } else {
+            m_ahead = m_ahead + 1 < nrounds ? m_ahead + 1 : m_first;
+            st_ahead = step_lo(m_ahead);
+        }
+    };
+    issue_round(m_first, m_first & 1);
+    issue_stage(st_ahead, 0);
+    advance();
+    issue_stage(st_ahead, 1);
+    advance();
     int gstage = 0;
 
     const float lse2 = q_ok ? p.lse[(size_t)bh * T + q] * kLog2e : 3.0e4f;
@@ -197,9 +224,18 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
     const int krow_off = key_of_row(n);
     const int fperm = swz_perm(krow_off);
 
-    for (int m = 0; m < nrounds; ++m) {
+    for (int m = m_first; m < nrounds; ++m) {
         const int mb = m & 1;
         const int k = m * NW + wave;
+        const int st_first = step_lo(m), st_last = step_hi(m);
+        // WIN: this lane's window of streamed keys for (q, k); empty if k itself is outside the band of q
+        [[maybe_unused]] int wlo = 0, whi = -1;
+        if constexpr (WIN) {
+            if (k <= jq && (!banded || q <= k + p.wb)) {
+                wlo = banded ? max(q - p.wa, k - p.lab) : 0;
+                whi = banded ? min(jq, k + p.rab) : jq;
+            }
+        }
 
         v8 bq[KS], bg[KS];
         bool built = false;
@@ -212,14 +248,14 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
                 accT[dt][i] = 0.f;
             }
 
-        for (int st = 0; st < nsteps; ++st, ++gstage) {
+        for (int st = st_first; st <= st_last; ++st, ++gstage) {
             // this wave's part of stage gstage (and, at a round's first step, its part of the round's
             // rows) has landed; after the barrier that holds for every wave's part, and every wave is
             // done with the buffer the next fetch overwrites
             barrier_keep_loads<LW>();
-            if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
+            if (st == st_first && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
             issue_stage(st_ahead, (gstage + 2) % NBUF);
-            st_ahead = st_ahead + 1 < nsteps ? st_ahead + 1 : 0;
+            advance();
             if (!built) {
                 // B operands of the score products of this round: alpha log2e Q (.) K2[k] and dO (.) V2[k]
                 built = true;
@@ -246,17 +282,23 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
 
             const E* sb = sStage + (gstage % NBUF) * STAGE;
             const E* sK1 = sb;
-            const E* sU = sb + 4096;
-            const E* sK1T = sb + 8192;
-            const E* sUT = sb + 8192 + NCOL * 32;
+            const E* sU = sb + D * 32;
+            const E* sK1T = sb + 2 * D * 32;
+            const E* sUT = sb + 2 * D * 32 + NCOL * 32;
             const int jb = st * 32;
-            const bool need_mask = (k > jfull) || (jb + 31 > jfull);
+            bool need_mask = (k > jfull) || (jb + 31 > jfull);
+            if constexpr (WIN) {
+                // inside the band of every query of the tile (q0 .. q0 + 31), for this wave's row k
+                if (banded)
+                    need_mask = !((k <= q0) && (q0 + 31 <= k + p.wb) && (jb >= max(q0 + 31 - p.wa, k - p.lab)) &&
+                                  (jb + 31 <= min(q0, k + p.rab)));
+            }
 
             // row operands in two batches of four k-steps: the second is read under the first products
             v8 ak[KS], au[KS];
             auto load_rows = [&](int first) {
 #pragma unroll
-                for (int ks = first; ks < first + 4; ++ks) {
+                for (int ks = first; ks < min(first + 4, KS); ++ks) {
                     const int roff = ((ks >> 2) * 32 + krow_off) * 64 + ((((ks & 3) * 2 + g) ^ fperm) * 8);
                     ak[ks] = *reinterpret_cast<const v8*>(sK1 + roff);
                     au[ks] = *reinterpret_cast<const v8*>(sU + roff);
@@ -273,9 +315,15 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows128_kernel(BwdParams<E> p
                 for (int i = 0; i < 16; ++i) c[i] = 0.f;
                 dp = M::mma(a_ones, b_delta, c);
                 if (need_mask) {
-                    const int lim = (k <= jq) ? jq - jb - 8 * g : -1;
+                    if constexpr (WIN) {
+                        const int lo = wlo - jb - 8 * g, hi = whi - jb - 8 * g;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) c[i] = key_of(0, i) <= lim ? 0.f : -3.0e4f;
+                        for (int i = 0; i < 16; ++i) c[i] = (key_of(0, i) >= lo && key_of(0, i) <= hi) ? 0.f : -3.0e4f;
+                    } else {
+                        const int lim = (k <= jq) ? jq - jb - 8 * g : -1;
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) c[i] = key_of(0, i) <= lim ? 0.f : -3.0e4f;
+                    }
                 }
                 s = M::mma(a_ones, b_lse, c);
             }

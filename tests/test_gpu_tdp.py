@@ -283,6 +283,23 @@ def test_mfma_backward_d128_bf16(seq_len, causal, shape, monkeypatch):
             assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
 
 
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("windows", WINDOWS)
+@pytest.mark.parametrize("seq_len", [33, 100, 300])
+def test_mfma_backward_windows_bf16(seq_len, windows, D):
+    """Windowed masks on the MFMA backward (rounds and steps over the band only), all five gradients."""
+    print(f"case mfma bwd windows T={seq_len} {windows} D={D}", flush=True)
+    inputs = orc.make_inputs(1, 2, seq_len, D, torch.bfloat16, seed=seq_len + D + 3 * sum(windows))
+    alpha = 1 / math.sqrt(D)
+    z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
+    out, g = util.run_tdp(inputs, alpha, True, windows, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+        if b.abs().max() > 0:
+            assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
+
+
 def test_mfma_backward_d128_fp16_matches_generic():
     """Head dimension 128, fp16, several batch entries and heads: MFMA kernels against the fp32 kernels."""
     inputs = orc.make_inputs(2, 5, 150, 128, torch.float16, seed=33)
