@@ -62,7 +62,7 @@ const char* tritt_status_string(int status);
  * tritt_tdp_bwd replaces FlashTrittention.backward and its five launches
  *   (triple_dot_product/flash_trittention.py:141-393, kernels/bwd_{dq,dk1,dk2,dv1,dv2}.py),
  *   including Delta = rowsum(dO*O) and the SiLU' factor on dV1.  On the 16-bit MFMA path
- *   (D = 64, full windows) dK1/dV1/dK2/dV2 are accumulated with fp32 atomics: equal to rounding
+ *   (16-bit tensors, D = 64 or 128, any mask) dK1/dV1/dK2/dV2 are accumulated with fp32 atomics: equal to rounding
  *   from run to run, not bitwise; dQ and every fp32-tensor result are bitwise reproducible.
  */
 size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
