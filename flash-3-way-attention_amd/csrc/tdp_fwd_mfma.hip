@@ -286,187 +286,9 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
             [[maybe_unused]] bool started[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) started[t] = false;
-            if constexpr (NT == 2 && !CAREFUL && !WIN) {
-                // Stages whose 64 keys lie inside the causal bound of both tiles of this wave: a loop
-                // without branches on tile validity, so the accumulators stay in place (no copies
-                // at control-flow joins) and the wave itself overlaps matrix and vector work.  The
-                // arbiter serves the oldest wave first and all waves of a workgroup reach the same
-                // phase together, so overlap between waves cannot be relied on: the second tile's
-                // score product is issued in between the exp2/pack work of the first, and the first
-                // tile's value product in between that of the second.  K1 and U^T operands are
-                // read once for both tiles; the K1 operands of a block are fetched during the
-                // previous block of the same stage.
-                const int nfull = min(nst, (min(jmax[0], jmax[1]) + 1) / JS);
-                // MASKED (the stages that straddle the causal bound): a key past the bound of its tile
-                // starts its score at -3e4 (C operand of the first k-step), so its P is exactly 0.
-                // Element i of a lane is key jb + key_of(0, i) + 8 g.
-                auto fused = [&](auto masked_tag, const E* utp, const E* k1_next, v8 (&kn)[KS], int jb) {
-                constexpr bool MASKED = decltype(masked_tag)::value;
-                v8 ka[KS], ua[DT][2];
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) ka[ks] = kn[ks];
-                f32x16 s0, s1;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    s0[i] = (MASKED && key_of(0, i) > jmax[0] - jb - 8 * g) ? -3.0e4f : 0.f;
-                    s1[i] = (MASKED && key_of(0, i) > jmax[1] - jb - 8 * g) ? -3.0e4f : 0.f;
-                }
-                v8 pa0[2], pa1[2];
-                // quarter r of a tile's exp2 / pack / row-sum work: 4 exp2, 2 packs, 2 dot2
-                auto quarter = [&](const f32x16& sc, v8 (&pa)[2], float& ls, int r) {
-                    const int h = r >> 1, e0 = 4 * (r & 1);
-#pragma unroll
-                    for (int e = e0; e < e0 + 4; e += 2) {
-                        const v2 pr = M::pack(fast_exp2(sc[h * 8 + e]), fast_exp2(sc[h * 8 + e + 1]));
-                        ls = M::add_pair(pr, ls);
-                        pa[h][e] = pr[0];
-                        pa[h][e + 1] = pr[1];
-                    }
-                };
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) s0 = M::mma(ka[ks], bq[0][ks], s0);
-                __builtin_amdgcn_sched_barrier(0);
-                // U^T operands are first needed two MFMA groups from here
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-                        ua[dt][h] = *reinterpret_cast<const v8*>(utp + dt * 32 * LDU + h * 16);
-                __builtin_amdgcn_sched_barrier(0);
-                static_assert(KS == 4 && DT == 2, "the interleave below is written for D = 64");
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    s1 = M::mma(ka[r], bq[1][r], s1);
-                    __builtin_amdgcn_sched_barrier(0);
-                    quarter(s0, pa0, lsum[0], r);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                // the K1 operands are dead now: fetch those of the next block (null: none in reach)
-                if (k1_next) {
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1_next + ks * 16);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    acc[0][r & 1] = M::mma(pa0[r >> 1], ua[r & 1][r >> 1], acc[0][r & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
-                    quarter(s1, pa1, lsum[1], r);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[1][r & 1] = M::mma(pa1[r >> 1], ua[r & 1][r >> 1], acc[1][r & 1]);
-                __builtin_amdgcn_sched_barrier(0);
-                };
-                for (; st < nfull; ++st, ++gstage) {
-                    const int sb = gstage & 1;
-                    issue_stage(st + 1 < nst ? st + 1 : 0);
-                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
-                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
-                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
-                    v8 kn[KS];
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
-                    static_assert(JS == 64 || NT != 2, "two blocks per stage");
-                    fused(std::false_type{}, utp, k1p + 32 * LDK, kn, 0);
-                    fused(std::false_type{}, utp + 32, nullptr, kn, 0);
-                    commit_stage(sb ^ 1);
-                    __syncthreads();
-                }
-                for (; st < nst; ++st, ++gstage) {  // the one or two stages on the diagonal
-                    const int sb = gstage & 1;
-                    issue_stage(st + 1 < nst ? st + 1 : 0);
-                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
-                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
-                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
-                    v8 kn[KS];
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
-                    fused(std::true_type{}, utp, k1p + 32 * LDK, kn, st * JS);
-                    if (st * JS + 32 <= jend) fused(std::true_type{}, utp + 32, nullptr, kn, st * JS + 32);
-                    commit_stage(sb ^ 1);
-                    __syncthreads();
-                }
-            }
-            if constexpr (NT == 1 && !CAREFUL && !WIN) {
-                // The same for one tile per wave (D = 128: two tiles do not fit the register file).
-                // The two 32-key steps of a stage play the part of the two tiles: the score product
-                // of the second step is issued between the exp2 / pack work of the first, the value
-                // product of the first between that of the second.  No branch on validity inside
-                // the loop; every operand is read ahead of its use.
-                static_assert(JS == 64, "two steps per stage");
-                const int nfull = min(nst, (jmax[0] + 1) / JS);
-                for (; st < nfull; ++st, ++gstage) {
-                    const int sb = gstage & 1;
-                    issue_stage(st + 1 < nst ? st + 1 : 0);
-                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
-                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
-                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
-                    v8 ka[KS], ua[DT][2], pa[2][2];
-                    f32x16 sc[2];
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        sc[0][i] = 0.f;
-                        sc[1][i] = 0.f;
-                    }
-                    auto load_k = [&](int half) {
-#pragma unroll
-                        for (int ks = 0; ks < KS; ++ks)
-                            ka[ks] = *reinterpret_cast<const v8*>(k1p + half * 32 * LDK + ks * 16);
-                    };
-                    auto load_u = [&](int half) {
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                            for (int h = 0; h < 2; ++h)
-                                ua[dt][h] = *reinterpret_cast<const v8*>(utp + half * 32 + dt * 32 * LDU + h * 16);
-                    };
-                    auto pair = [&](int half, int r) {  // register pair r (0..7): 2 exp2, 1 pack, 1 row-sum step
-                        const int h = r >> 2, e = 2 * (r & 3);
-                        const v2 pr = M::pack(fast_exp2(sc[half][h * 8 + e]), fast_exp2(sc[half][h * 8 + e + 1]));
-                        lsum[0] = M::add_pair(pr, lsum[0]);
-                        pa[half][h][e] = pr[0];
-                        pa[half][h][e + 1] = pr[1];
-                    };
-                    auto value_mma = [&](int half, int r) {  // r = 0 .. 2 DT - 1; dependent ones are DT apart
-                        const int h = r / DT, dt = r % DT;
-                        acc[0][dt] = M::mma(pa[half][h], ua[dt][h], acc[0][dt]);
-                    };
-                    load_k(0);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) sc[0] = M::mma(ka[ks], bq[0][ks], sc[0]);
-                    __builtin_amdgcn_sched_barrier(0);
-                    load_k(1);
-                    load_u(0);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) {
-                        sc[1] = M::mma(ka[ks], bq[0][ks], sc[1]);
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int r = ks * 8 / KS; r < (ks + 1) * 8 / KS; ++r) pair(0, r);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-#pragma unroll
-                    for (int r = 0; r < 2 * DT; ++r) {
-                        value_mma(0, r);
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int q2 = r * 8 / (2 * DT); q2 < (r + 1) * 8 / (2 * DT); ++q2) pair(1, q2);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    load_u(1);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int r = 0; r < 2 * DT; ++r) value_mma(1, r);
-                    __builtin_amdgcn_sched_barrier(0);
-                    commit_stage(sb ^ 1);
-                    __syncthreads();
-                }
-            }
-            for (; st <= st_hi; ++st, ++gstage) {
+            // the general loop: any mask, any tile validity, FAST or CAREFUL; runs the stages st .. upto - 1
+            auto general_until = [&](int upto) {
+            for (; st < upto; ++st, ++gstage) {
                 const int sb = gstage & 1;
                 // the first stage is fetched again after the last one: the next k-tile, or a CAREFUL
                 // repeat of this one, starts from it
@@ -590,6 +412,199 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 if (more) commit_stage(sb ^ 1);
                 __syncthreads();
             }
+            };
+            if constexpr (NT == 2 && !CAREFUL && !WIN) {
+                // Stages whose 64 keys lie inside the causal bound of both tiles of this wave: a loop
+                // without branches on tile validity, so the accumulators stay in place (no copies
+                // at control-flow joins) and the wave itself overlaps matrix and vector work.  The
+                // arbiter serves the oldest wave first and all waves of a workgroup reach the same
+                // phase together, so overlap between waves cannot be relied on: the second tile's
+                // score product is issued in between the exp2/pack work of the first, and the first
+                // tile's value product in between that of the second.  K1 and U^T operands are
+                // read once for both tiles; the K1 operands of a block are fetched during the
+                // previous block of the same stage.
+                const int nfull = min(nst, (min(jmax[0], jmax[1]) + 1) / JS);
+                // MASKED (the stages that straddle the causal bound): a key past the bound of its tile
+                // starts its score at -3e4 (C operand of the first k-step), so its P is exactly 0.
+                // Element i of a lane is key jb + key_of(0, i) + 8 g.
+                auto fused = [&](auto masked_tag, const E* utp, const E* k1_next, v8 (&kn)[KS], int jb) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
+                v8 ka[KS], ua[DT][2];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) ka[ks] = kn[ks];
+                f32x16 s0, s1;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s0[i] = (MASKED && key_of(0, i) > jmax[0] - jb - 8 * g) ? -3.0e4f : 0.f;
+                    s1[i] = (MASKED && key_of(0, i) > jmax[1] - jb - 8 * g) ? -3.0e4f : 0.f;
+                }
+                v8 pa0[2], pa1[2];
+                // quarter r of a tile's exp2 / pack / row-sum work: 4 exp2, 2 packs, 2 dot2
+                auto quarter = [&](const f32x16& sc, v8 (&pa)[2], float& ls, int r) {
+                    const int h = r >> 1, e0 = 4 * (r & 1);
+#pragma unroll
+                    for (int e = e0; e < e0 + 4; e += 2) {
+                        const v2 pr = M::pack(fast_exp2(sc[h * 8 + e]), fast_exp2(sc[h * 8 + e + 1]));
+                        ls = M::add_pair(pr, ls);
+                        pa[h][e] = pr[0];
+                        pa[h][e + 1] = pr[1];
+                    }
+                };
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) s0 = M::mma(ka[ks], bq[0][ks], s0);
+                __builtin_amdgcn_sched_barrier(0);
+                // U^T operands are first needed two MFMA groups from here
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        ua[dt][h] = *reinterpret_cast<const v8*>(utp + dt * 32 * LDU + h * 16);
+                __builtin_amdgcn_sched_barrier(0);
+                static_assert(KS == 4 && DT == 2, "the interleave below is written for D = 64");
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    s1 = M::mma(ka[r], bq[1][r], s1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    quarter(s0, pa0, lsum[0], r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // the K1 operands are dead now: fetch those of the next block (null: none in reach)
+                if (k1_next) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1_next + ks * 16);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    acc[0][r & 1] = M::mma(pa0[r >> 1], ua[r & 1][r >> 1], acc[0][r & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    quarter(s1, pa1, lsum[1], r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[1][r & 1] = M::mma(pa1[r >> 1], ua[r & 1][r >> 1], acc[1][r & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                };
+                for (; st < nfull; ++st, ++gstage) {
+                    const int sb = gstage & 1;
+                    issue_stage(st + 1 < nst ? st + 1 : 0);
+                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
+                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
+                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
+                    v8 kn[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
+                    static_assert(JS == 64 || NT != 2, "two blocks per stage");
+                    fused(std::false_type{}, utp, k1p + 32 * LDK, kn, 0);
+                    fused(std::false_type{}, utp + 32, nullptr, kn, 0);
+                    commit_stage(sb ^ 1);
+                    __syncthreads();
+                }
+                for (; st < nst; ++st, ++gstage) {  // the one or two stages on the diagonal
+                    const int sb = gstage & 1;
+                    issue_stage(st + 1 < nst ? st + 1 : 0);
+                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
+                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
+                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
+                    v8 kn[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
+                    fused(std::true_type{}, utp, k1p + 32 * LDK, kn, st * JS);
+                    if (st * JS + 32 <= jend) fused(std::true_type{}, utp + 32, nullptr, kn, st * JS + 32);
+                    commit_stage(sb ^ 1);
+                    __syncthreads();
+                }
+            }
+            if constexpr (NT == 1 && !CAREFUL) {
+                // The same for one tile per wave (D = 128: two tiles do not fit the register file).
+                // The two 32-key steps of a stage play the part of the two tiles: the score product
+                // of the second step is issued between the exp2 / pack work of the first, the value
+                // product of the first between that of the second.  No branch on validity inside
+                // the loop; every operand is read ahead of its use.
+                static_assert(JS == 64, "two steps per stage");
+                int nfull = min(nst, (jmax[0] + 1) / JS);
+                if constexpr (WIN) {
+                    if (banded) {
+                        // stages whose 64 keys are inside the band of every (q, k) of this tile; the stages
+                        // before them go through the general loop first
+                        const int q = qrow[0], k0 = kt * 32;
+                        const bool rows_in = (k0 + 31 <= jmax[0]) && (q <= k0 + p.wb);
+                        const int in_lo = (max(0, max(q - p.wa, k0 + 31 - p.lab)) + JS - 1) / JS;
+                        nfull = rows_in ? min(st_hi + 1, (min(jmax[0], k0 + p.rab) + 1) / JS) : 0;
+                        general_until(min(st_hi + 1, max(st_lo, min(in_lo, nfull))));
+                    }
+                }
+                for (; st < nfull; ++st, ++gstage) {
+                    const int sb = gstage & 1;
+                    issue_stage(st < st_hi ? st + 1 : st_next);
+                    if (st == st_lo && kt + 1 < nkt) issue_ktile(kt + 1);
+                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
+                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
+                    v8 ka[KS], ua[DT][2], pa[2][2];
+                    f32x16 sc[2];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        sc[0][i] = 0.f;
+                        sc[1][i] = 0.f;
+                    }
+                    auto load_k = [&](int half) {
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks)
+                            ka[ks] = *reinterpret_cast<const v8*>(k1p + half * 32 * LDK + ks * 16);
+                    };
+                    auto load_u = [&](int half) {
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                            for (int h = 0; h < 2; ++h)
+                                ua[dt][h] = *reinterpret_cast<const v8*>(utp + half * 32 + dt * 32 * LDU + h * 16);
+                    };
+                    auto pair = [&](int half, int r) {  // register pair r (0..7): 2 exp2, 1 pack, 1 row-sum step
+                        const int h = r >> 2, e = 2 * (r & 3);
+                        const v2 pr = M::pack(fast_exp2(sc[half][h * 8 + e]), fast_exp2(sc[half][h * 8 + e + 1]));
+                        lsum[0] = M::add_pair(pr, lsum[0]);
+                        pa[half][h][e] = pr[0];
+                        pa[half][h][e + 1] = pr[1];
+                    };
+                    auto value_mma = [&](int half, int r) {  // r = 0 .. 2 DT - 1; dependent ones are DT apart
+                        const int h = r / DT, dt = r % DT;
+                        acc[0][dt] = M::mma(pa[half][h], ua[dt][h], acc[0][dt]);
+                    };
+                    load_k(0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) sc[0] = M::mma(ka[ks], bq[0][ks], sc[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_k(1);
+                    load_u(0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        sc[1] = M::mma(ka[ks], bq[0][ks], sc[1]);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int r = ks * 8 / KS; r < (ks + 1) * 8 / KS; ++r) pair(0, r);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 2 * DT; ++r) {
+                        value_mma(0, r);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int q2 = r * 8 / (2 * DT); q2 < (r + 1) * 8 / (2 * DT); ++q2) pair(1, q2);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    load_u(1);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int r = 0; r < 2 * DT; ++r) value_mma(1, r);
+                    __builtin_amdgcn_sched_barrier(0);
+                    commit_stage(sb ^ 1);
+                    __syncthreads();
+                }
+            }
+            general_until(st_hi + 1);
         };
 
         sweep(std::false_type{});
@@ -759,12 +774,13 @@ static hipError_t launch_d64(const MfmaFwdArgs& a, hipStream_t st) {
 
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
     if (a.windowed) {
-        // one tile per wave; D = 64 with four waves per SIMD (the general loop has no interleave of its own)
+        // one tile per wave, eight waves: the stages inside the band run the two-step interleaved loop,
+        // the stages on its edges the general one
         if (a.is_bf16) {
-            if (a.D == 64) return launch<__bf16, 64, 1, 16, 4, 64, true>(a, st);
+            if (a.D == 64) return launch<__bf16, 64, 1, 8, 2, 64, true>(a, st);
             if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64, true>(a, st);
         } else {
-            if (a.D == 64) return launch<_Float16, 64, 1, 16, 4, 64, true>(a, st);
+            if (a.D == 64) return launch<_Float16, 64, 1, 8, 2, 64, true>(a, st);
             if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64, true>(a, st);
         }
         return hipErrorInvalidValue;
