@@ -35,6 +35,20 @@ def triples(B, H, T, causal=True):
     return B * H * (T * (T + 1) * (2 * T + 1) // 6 if causal else T ** 3)
 
 
+def windowed_triples(T, w1, w2, kl, kr):
+    """Valid (q, j, k) of one head under the windowed causal mask, by the predicate the kernels use:
+    j, k <= q, q - j <= w1, q - k <= w2, k - j <= kl, j - k <= kr."""
+    import numpy as np
+
+    total = 0
+    for q in range(T):
+        j = np.arange(max(0, q - w1), q + 1)
+        lo = np.maximum(max(0, q - w2), j - kr)
+        hi = np.minimum(q, j + kl)
+        total += int(np.maximum(hi - lo + 1, 0).sum())
+    return total
+
+
 def time_events(fn, iters, warmup, torch):
     """Average milliseconds per call, HIP events on the stream the kernels run on
     (torch's current stream, which is the stream handed to the library)."""
@@ -92,11 +106,14 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "dps"], default="both",
+    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "dps", "tdp"], default="both",
                     help="fwd: time only the forward (for profiling runs); copy: a plain 256 MiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against; "
                          "sweep: triple-dot forward at B=1 H=16 D=128 bf16 over T in 512..4096; "
-                         "dps: dot-product-sum forward+backward at --B --H --T --D")
+                         "dps: dot-product-sum forward+backward at --B --H --T --D; "
+                         "tdp: triple-dot forward+backward at --B --H --T --D with --windows (secondary shapes: "
+                         "D=128, windowed masks)")
+    ap.add_argument("--windows", default="", help="k1_window,k2_window,kk_left,kk_right for --mode tdp (empty: full)")
     ap.add_argument("--B", type=int, default=4)
     ap.add_argument("--H", type=int, default=8)
     ap.add_argument("--T", type=int, default=1024)
@@ -191,6 +208,21 @@ def main():
 
     n = triples(B, H, T)
     f_fwd, f_bwd = 4 * D * n, 12 * D * n
+
+    if args.mode == "tdp":
+        win = [int(x) for x in args.windows.split(",")] if args.windows else None
+        if win:
+            kw.update(k1_window=win[0], k2_window=win[1], kk_left=win[2], kk_right=win[3])
+            n = B * H * windowed_triples(T, *win)
+            f_fwd, f_bwd = 4 * D * n, 12 * D * n
+        ms_fwd = time_events(fwd_only, args.steps, args.warmup, torch)
+        fwd_graph()
+        ms_bwd = time_events(bwd_only, args.steps, args.warmup, torch)
+        print(json.dumps({"metric": "triple-dot trittention fwd / bwd", "unit": "ms", "fwd_ms": ms_fwd, "bwd_ms": ms_bwd,
+                          "fwd_tflops": f_fwd / ms_fwd / 1e9, "bwd_tflops": f_bwd / ms_bwd / 1e9, "valid_triples": n,
+                          "config": {"workload": f"triple-dot fwd+bwd B={B} H={H} T={T} D={D} bf16 causal",
+                                     "windows": win}}), flush=True)
+        return
 
     if args.mode == "fwd":
         ms_fwd = time_events(fwd_only, args.steps, args.warmup, torch)
