@@ -728,12 +728,11 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
     constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS>();
     auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN>;
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
+    {
+        // per call: the attribute belongs to the current device, and a process may drive several
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return e;
-        attr_set = true;
     }
     const int groups = (a.BH + 7) / 8;
     hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(64 * WAVES), smem, st, p);
