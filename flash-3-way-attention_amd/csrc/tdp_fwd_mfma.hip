@@ -744,7 +744,7 @@ size_t mfma_tdp_fwd_workspace(int BH, int T, int D) {
     return (size_t)BH * D * Tp * 2;
 }
 
-bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
+bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
 
 // Tile shape used for D = 64.  TRITT_FWD_VARIANT (read once) selects another instantiation for
 // tuning sweeps: "nt2w8" (default), "nt1w16", "nt1w8".
@@ -776,18 +776,22 @@ hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
         // one tile per wave, eight waves: the stages inside the band run the two-step interleaved loop,
         // the stages on its edges the general one
         if (a.is_bf16) {
+            if (a.D == 32) return launch<__bf16, 32, 1, 8, 2, 64, true>(a, st);
             if (a.D == 64) return launch<__bf16, 64, 1, 8, 2, 64, true>(a, st);
             if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64, true>(a, st);
         } else {
+            if (a.D == 32) return launch<_Float16, 32, 1, 8, 2, 64, true>(a, st);
             if (a.D == 64) return launch<_Float16, 64, 1, 8, 2, 64, true>(a, st);
             if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64, true>(a, st);
         }
         return hipErrorInvalidValue;
     }
     if (a.is_bf16) {
+        if (a.D == 32) return launch<__bf16, 32, 1, 8, 2, 64>(a, st);
         if (a.D == 64) return launch_d64<__bf16>(a, st);
         if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64>(a, st);
     } else {
+        if (a.D == 32) return launch<_Float16, 32, 1, 8, 2, 64>(a, st);
         if (a.D == 64) return launch_d64<_Float16>(a, st);
         if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64>(a, st);
     }

@@ -156,7 +156,7 @@ def test_input_precision_warns_and_is_ignored():
 FORCE_GENERIC, FORCE_MFMA = 1, 2
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("seq_len", [1, 16, 33, 100, 129, 256])
 def test_mfma_forward_bf16(seq_len, causal, D):
@@ -167,14 +167,15 @@ def test_mfma_forward_bf16(seq_len, causal, D):
     z, _, _ = util.oracle_tdp(inputs, alpha, causal)
     out, _ = util.run_tdp(inputs, alpha, causal, backward=False, flags=FORCE_MFMA)
     util.assert_close("out", out, z, **LOWP)
-    assert util.rel_err(out, z) <= 2e-2, util.rel_err(out, z)
+    # unmasked rows average ~T^2 terms: the outputs are small and the 16-bit rounding of P shows in max-relative terms
+    assert util.rel_err(out, z) <= (3e-2 if D == 32 else 2e-2), util.rel_err(out, z)
 
 
 WINDOWS = [(8, 8, 4, 4), (5, 3, 4, 1), (2, 70, 0, 3), (40, 100, 20, 7), (64, 64, 64, 64), (100, 10, 50, 0),
            (1, 1, 1, 1), (300, 300, 0, 0)]
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("windows", WINDOWS)
 @pytest.mark.parametrize("seq_len", [33, 100, 300])
 def test_mfma_forward_windows_bf16(seq_len, windows, D):
