@@ -38,7 +38,7 @@ struct DpsArgs {
 hipError_t dps_fwd(const DpsArgs& a, hipStream_t st);
 hipError_t dps_bwd(const DpsArgs& a, hipStream_t st);
 
-// 16-bit MFMA triple-dot forward (full causal windows or no mask; D = 64 or 128).
+// 16-bit MFMA triple-dot forward (any mask; D = 32, 64 or 128).
 struct MfmaFwdArgs {
     const void *q, *k1, *k2, *v1, *v2;
     void* o;

@@ -1,5 +1,6 @@
-// Triple-dot-product trittention backward on MFMA (gfx950), 16-bit tensors, D = 64,
-// full causal windows or no mask.
+// Triple-dot-product trittention backward on MFMA (gfx950), 16-bit tensors.  This file: the kernel
+// for D = 64 with full causal windows or no mask, the scratch producers / consumers and the launcher;
+// tdp_bwd_rows_general.hpp: D = 128 and windowed masks.
 //
 // With virtual query rows (q,k):  A = alpha*log2e * Q[q] (.) K2[k],  G = dO[q] (.) V2[k],
 //   S = A K1^T (log2 units),  P = exp2(S - LSE2[q]),  dP = G U^T,  dS = P (dP - Delta[q])

@@ -1,5 +1,5 @@
-// Triple-dot-product trittention forward on MFMA (gfx950), 16-bit tensors, full causal
-// windows or no mask.
+// Triple-dot-product trittention forward on MFMA (gfx950), 16-bit tensors, D = 32, 64 or 128;
+// full causal windows or no mask, and (WIN instantiations) windowed causal masks.
 //
 // Formulation.  For a fixed key-2 row k the scores of query q are an ordinary attention row:
 //   s[q,j,k] = (alpha * Q[q] (.) K2[k]) . K1[j]
