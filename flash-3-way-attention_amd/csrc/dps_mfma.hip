@@ -28,6 +28,7 @@ namespace {
 
 constexpr int kW = 4;     // waves per workgroup
 constexpr int kLdr = 33;  // LDS row stride (floats) of the cross-wave reduction tiles
+constexpr float kLazyRaise = 8.0f;  // log2 units a score may exceed the running reference before it is raised
 
 template <typename E>
 __device__ __forceinline__ typename Mma<E>::v8 ld8(const E* p) {
@@ -130,9 +131,24 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
             for (int kk = 0; kk < 2; ++kk)
                 vn[dt][kk] = ld8<E>(VT + (size_t)(32 * dt + n) * Tp + t * 32 + 16 * kk + 8 * g);
     };
+    float b[16];  // per-key bias of the tile (0 without one), fetched ahead like the operands
+#pragma unroll
+    for (int i = 0; i < 16; ++i) b[i] = 0.f;
+    auto fetch_b = [&](int t) {
+        if (bias) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const float4 v = *reinterpret_cast<const float4*>(bias + t * 32 + 16 * h + 8 * g + 4 * c);
+                    b[8 * h + 4 * c] = v.x; b[8 * h + 4 * c + 1] = v.y; b[8 * h + 4 * c + 2] = v.z; b[8 * h + 4 * c + 3] = v.w;
+                }
+        }
+    };
     const int t_first = a_lo / 32 + wave, t_last = a_hi / 32;
     if (t_first <= t_last) {
         fetch_k(t_first);
+        fetch_b(t_first);
         fetch_v(t_first);
     }
     for (int t = t_first; t <= t_last; t += kW) {
@@ -144,43 +160,48 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) s = M::mma(kn[ks], xb[ks], s);
         if (more) fetch_k(t + kW);
-        float b[16];
+        // Only tiles on an edge of the band (or past the end of the sequence) need the element-wise mask.
+        const bool edge = (a0 + 31 >= T) || (p.causal && ((a0 + 31 > r0) || (r0 + 31 - a0 > p.k_diff)));
+        float sv[16];
+        if (edge) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) b[i] = 0.f;
-        if (bias) {
+            for (int i = 0; i < 16; ++i) {
+                const int a = a0 + key_of(g, i);
+                const bool ok = (a < T) & ((!p.causal) | ((a <= r) & (r - a <= p.k_diff)));
+                sv[i] = ok ? fmaf(s[i], p.scale_log2, b[i]) : -INFINITY;
+            }
+        } else {
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const float4 v = *reinterpret_cast<const float4*>(bias + a0 + 16 * h + 8 * g + 4 * c);
-                    b[8 * h + 4 * c] = v.x; b[8 * h + 4 * c + 1] = v.y; b[8 * h + 4 * c + 2] = v.z; b[8 * h + 4 * c + 3] = v.w;
-                }
+            for (int i = 0; i < 16; ++i) sv[i] = fmaf(s[i], p.scale_log2, b[i]);
         }
-        float sv[16], tmax = -INFINITY;
+        if (more) fetch_b(t + kW);
+        float tmax = fmaxf(sv[0], sv[1]);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int a = a0 + key_of(g, i);
-            const bool ok = (a < T) & ((!p.causal) | ((a <= r) & (r - a <= p.k_diff)));
-            sv[i] = ok ? fmaf(s[i], p.scale_log2, b[i]) : -INFINITY;
-            tmax = fmaxf(tmax, sv[i]);
-        }
+        for (int i = 2; i < 16; i += 2) tmax = fmaxf(fmaxf(tmax, sv[i]), sv[i + 1]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m, tmax);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float f = fast_exp2(m - m_use);
-        m = m_new;
-        l *= f;
+        // The reference maximum is raised lazily: only when some row's scores exceed it by more than 2^8
+        // (the first tile always does: m starts at -inf), so most tiles skip the rescaling.
+        if (__any(tmax > m + kLazyRaise)) {
+            const float m_new = fmaxf(m, tmax);
+            const float f = fast_exp2(m - (m_new == -INFINITY ? 0.f : m_new));
+            m = m_new;
+            l *= f;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[dt][i] *= f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            sv[i] = fast_exp2(sv[i] - m_use);
-            l += sv[i];
+                for (int i = 0; i < 16; ++i) acc[dt][i] *= f;
         }
+        const float m_use = m == -INFINITY ? 0.f : m;
         v8 pb[2];
-        pack16<E>(sv, pb);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                const typename M::v2 pr = M::pack(fast_exp2(sv[8 * h + e] - m_use), fast_exp2(sv[8 * h + e + 1] - m_use));
+                l = M::add_pair(pr, l);  // the row sum of what the value product sees
+                pb[h][e] = pr[0];
+                pb[h][e + 1] = pr[1];
+            }
         // O^T[d][r] += V^T[d][a] P^T[a][r]
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
