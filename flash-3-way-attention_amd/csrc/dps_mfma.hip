@@ -17,9 +17,15 @@
 // Every tile is computed transposed where needed so that the owner index sits on the MFMA column
 // (= lane) axis: softmax statistics, LSE and Delta stay lane-local, and with the permuted row order
 // of mfma.hpp the probabilities leave one MFMA in exactly the operand layout of the next.
-// Operands are read straight from global memory in MFMA layout (16 B per lane); contraction over
-// a row index reads the [D][Tp] transposed copies that the prep kernel / the producing epilogue
-// writes.  Every output element has one owner: no atomics, bitwise reproducible.
+// Streamed operands are read straight from global memory, 16 B per lane, from operand-packed
+// copies: the 64 x 16 B that one MFMA operand load needs are one contiguous kilobyte (a gather of
+// 16-byte pieces from 32 different rows costs one cache-line lookup per row, and that address
+// traffic, not MFMA or bandwidth, was what bound these kernels).  Two packings of a [T][D] tensor,
+// both in tiles of 32 rows and both exactly Tp x D elements:
+//   P1 (k-slots run along d; rows permuted by key_of_row):  [tile][ks][lane][8]
+//   P2 (k-slots run along the row index; "transposed use"): [tile][dt][kk][lane][8]
+// The prep kernel writes them for the inputs, the producing epilogues for W and dR.  Every output
+// element has one owner: no atomics, bitwise reproducible.
 #include "kernels.hpp"
 #include "mfma.hpp"
 
@@ -29,6 +35,31 @@ namespace {
 constexpr int kW = 4;     // waves per workgroup
 constexpr int kLdr = 33;  // LDS row stride (floats) of the cross-wave reduction tiles
 constexpr float kLazyRaise = 8.0f;  // log2 units a score may exceed the running reference before it is raised
+
+// MFMA row that holds key offset k of a 32-key tile (inverse of key_of_row)
+__device__ __forceinline__ int row_of_key(int k) {
+    const int i = 8 * (k >> 4) + (k & 7), g = (k >> 3) & 1;
+    return ((i >> 2) << 3) | (g << 2) | (i & 3);
+}
+// element offsets of (row, d) in the two packings
+template <int D>
+__device__ __forceinline__ size_t p1_index(int row, int d) {
+    return ((size_t)((row >> 5) * (D / 16) + (d >> 4)) * 64 + ((d >> 3) & 1) * 32 + row_of_key(row & 31)) * 8 + (d & 7);
+}
+template <int D>
+__device__ __forceinline__ size_t p2_index(int row, int d) {
+    const int a = row & 31;
+    return ((size_t)(((row >> 5) * (D / 32) + (d >> 5)) * 2 + (a >> 4)) * 64 + ((a >> 3) & 1) * 32 + (d & 31)) * 8 + (a & 7);
+}
+// the operand loads: lane's 16 bytes of (tile t, k-step ks) / (tile t, d-tile dt, half kk)
+template <typename E, int D>
+__device__ __forceinline__ const E* p1_at(const E* z, int t, int ks, int lane) {
+    return z + ((size_t)(t * (D / 16) + ks) * 64 + lane) * 8;
+}
+template <typename E, int D>
+__device__ __forceinline__ const E* p2_at(const E* z, int t, int dt, int kk, int lane) {
+    return z + ((size_t)((t * (D / 32) + dt) * 2 + kk) * 64 + lane) * 8;
+}
 
 template <typename E>
 __device__ __forceinline__ typename Mma<E>::v8 ld8(const E* p) {
@@ -65,14 +96,15 @@ __device__ __forceinline__ void spill_tiles(float* sO, int wave, const f32x16 (&
 template <typename E>
 struct AttnFwdP {
     const E* x;         // [BH][T][D]   query-like rows
-    const E* k;         // [BH][T][D]   key-like rows
-    const E* vt;        // [BH][D][Tp]  values, transposed, zero padded
+    const E* kp;        // [BH][Tp*D]   key-like rows, packing P1
+    const E* vp2;       // [BH][Tp*D]   values, packing P2
     const float* bias;  // [BH][Tp] per-key bias in log2 units, or null
     const E* mul;       // [BH][T][D] or null
     E* out;             // [BH][T][D] or null
     float* out_f32;     // [BH][T][D] or null
     E* outm;            // out * mul, [BH][T][D] or null
-    E* outm_t;          // out * mul, [BH][D][Tp] or null
+    E* outm_p1;         // out * mul, packing P1, or null
+    E* outm_p2;         // out * mul, packing P2, or null
     float* lse;         // [BH][lse_stride]
     int lse_stride;
     float lse_scale;    // lse = lse_scale * log2-sum-exp2
@@ -97,8 +129,8 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     const int T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
     const E* __restrict__ X = p.x + base;
-    const E* __restrict__ K = p.k + base;
-    const E* __restrict__ VT = p.vt + tb;
+    const E* __restrict__ KP = p.kp + tb;
+    const E* __restrict__ VP2 = p.vp2 + tb;
     const float* __restrict__ bias = p.bias ? p.bias + vb : nullptr;
     const int r = r0 + n;
 
@@ -120,16 +152,15 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     // tile would be most of its time).
     v8 kn[KS], vn[DT][2];
     auto fetch_k = [&](int t) {
-        const E* krow = K + (size_t)min(t * 32 + key_of_row(n), T - 1) * D + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kn[ks] = ld8<E>(krow + 16 * ks);
+        for (int ks = 0; ks < KS; ++ks) kn[ks] = ld8<E>(p1_at<E, D>(KP, t, ks, lane));
     };
     auto fetch_v = [&](int t) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
-                vn[dt][kk] = ld8<E>(VT + (size_t)(32 * dt + n) * Tp + t * 32 + 16 * kk + 8 * g);
+                vn[dt][kk] = ld8<E>(p2_at<E, D>(VP2, t, dt, kk, lane));
     };
     float b[16];  // per-key bias of the tile (0 without one), fetched ahead like the operands
 #pragma unroll
@@ -265,9 +296,10 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) wv[j] = (E)(row < T ? o[j] * (float)mv[j] : 0.f);
             if (p.outm && row < T) *reinterpret_cast<v8*>(p.outm + off) = wv;
-            if (p.outm_t)
+            if (p.outm_p1) *reinterpret_cast<v8*>(p.outm_p1 + tb + p1_index<D>(row, d0)) = wv;  // 8 consecutive d: one piece
+            if (p.outm_p2)
 #pragma unroll
-                for (int j = 0; j < 8; ++j) p.outm_t[tb + (size_t)(d0 + j) * Tp + row] = wv[j];
+                for (int j = 0; j < 8; ++j) p.outm_p2[tb + p2_index<D>(row, d0 + j)] = wv[j];
         }
     }
 }
@@ -275,9 +307,11 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
 // ------------------------------------------------------------------------------ backward, rows
 template <typename E>
 struct AttnBwdP {
-    const E *x, *g, *k, *v;  // [BH][T][D] row-major: query-like rows, their upstream gradient, keys, values
-    const E *kt;             // K^T [BH][D][Tp]   (row kernel)
-    const E *xt, *gt;        // X^T, G^T [BH][D][Tp]  (column kernel)
+    // [BH][T][D] row-major: what the owner tile loads once (row kernel: x, g; column kernel: k, v)
+    const E *x, *g, *k, *v;
+    // streamed, operand-packed [BH][Tp*D]: row kernel kp, vp (P1) and kp2 (P2);
+    // column kernel xp, gp (P1) and xp2, gp2 (P2)
+    const E *kp, *vp, *kp2, *xp, *gp, *xp2, *gp2;
     const float* bias;       // [BH][Tp] log2 units or null
     const float* lse2;       // [BH][Tp] log2 units
     const float* delta;      // [BH][Tp]
@@ -296,7 +330,7 @@ struct AttnBwdP {
     // LINK == true: dW = sum;  dV2 = dW R;  dR = dW V2;  delta1 = rowsum(dR R) - dbias
     const float* r_f32;
     const E* v2;
-    E *dv2, *dr, *dr_t;
+    E *dv2, *dr, *dr_p1, *dr_p2;
     float* delta1;           // [BH][Tp]
 };
 
@@ -313,9 +347,9 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
-    const E* __restrict__ K = p.k + base;
-    const E* __restrict__ V = p.v + base;
-    const E* __restrict__ KT = p.kt + tb;
+    const E* __restrict__ KP = p.kp + tb;
+    const E* __restrict__ VP = p.vp + tb;
+    const E* __restrict__ KP2 = p.kp2 + tb;
     const float* __restrict__ bias = p.bias ? p.bias + vb : nullptr;
     const int r = r0 + n, rc = min(r, T - 1);
     const float scale_log2 = p.alpha * kLog2e;
@@ -336,47 +370,80 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
 
-    for (int t = a_lo / 32 + wave; t <= a_hi / 32; t += kW) {
+    // streamed operands and the bias of a tile are fetched one tile ahead, into the registers the
+    // previous tile has just consumed
+    v8 kn[KS], vn[KS], k2n[DT][2];
+    float b[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) b[i] = 0.f;
+    auto fetch_rows = [&](int t) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            kn[ks] = ld8<E>(p1_at<E, D>(KP, t, ks, lane));
+            vn[ks] = ld8<E>(p1_at<E, D>(VP, t, ks, lane));
+        }
+    };
+    auto fetch_bias = [&](int t) {
+        if (bias) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const float4 v = *reinterpret_cast<const float4*>(bias + t * 32 + 16 * h + 8 * g + 4 * c);
+                    b[8 * h + 4 * c] = v.x; b[8 * h + 4 * c + 1] = v.y; b[8 * h + 4 * c + 2] = v.z; b[8 * h + 4 * c + 3] = v.w;
+                }
+        }
+    };
+    auto fetch_cols = [&](int t) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) k2n[dt][kk] = ld8<E>(p2_at<E, D>(KP2, t, dt, kk, lane));
+    };
+    const int t_first = a_lo / 32 + wave, t_last = a_hi / 32;
+    if (t_first <= t_last) {
+        fetch_rows(t_first);
+        fetch_bias(t_first);
+        fetch_cols(t_first);
+    }
+    for (int t = t_first; t <= t_last; t += kW) {
         const int a0 = t * 32;
+        const bool more = t + kW <= t_last;
         f32x16 s, dp;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             s[i] = 0.f;
             dp[i] = 0.f;
         }
-        const size_t ro = (size_t)min(a0 + key_of_row(n), T - 1) * D + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = M::mma(ld8<E>(K + ro + 16 * ks), xb[ks], s);
+        for (int ks = 0; ks < KS; ++ks) s = M::mma(kn[ks], xb[ks], s);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dp = M::mma(ld8<E>(V + ro + 16 * ks), gb[ks], dp);
-        float b[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) b[i] = 0.f;
-        if (bias) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const float4 v = *reinterpret_cast<const float4*>(bias + a0 + 16 * h + 8 * g + 4 * c);
-                    b[8 * h + 4 * c] = v.x; b[8 * h + 4 * c + 1] = v.y; b[8 * h + 4 * c + 2] = v.z; b[8 * h + 4 * c + 3] = v.w;
-                }
-        }
+        for (int ks = 0; ks < KS; ++ks) dp = M::mma(vn[ks], gb[ks], dp);
+        if (more) fetch_rows(t + kW);
+        // only tiles on an edge of the band (or past the end of the sequence) need the element-wise mask
+        const bool edge = (a0 + 31 >= T) || (r0 + 31 >= T) || (p.causal && ((a0 + 31 > r0) || (r0 + 31 - a0 > p.k_diff)));
         float ds[16];
+        if (edge) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int a = a0 + key_of(g, i);
-            const bool ok = pair_ok(T, p.causal, p.k_diff, r, a);
-            const float pr = ok ? fast_exp2(fmaf(s[i], scale_log2, b[i] - lse2)) : 0.f;
-            ds[i] = pr * (dp[i] - dl);
+            for (int i = 0; i < 16; ++i) {
+                const int a = a0 + key_of(g, i);
+                const bool ok = pair_ok(T, p.causal, p.k_diff, r, a);
+                const float pr = ok ? fast_exp2(fmaf(s[i], scale_log2, b[i] - lse2)) : 0.f;
+                ds[i] = pr * (dp[i] - dl);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ds[i] = fast_exp2(fmaf(s[i], scale_log2, b[i] - lse2)) * (dp[i] - dl);
         }
+        if (more) fetch_bias(t + kW);
         v8 dsb[2];
         pack16<E>(ds, dsb);
         // dX^T[d][r] += K^T[d][a] dS^T[a][r]
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
-                acc[dt] = M::mma(ld8<E>(KT + (size_t)(32 * dt + n) * Tp + a0 + 16 * kk + 8 * g), dsb[kk], acc[dt]);
+            for (int kk = 0; kk < 2; ++kk) acc[dt] = M::mma(k2n[dt][kk], dsb[kk], acc[dt]);
+        if (more) fetch_cols(t + kW);
     }
 
     spill_tiles<D>(sO, wave, acc, n, g);
@@ -417,10 +484,10 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
-    const E* __restrict__ X = p.x + base;
-    const E* __restrict__ G = p.g + base;
-    const E* __restrict__ XT = p.xt + tb;
-    const E* __restrict__ GT = p.gt + tb;
+    const E* __restrict__ XP = p.xp + tb;
+    const E* __restrict__ GP = p.gp + tb;
+    const E* __restrict__ XP2 = p.xp2 + tb;
+    const E* __restrict__ GP2 = p.gp2 + tb;
     const float* __restrict__ lse2 = p.lse2 + vb;
     const float* __restrict__ delta = p.delta + vb;
     const int a = c0 + n, ac = min(a, T - 1);
@@ -446,38 +513,78 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
         }
     float db = 0.f;
 
-    for (int t = r_lo / 32 + wave; t <= r_hi / 32; t += kW) {
+    // streamed operands and the per-row statistics of a tile are fetched one tile ahead, into the
+    // registers the previous tile has just consumed
+    v8 xn[KS], gn[KS], x2n[DT][2], g2n[DT][2];
+    float ls[16], dl[16];
+    auto fetch_rows = [&](int t) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            xn[ks] = ld8<E>(p1_at<E, D>(XP, t, ks, lane));
+            gn[ks] = ld8<E>(p1_at<E, D>(GP, t, ks, lane));
+        }
+    };
+    auto fetch_stats = [&](int t) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const float4 v = *reinterpret_cast<const float4*>(lse2 + t * 32 + 16 * h + 8 * g + 4 * c);
+                const float4 w = *reinterpret_cast<const float4*>(delta + t * 32 + 16 * h + 8 * g + 4 * c);
+                ls[8 * h + 4 * c] = v.x; ls[8 * h + 4 * c + 1] = v.y; ls[8 * h + 4 * c + 2] = v.z; ls[8 * h + 4 * c + 3] = v.w;
+                dl[8 * h + 4 * c] = w.x; dl[8 * h + 4 * c + 1] = w.y; dl[8 * h + 4 * c + 2] = w.z; dl[8 * h + 4 * c + 3] = w.w;
+            }
+    };
+    auto fetch_cols = [&](int t) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                x2n[dt][kk] = ld8<E>(p2_at<E, D>(XP2, t, dt, kk, lane));
+                g2n[dt][kk] = ld8<E>(p2_at<E, D>(GP2, t, dt, kk, lane));
+            }
+    };
+    const int t_first = r_lo / 32 + wave, t_last = r_hi / 32;
+    if (t_first <= t_last) {
+        fetch_rows(t_first);
+        fetch_stats(t_first);
+        fetch_cols(t_first);
+    }
+    for (int t = t_first; t <= t_last; t += kW) {
         const int r0 = t * 32;
+        const bool more = t + kW <= t_last;
         f32x16 s, dp;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             s[i] = 0.f;
             dp[i] = 0.f;
         }
-        const size_t ro = (size_t)min(r0 + key_of_row(n), T - 1) * D + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = M::mma(ld8<E>(X + ro + 16 * ks), kb[ks], s);
+        for (int ks = 0; ks < KS; ++ks) s = M::mma(xn[ks], kb[ks], s);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dp = M::mma(ld8<E>(G + ro + 16 * ks), vbv[ks], dp);
-        float ls[16], dl[16];
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const float4 v = *reinterpret_cast<const float4*>(lse2 + r0 + 16 * h + 8 * g + 4 * c);
-                const float4 w = *reinterpret_cast<const float4*>(delta + r0 + 16 * h + 8 * g + 4 * c);
-                ls[8 * h + 4 * c] = v.x; ls[8 * h + 4 * c + 1] = v.y; ls[8 * h + 4 * c + 2] = v.z; ls[8 * h + 4 * c + 3] = v.w;
-                dl[8 * h + 4 * c] = w.x; dl[8 * h + 4 * c + 1] = w.y; dl[8 * h + 4 * c + 2] = w.z; dl[8 * h + 4 * c + 3] = w.w;
-            }
+        for (int ks = 0; ks < KS; ++ks) dp = M::mma(gn[ks], vbv[ks], dp);
+        if (more) fetch_rows(t + kW);
+        // only tiles on an edge of the band (or past the end of the sequence) need the element-wise mask
+        const bool edge = (r0 + 31 >= T) || (c0 + 31 >= T) || (p.causal && ((c0 + 31 > r0) || (r0 + 31 - c0 > p.k_diff)));
         float pr[16], ds[16];
+        if (edge) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int r = r0 + key_of(g, i);
-            const bool ok = pair_ok(T, p.causal, p.k_diff, r, a);
-            pr[i] = ok ? fast_exp2(fmaf(s[i], scale_log2, ba - ls[i])) : 0.f;
-            ds[i] = ok ? pr[i] * (dp[i] - dl[i]) : 0.f;
-            db += ds[i];
+            for (int i = 0; i < 16; ++i) {
+                const int r = r0 + key_of(g, i);
+                const bool ok = pair_ok(T, p.causal, p.k_diff, r, a);
+                pr[i] = ok ? fast_exp2(fmaf(s[i], scale_log2, ba - ls[i])) : 0.f;
+                ds[i] = ok ? pr[i] * (dp[i] - dl[i]) : 0.f;
+                db += ds[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                pr[i] = fast_exp2(fmaf(s[i], scale_log2, ba - ls[i]));
+                ds[i] = pr[i] * (dp[i] - dl[i]);
+                db += ds[i];
+            }
         }
+        if (more) fetch_stats(t + kW);
         v8 pb[2], dsb[2];
         pack16<E>(pr, pb);
         pack16<E>(ds, dsb);
@@ -486,10 +593,10 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
-                const size_t to = (size_t)(32 * dt + n) * Tp + r0 + 16 * kk + 8 * g;
-                acck[dt] = M::mma(ld8<E>(XT + to), dsb[kk], acck[dt]);
-                accv[dt] = M::mma(ld8<E>(GT + to), pb[kk], accv[dt]);
+                acck[dt] = M::mma(x2n[dt][kk], dsb[kk], acck[dt]);
+                accv[dt] = M::mma(g2n[dt][kk], pb[kk], accv[dt]);
             }
+        if (more) fetch_cols(t + kW);
     }
     db += __shfl_xor(db, 32, 64);
 
@@ -570,8 +677,9 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
                 *reinterpret_cast<v8*>(p.dv2 + off) = dv2;
                 *reinterpret_cast<v8*>(p.dr + off) = dr;
             }
+            *reinterpret_cast<v8*>(p.dr_p1 + tb + p1_index<D>(row, d0)) = dr;  // zeros for the padding rows
 #pragma unroll
-            for (int j = 0; j < 8; ++j) p.dr_t[tb + (size_t)(d0 + j) * Tp + row] = dr[j];
+            for (int j = 0; j < 8; ++j) p.dr_p2[tb + p2_index<D>(row, d0 + j)] = dr[j];
         }
     }
     if constexpr (LINK) {
@@ -589,39 +697,53 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
 }
 
 // --------------------------------------------------------------------------------------- prep
-// Transposed, zero padded [D][Tp] copies (U = SiLU(V1)), U row-major, and the padded per-row
-// vectors of the backward (LSE in log2 units, Delta = rowsum(dO * O)).  Null pointers are skipped.
+// Operand-packed copies of the inputs (U = SiLU(V1); rows past T are written as zeros), U row-major, and
+// the padded per-row vectors of the backward (LSE in log2 units, Delta = rowsum(dO * O)).  Null
+// pointers are skipped.
 template <typename E>
 struct PrepP {
     const E *v1, *k1, *k2, *q, *o, *d_o;
     const float* lse;
-    E *u, *ut, *k1t, *k2t, *qt, *dot;
+    E* u;                            // row-major
+    E *up1, *k1p1, *k2p1, *qp1, *dop1;  // packing P1
+    E *up2, *k1p2, *k2p2, *qp2, *dop2;  // packing P2
     float *lse2, *delta;
-    int T, Tp, D;
+    int T, Tp;
 };
 
-template <typename E>
+template <typename E, int D>
 __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
-    const int bh = blockIdx.y, j0 = blockIdx.x * 32, T = p.T, Tp = p.Tp, D = p.D;
+    using v8 = typename Mma<E>::v8;
+    const int bh = blockIdx.y, j0 = blockIdx.x * 32, T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp;
-    for (int idx = threadIdx.x; idx < D * 32; idx += 256) {
-        const int d = idx >> 5, j = j0 + (idx & 31);
+    // one 16-byte piece (8 consecutive d of one row) per step: it is one piece of P1 and 8 elements of P2
+    for (int idx = threadIdx.x; idx < 32 * (D / 8); idx += 256) {
+        const int j = j0 + idx / (D / 8), d0 = (idx % (D / 8)) * 8;
         const bool in = j < T;
-        const size_t off = base + (size_t)(in ? j : 0) * D + d, to = tb + (size_t)d * Tp + j;
-        if (p.ut) p.ut[to] = (E)(in ? silu_f((float)p.v1[off]) : 0.f);
-        if (p.k1t) p.k1t[to] = in ? p.k1[off] : (E)0.f;
-        if (p.k2t) p.k2t[to] = in ? p.k2[off] : (E)0.f;
-        if (p.qt) p.qt[to] = in ? p.q[off] : (E)0.f;
-        if (p.dot) p.dot[to] = in ? p.d_o[off] : (E)0.f;
-    }
-    if (p.u)
-        for (int idx = threadIdx.x; idx < D * 32; idx += 256) {
-            const int j = j0 + idx / D;
-            if (j < T) {
-                const size_t off = base + (size_t)j * D + idx % D;
-                p.u[off] = (E)silu_f((float)p.v1[off]);
+        const size_t off = base + (size_t)(in ? j : 0) * D + d0;
+        const size_t o1 = tb + p1_index<D>(j, d0);
+        auto emit = [&](const E* src, E* dst1, E* dst2, bool silu) {
+            if (!dst1 && !dst2 && !(silu && p.u)) return;
+            v8 x;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (E)0.f;
+            if (in) x = *reinterpret_cast<const v8*>(src + off);
+            if (silu) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (E)(in ? silu_f((float)x[e]) : 0.f);
+                if (p.u && in) *reinterpret_cast<v8*>(p.u + off) = x;
             }
-        }
+            if (dst1) *reinterpret_cast<v8*>(dst1 + o1) = x;
+            if (dst2)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) dst2[tb + p2_index<D>(j, d0 + e)] = x[e];
+        };
+        emit(p.v1, p.up1, p.up2, true);
+        emit(p.k1, p.k1p1, p.k1p2, false);
+        emit(p.k2, p.k2p1, p.k2p2, false);
+        if (p.q) emit(p.q, p.qp1, p.qp2, false);
+        if (p.d_o) emit(p.d_o, p.dop1, p.dop2, false);
+    }
     if (p.delta) {
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         for (int jj = wave; jj < 32; jj += 4) {
@@ -640,7 +762,9 @@ __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
 }
 
 struct Layout {
-    size_t u, ut, k1t, k2t, qt, dot, w, wt, dr, drt, r, dk2p, lse1, lse2, delta, delta1, total;
+    size_t up2, k1p1, k2p1, wp2, lse1;                                            // forward
+    size_t u, up1, k1p2, k2p2, qp1, qp2, dop1, dop2, w, wp1, dr, drp1, drp2, r, dk2p, lse2, delta, delta1;  // backward
+    size_t total;
 };
 Layout layout(int BH, int T, int D, bool bwd) {
     const size_t Tp = (size_t)(T + 31) / 32 * 32, n = (size_t)BH * T * D, nt = (size_t)BH * D * Tp, nv = (size_t)BH * Tp;
@@ -652,18 +776,25 @@ Layout layout(int BH, int T, int D, bool bwd) {
         off += bytes;
         return r;
     };
-    l.ut = take(nt * 2);
-    l.wt = take(nt * 2);
+    l.up2 = take(nt * 2);
+    l.k1p1 = take(nt * 2);
+    l.k2p1 = take(nt * 2);
+    l.wp2 = take(nt * 2);
     l.lse1 = take(nv * 4);
     if (bwd) {
         l.u = take(n * 2);
-        l.k1t = take(nt * 2);
-        l.k2t = take(nt * 2);
-        l.qt = take(nt * 2);
-        l.dot = take(nt * 2);
+        l.up1 = take(nt * 2);
+        l.k1p2 = take(nt * 2);
+        l.k2p2 = take(nt * 2);
+        l.qp1 = take(nt * 2);
+        l.qp2 = take(nt * 2);
+        l.dop1 = take(nt * 2);
+        l.dop2 = take(nt * 2);
         l.w = take(n * 2);
+        l.wp1 = take(nt * 2);
         l.dr = take(n * 2);
-        l.drt = take(nt * 2);
+        l.drp1 = take(nt * 2);
+        l.drp2 = take(nt * 2);
         l.r = take(n * 4);
         l.dk2p = take(n * 4);
         l.lse2 = take(nv * 4);
@@ -697,25 +828,27 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     if (e != hipSuccess) return e;
     const float sl2 = a.alpha * kLog2e;
 
-    if (!for_bwd) {  // the backward's prep kernel has already written U^T
+    if (!for_bwd) {  // the backward's prep kernel has already written these
         PrepP<E> pp{};
-        pp.v1 = (const E*)a.v1; pp.ut = (E*)(ws + l.ut);
-        pp.T = a.T; pp.Tp = Tp; pp.D = D;
-        hipLaunchKernelGGL(dps_prep_kernel<E>, grid, dim3(256), 0, st, pp);
+        pp.v1 = (const E*)a.v1; pp.k1 = (const E*)a.k1; pp.k2 = (const E*)a.k2;
+        pp.up2 = (E*)(ws + l.up2); pp.k1p1 = (E*)(ws + l.k1p1); pp.k2p1 = (E*)(ws + l.k2p1);
+        pp.T = a.T; pp.Tp = Tp;
+        hipLaunchKernelGGL((dps_prep_kernel<E, D>), grid, dim3(256), 0, st, pp);
     }
     // inner: rows K2[t], keys K1, values U; R (fp32, backward only), W = R * V2 and W^T, lse1 (log2)
     AttnFwdP<E> p{};
-    p.x = (const E*)a.k2; p.k = (const E*)a.k1; p.vt = (const E*)(ws + l.ut); p.mul = (const E*)a.v2;
+    p.x = (const E*)a.k2; p.kp = (const E*)(ws + l.k1p1); p.vp2 = (const E*)(ws + l.up2); p.mul = (const E*)a.v2;
     p.out_f32 = for_bwd ? (float*)(ws + l.r) : nullptr;
     p.outm = for_bwd ? (E*)(ws + l.w) : nullptr;
-    p.outm_t = (E*)(ws + l.wt);
+    p.outm_p1 = for_bwd ? (E*)(ws + l.wp1) : nullptr;
+    p.outm_p2 = (E*)(ws + l.wp2);
     p.lse = (float*)(ws + l.lse1); p.lse_stride = Tp; p.lse_scale = 1.0f;
     p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff;
     hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, p);
     if (for_bwd) return hipGetLastError();
     // outer: rows Q[q], keys K2 with bias lse1, values W; O and LSE (natural log)
     AttnFwdP<E> o{};
-    o.x = (const E*)a.q; o.k = (const E*)a.k2; o.vt = (const E*)(ws + l.wt); o.bias = (const float*)(ws + l.lse1);
+    o.x = (const E*)a.q; o.kp = (const E*)(ws + l.k2p1); o.vp2 = (const E*)(ws + l.wp2); o.bias = (const float*)(ws + l.lse1);
     o.out = (E*)a.o_out; o.lse = a.lse_out; o.lse_stride = a.T; o.lse_scale = kLn2;
     o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T;
     hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, o);
@@ -739,11 +872,14 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     PrepP<E> pp{};
     pp.v1 = (const E*)a.v1; pp.k1 = (const E*)a.k1; pp.k2 = (const E*)a.k2; pp.q = (const E*)a.q;
     pp.o = (const E*)a.o; pp.d_o = (const E*)a.d_o; pp.lse = a.lse_in;
-    pp.u = (E*)(ws + l.u); pp.ut = (E*)(ws + l.ut); pp.k1t = (E*)(ws + l.k1t); pp.k2t = (E*)(ws + l.k2t);
-    pp.qt = (E*)(ws + l.qt); pp.dot = (E*)(ws + l.dot);
+    pp.u = (E*)(ws + l.u);
+    pp.up1 = (E*)(ws + l.up1); pp.k1p1 = (E*)(ws + l.k1p1); pp.k2p1 = (E*)(ws + l.k2p1);
+    pp.qp1 = (E*)(ws + l.qp1); pp.dop1 = (E*)(ws + l.dop1);
+    pp.up2 = (E*)(ws + l.up2); pp.k1p2 = (E*)(ws + l.k1p2); pp.k2p2 = (E*)(ws + l.k2p2);
+    pp.qp2 = (E*)(ws + l.qp2); pp.dop2 = (E*)(ws + l.dop2);
     pp.lse2 = (float*)(ws + l.lse2); pp.delta = (float*)(ws + l.delta);
-    pp.T = a.T; pp.Tp = Tp; pp.D = D;
-    hipLaunchKernelGGL(dps_prep_kernel<E>, grid, dim3(256), 0, st, pp);
+    pp.T = a.T; pp.Tp = Tp;
+    hipLaunchKernelGGL((dps_prep_kernel<E, D>), grid, dim3(256), 0, st, pp);
     // recompute the inner pass: R, W, W^T, lse1
     e = run_fwd<E, D>(a, st, true);
     if (e != hipSuccess) return e;
@@ -751,20 +887,24 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     // outer pass: X = Q, G = dO, K = K2 (bias lse1), V = W
     AttnBwdP<E> o{};
     o.x = (const E*)a.q; o.g = (const E*)a.d_o; o.k = (const E*)a.k2; o.v = (const E*)(ws + l.w);
-    o.kt = (const E*)(ws + l.k2t); o.xt = (const E*)(ws + l.qt); o.gt = (const E*)(ws + l.dot);
+    o.kp = (const E*)(ws + l.k2p1); o.vp = (const E*)(ws + l.wp1); o.kp2 = (const E*)(ws + l.k2p2);
+    o.xp = (const E*)(ws + l.qp1); o.gp = (const E*)(ws + l.dop1);
+    o.xp2 = (const E*)(ws + l.qp2); o.gp2 = (const E*)(ws + l.dop2);
     o.bias = (const float*)(ws + l.lse1); o.lse2 = (const float*)(ws + l.lse2); o.delta = (const float*)(ws + l.delta);
     o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T;
     o.dx = (E*)a.dq;
     o.dk_f32 = (float*)(ws + l.dk2p);
     o.r_f32 = (const float*)(ws + l.r); o.v2 = (const E*)a.v2; o.dv2 = (E*)a.dv2;
-    o.dr = (E*)(ws + l.dr); o.dr_t = (E*)(ws + l.drt); o.delta1 = (float*)(ws + l.delta1);
+    o.dr = (E*)(ws + l.dr); o.dr_p1 = (E*)(ws + l.drp1); o.dr_p2 = (E*)(ws + l.drp2); o.delta1 = (float*)(ws + l.delta1);
     hipLaunchKernelGGL(krow, grid, dim3(64 * kW), row_smem<D>(), st, o);
     hipLaunchKernelGGL(kcol_link, grid, dim3(64 * kW), col_smem<D>(), st, o);
 
     // inner pass: X = K2, G = dR, K = K1, V = U
     AttnBwdP<E> i{};
     i.x = (const E*)a.k2; i.g = (const E*)(ws + l.dr); i.k = (const E*)a.k1; i.v = (const E*)(ws + l.u);
-    i.kt = (const E*)(ws + l.k1t); i.xt = (const E*)(ws + l.k2t); i.gt = (const E*)(ws + l.drt);
+    i.kp = (const E*)(ws + l.k1p1); i.vp = (const E*)(ws + l.up1); i.kp2 = (const E*)(ws + l.k1p2);
+    i.xp = (const E*)(ws + l.k2p1); i.gp = (const E*)(ws + l.drp1);
+    i.xp2 = (const E*)(ws + l.k2p2); i.gp2 = (const E*)(ws + l.drp2);
     i.lse2 = (const float*)(ws + l.lse1); i.delta = (const float*)(ws + l.delta1);
     i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff;
     i.addend = (const float*)(ws + l.dk2p); i.dx = (E*)a.dk2;
