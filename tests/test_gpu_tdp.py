@@ -301,6 +301,30 @@ def test_mfma_backward_windows_bf16(seq_len, windows, D):
             assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_mfma_windows_fp16_batched(D):
+    """fp16, several batch entries and heads, odd window sizes: forward and all five gradients."""
+    windows = (33, 47, 9, 12)
+    inputs = orc.make_inputs(2, 3, 150, D, torch.float16, seed=77 + D)
+    alpha = 1 / math.sqrt(D)
+    z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
+    out, g = util.run_tdp(inputs, alpha, True, windows, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+        assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
+
+
+def test_mfma_windows_ignored_without_causal():
+    """causal=False ignores the windows (as the naive reference module does)."""
+    inputs = orc.make_inputs(1, 2, 100, 64, torch.bfloat16, seed=78)
+    a, ga = util.run_tdp(inputs, 1 / 8, False, (5, 3, 4, 1), flags=FORCE_MFMA)
+    b, gb = util.run_tdp(inputs, 1 / 8, False, flags=FORCE_MFMA)
+    assert torch.equal(a, b)
+    for x, y in zip(ga, gb):
+        util.assert_close("grad", x, y, **LOWP)
+
+
 def test_mfma_backward_d128_fp16_matches_generic():
     """Head dimension 128, fp16, several batch entries and heads: MFMA kernels against the fp32 kernels."""
     inputs = orc.make_inputs(2, 5, 150, 128, torch.float16, seed=33)
