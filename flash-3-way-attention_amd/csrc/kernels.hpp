@@ -55,7 +55,7 @@ size_t mfma_tdp_fwd_workspace(int BH, int T, int D);
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st);
 
-// 16-bit MFMA triple-dot backward (D = 64 or 128).
+// 16-bit MFMA triple-dot backward (any mask; D = 32, 64 or 128).
 struct MfmaBwdArgs {
     const void *q, *k1, *k2, *v1, *v2, *o, *d_o;
     const float* lse;

@@ -549,10 +549,15 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     void (*kern_dq)(BwdParams<E>);
     void (*kern_nodq)(BwdParams<E>);
     int nthreads = 512, col_parts = 1;
-    if (a.windowed) {
+    if constexpr (D == 32) {
+        // one shape, the banded instantiation for every mask (full windows are windows of T)
+        smem = bwdg_smem(32, 8, 32, true);
+        kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true>;
+        kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true>;
+    } else if (a.windowed) {
         smem = bwdg_smem(D, 8, 64, true);
-        kern_dq = tdp_bwd_rows_general_kernel<E, D, true, 8, 64, true>;
-        kern_nodq = tdp_bwd_rows_general_kernel<E, D, false, 8, 64, true>;
+        kern_dq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), true, 8, 64, true>;
+        kern_nodq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), false, 8, 64, true>;
         col_parts = D / 64;
     } else if constexpr (D == 128) {
         // One wave per SIMD with all 128 columns is ~10 % faster once the grid fills the chip several times
@@ -575,8 +580,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
             nthreads = 256;
         }
     } else {
-        smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * D + 2 * 32 * (D + 8) + 2 * (D / 32) * 64 * 16) +
-               4 * (size_t)(4 * 32 * D);
+        smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * 64 + 2 * 32 * (64 + 8) + 2 * (64 / 32) * 64 * 16) +
+               4 * (size_t)(4 * 32 * 64);
         kern_dq = tdp_bwd_rows_kernel<E, 64, true>;
         kern_nodq = tdp_bwd_rows_kernel<E, 64, false>;
     }
@@ -613,9 +618,10 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
 }
 
 size_t mfma_tdp_bwd_workspace(int BH, int T, int D) { return bwd_layout(BH, T, D).total; }
-bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
+bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
 
 hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st) {
+    if (a.D == 32) return a.is_bf16 ? launch_bwd<__bf16, 32>(a, st) : launch_bwd<_Float16, 32>(a, st);
     if (a.D == 64) return a.is_bf16 ? launch_bwd<__bf16, 64>(a, st) : launch_bwd<_Float16, 64>(a, st);
     if (a.D == 128) return a.is_bf16 ? launch_bwd<__bf16, 128>(a, st) : launch_bwd<_Float16, 128>(a, st);
     return hipErrorInvalidValue;

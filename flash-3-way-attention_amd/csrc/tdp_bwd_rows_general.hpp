@@ -1,6 +1,6 @@
 // Triple-dot-product trittention backward on MFMA: the general form of the rows kernel (included by
-// tdp_bwd_mfma.hip after BwdParams).  It serves head dimension 128 and, for head dimensions 64 and
-// 128, windowed causal masks (WIN): rounds and steps then cover the band only, and a key outside the
+// tdp_bwd_mfma.hip after BwdParams).  It serves head dimensions 32 and 128 and, for head dimensions
+// 64 and 128, windowed causal masks (WIN): rounds and steps then cover the band only, and a key outside the
 // window of its (q, k) is masked like one past the causal bound.
 //
 // Same decomposition as tdp_bwd_rows_kernel (rows = one K2/V2 row k per wave and round, K1 / U
@@ -17,7 +17,8 @@
 // as 64 x 64 tiles (tile row = 32 * (d / 64) + key, the swizzle of direct_lds.hpp), K1^T and U^T
 // of the workgroup's columns as compact [NCOL d][32 keys] tiles; three buffers, fetched
 // direct-to-LDS two steps ahead, one workgroup barrier per step.  D = 64 (WIN only; the full-window
-// case has its own kernel): NW = 8, NCOL = 64, the row tiles have 32 rows.
+// case has its own kernel): NW = 8, NCOL = 64, the row tiles have 32 rows.  D = 32: NW = 8,
+// NCOL = 32, the row tiles have 32 rows of 64 bytes (swizzled like the transposed tiles).
 #pragma once
 
 namespace tritt {
@@ -55,9 +56,11 @@ __device__ __forceinline__ typename Mma<E>::v8 offset_operand(float x, int g) {
 __device__ __forceinline__ constexpr int swz_t(int r) { return (r >> 2) & 3; }
 
 constexpr int bwdg_stage_bytes(int d, int ncol) { return 2 * d * 64 + 2 * ncol * 64; }
+// rows of a round buffer: the round's NW rows, or what one 1 KB load brings in if that is more
+constexpr int bwdg_round_rows(int d, int nw) { return nw > 512 / d ? nw : 512 / d; }
 constexpr size_t bwdg_smem(int d, int nw, int ncol, bool with_dq) {
     return 3 * (size_t)bwdg_stage_bytes(d, ncol)               // stage buffers
-           + 2 * (2 * nw * d * 2)                               // K2 / V2 rows of two rounds
+           + 2 * (2 * bwdg_round_rows(d, nw) * d * 2)           // K2 / V2 rows of two rounds
            + 2 * (32 * (d + 8) * 2)                             // Q and dO tiles
            + (with_dq ? (nw / 2) * (32 * ncol * 4) : 0)         // dQ slices (one per pair of waves)
            + (ncol == 64 ? 2 * (2 * 64 * 16 * 2) : 0);          // Q and dO in accumulator layout (NCOL = 64)
@@ -75,15 +78,19 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     constexpr int NBUF = 3, LW = NBLK / NW;  // stage buffers; direct loads per wave per stage
     constexpr int STAGE = bwdg_stage_bytes(D, NCOL) / 2;  // elements
     constexpr bool EPI_TILES = NCOL == 64;   // Q / dO kept a second time in accumulator layout
-    static_assert(D == 64 || D == 128, "head dimension");
-    static_assert((NW == 8 && NCOL == 64) || (D == 128 && NW == 4 && NCOL == 128), "workgroup shapes");
+    constexpr int RW = D < 64 ? D : 64;      // elements of a row-major tile row (D = 128: two rows per key)
+    constexpr int CPR = RW / 8, RPB = 64 / CPR;  // 16-byte chunks per tile row, tile rows per 1 KB block
+    constexpr int RR = bwdg_round_rows(D, NW);   // rows of a round buffer
+    static_assert(D == 32 || D == 64 || D == 128, "head dimension");
+    static_assert((NW == 8 && NCOL == 64 && D >= 64) || (D == 128 && NW == 4 && NCOL == 128) ||
+                  (D == 32 && NW == 8 && NCOL == 32), "workgroup shapes");
     static_assert(NBLK % NW == 0, "whole blocks per wave");
 
     extern __shared__ __align__(16) char smem[];
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows 4096 | U rows 4096 | K1^T 2048 | U^T 2048]
-    E* sKr = sStage + NBUF * STAGE;          // [2][NW][D]
-    E* sVr = sKr + 2 * NW * D;
-    E* sQb = sVr + 2 * NW * D;               // [BQ][LDK]
+    E* sKr = sStage + NBUF * STAGE;          // [2][RR][D]
+    E* sVr = sKr + 2 * RR * D;
+    E* sQb = sVr + 2 * RR * D;               // [BQ][LDK]
     E* sOb = sQb + BQ * LDK;
     float* sDQall = reinterpret_cast<float*>(sOb + BQ * LDK);  // [NW/2][BQ * DH], accumulator layout (WITH_DQ)
     float* sDQ = sDQall + (wave_of(threadIdx.x) >> 1) * (BQ * DH);
@@ -138,8 +145,8 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     for (int c = 0; c < LW; ++c) {
         const int b = wave * LW + c;
         if (b < 2 * RB) {
-            const int R = (b % RB) * 8 + (lane >> 3), hh = R >> 5, r = R & 31;
-            const int chunk = (lane & 7) ^ swz_perm(r);
+            const int R = (b % RB) * RPB + lane / CPR, hh = R >> 5, r = R & 31;
+            const int chunk = (lane % CPR) ^ (D == 32 ? swz_t(r) : swz_perm(r));
             gsrc[c] = uniform_ptr((b < RB ? p.st_k : p.st_v) + base);
             rowkey[c] = r;
             rowrest[c] = (unsigned)(hh * 64 + chunk * 8) * 2;
@@ -168,16 +175,16 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     };
     // the round's K2 / V2 rows NW m .. NW m + NW - 1: one load moves 1 KB = RPL rows
     auto issue_round = [&](int m, int buf) {
-        constexpr int RPL = 512 / D, LPR = D / 8;  // rows per load, lanes per row
-        constexpr int LR = NW / RPL;               // loads per tensor
-        static_assert(LR >= 1 && 2 * LR <= NW, "round loader");
+        constexpr int RPL = 512 / D, LPR = D / 8;    // rows per load, lanes per row
+        constexpr int LR = NW > RPL ? NW / RPL : 1;  // loads per tensor (D = 32: one load brings 16 rows, 8 are used)
+        static_assert(2 * LR <= NW, "round loader");
         if (wave < 2 * LR) {
             int ln = lane;
             asm volatile("" : "+v"(ln));
             const int part = wave % LR;
             const bool second = wave >= LR;
             const unsigned off = (unsigned)min(m * NW + part * RPL + ln / LPR, T - 1) * (D * 2) + (ln % LPR) * 16;
-            direct_load_16(uniform_ptr(second ? V2 : K2), off, (second ? sVr : sKr) + buf * NW * D + part * RPL * D);
+            direct_load_16(uniform_ptr(second ? V2 : K2), off, (second ? sVr : sKr) + buf * RR * D + part * RPL * D);
         }
     };
 
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     const v8 a_ones = ones_operand<E>(g);
     const v8 b_lse = offset_operand<E>(lse2, g), b_delta = offset_operand<E>(delta, g);
     const int krow_off = key_of_row(n);
-    const int fperm = swz_perm(krow_off);
+    const int fperm = D == 32 ? swz_t(krow_off) : swz_perm(krow_off);
 
     for (int m = m_first; m < nrounds; ++m) {
         const int mb = m & 1;
@@ -262,8 +269,8 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const int off = ks * 16 + g * 8;
-                    const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * NW + wave) * D + off);
-                    const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * NW + wave) * D + off);
+                    const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * RR + wave) * D + off);
+                    const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * RR + wave) * D + off);
                     const v8 qv = *reinterpret_cast<const v8*>(sQb + n * LDK + off);
                     const v8 dv = *reinterpret_cast<const v8*>(sOb + n * LDK + off);
                     v8 a, b;
@@ -299,7 +306,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             auto load_rows = [&](int first) {
 #pragma unroll
                 for (int ks = first; ks < min(first + 4, KS); ++ks) {
-                    const int roff = ((ks >> 2) * 32 + krow_off) * 64 + ((((ks & 3) * 2 + g) ^ fperm) * 8);
+                    const int roff = ((ks >> 2) * 32 + krow_off) * RW + ((((ks & 3) * 2 + g) ^ fperm) * 8);
                     ak[ks] = *reinterpret_cast<const v8*>(sK1 + roff);
                     au[ks] = *reinterpret_cast<const v8*>(sU + roff);
                 }
@@ -367,7 +374,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             };
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                grad(0, r);
+                if (r < 2 * DT) grad(0, r);
                 __builtin_amdgcn_sched_barrier(0);
                 softmax_pair(4 + r);
                 __builtin_amdgcn_sched_barrier(0);
@@ -383,7 +390,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
         [[maybe_unused]] auto add_dq = [&]() {  // slice += Yq (.) K2[k]
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const float kd = (float)sKr[(mb * NW + wave) * D + c0 + dt * 32 + n];
+                const float kd = (float)sKr[(mb * RR + wave) * D + c0 + dt * 32 + n];
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
                     float4* slot4 = reinterpret_cast<float4*>(sDQ + ((dt * 4 + i4) * 64 + lane) * 4);
@@ -442,8 +449,9 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
         // dQ: sum the pairs' slices; a thread takes four consecutive accumulator registers (= four consecutive
         // query rows of one column) at a time
 #pragma unroll
-        for (int t = 0; t < BQ * DH / 4 / NTH; ++t) {
+        for (int t = 0; t < (BQ * DH / 4 + NTH - 1) / NTH; ++t) {
             const int idx4 = t * NTH + tid, slot4 = idx4 >> 6, ln = idx4 & 63;
+            if (idx4 >= BQ * DH / 4) break;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
             for (int sl = 0; sl < NW / 2; ++sl) {

@@ -284,7 +284,7 @@ def test_mfma_backward_d128_bf16(seq_len, causal, shape, monkeypatch):
             assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
 
 
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("windows", WINDOWS)
 @pytest.mark.parametrize("seq_len", [33, 100, 300])
 def test_mfma_backward_windows_bf16(seq_len, windows, D):
@@ -323,6 +323,22 @@ def test_mfma_windows_ignored_without_causal():
     assert torch.equal(a, b)
     for x, y in zip(ga, gb):
         util.assert_close("grad", x, y, **LOWP)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("seq_len", [1, 33, 100, 256, 300])
+def test_mfma_backward_d32_bf16(seq_len, causal):
+    """Head dimension 32 (row tiles of 64 bytes): forward and all five gradients."""
+    print(f"case mfma bwd D=32 T={seq_len} causal={causal}", flush=True)
+    inputs = orc.make_inputs(2, 3, seq_len, 32, torch.bfloat16, seed=seq_len + 9)
+    alpha = 1 / math.sqrt(32)
+    z, _, grads = util.oracle_tdp(inputs, alpha, causal)
+    out, g = util.run_tdp(inputs, alpha, causal, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+        if seq_len > 1:
+            assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
 
 
 def test_mfma_backward_d128_fp16_matches_generic():
