@@ -264,8 +264,8 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     const float inv = 1.0f / ll;
     if (dg == 0 && row < T) p.lse[(size_t)bh * p.lse_stride + row] = (mm + fast_log2(ll)) * p.lse_scale;
 #pragma unroll
-    for (int c = 0; c < D / 64; ++c) {
-        const int d0 = dg * (D / 8) + 8 * c;
+    for (int c = dg; c < D / 8; c += 8) {  // 16-byte pieces dg, dg + 8, ... of the row
+        const int d0 = 8 * c;
         float o[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -451,8 +451,8 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
     const int rr = tid & 31, dg = tid >> 5, row = r0 + rr;
     if (row >= T) return;
 #pragma unroll
-    for (int c = 0; c < D / 64; ++c) {
-        const int d0 = dg * (D / 8) + 8 * c;
+    for (int c = dg; c < D / 8; c += 8) {  // 16-byte pieces dg, dg + 8, ... of the row
+        const int d0 = 8 * c;
         const size_t off = base + (size_t)row * D + d0;
         v8 ov;
 #pragma unroll
@@ -607,8 +607,8 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     __syncthreads();
     if (row < T) {
 #pragma unroll
-        for (int c = 0; c < D / 64; ++c) {
-            const int d0 = dg * (D / 8) + 8 * c;
+        for (int c = dg; c < D / 8; c += 8) {
+            const int d0 = 8 * c;
             const size_t off = base + (size_t)row * D + d0;
             float o[8];
 #pragma unroll
@@ -636,8 +636,8 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     __syncthreads();
     float part = 0.f;
 #pragma unroll
-    for (int c = 0; c < D / 64; ++c) {
-        const int d0 = dg * (D / 8) + 8 * c;
+    for (int c = dg; c < D / 8; c += 8) {  // 16-byte pieces dg, dg + 8, ... of the row
+        const int d0 = 8 * c;
         const size_t off = base + (size_t)row * D + d0;
         float o[8];
 #pragma unroll
@@ -916,17 +916,19 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
 
 }  // namespace
 
-bool mfma_dps_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 64 || D == 128); }
+bool mfma_dps_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
 size_t mfma_dps_fwd_workspace(int BH, int T, int D) { return layout(BH, T, D, false).total; }
 size_t mfma_dps_bwd_workspace(int BH, int T, int D) { return layout(BH, T, D, true).total; }
 
 hipError_t mfma_dps_fwd(const MfmaDpsArgs& a, hipStream_t st) {
+    if (a.D == 32) return a.is_bf16 ? run_fwd<__bf16, 32>(a, st, false) : run_fwd<_Float16, 32>(a, st, false);
     if (a.D == 64) return a.is_bf16 ? run_fwd<__bf16, 64>(a, st, false) : run_fwd<_Float16, 64>(a, st, false);
     if (a.D == 128) return a.is_bf16 ? run_fwd<__bf16, 128>(a, st, false) : run_fwd<_Float16, 128>(a, st, false);
     return hipErrorInvalidValue;
 }
 
 hipError_t mfma_dps_bwd(const MfmaDpsArgs& a, hipStream_t st) {
+    if (a.D == 32) return a.is_bf16 ? run_bwd<__bf16, 32>(a, st) : run_bwd<_Float16, 32>(a, st);
     if (a.D == 64) return a.is_bf16 ? run_bwd<__bf16, 64>(a, st) : run_bwd<_Float16, 64>(a, st);
     if (a.D == 128) return a.is_bf16 ? run_bwd<__bf16, 128>(a, st) : run_bwd<_Float16, 128>(a, st);
     return hipErrorInvalidValue;

@@ -72,7 +72,7 @@ size_t mfma_tdp_bwd_workspace(int BH, int T, int D);
 bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st);
 
-// 16-bit MFMA dot-product-sum (two chained banded attentions; D = 64 or 128).
+// 16-bit MFMA dot-product-sum (two chained banded attentions; D = 32, 64 or 128).
 struct MfmaDpsArgs {
     const void *q, *k1, *k2, *v1, *v2;
     void* o_out;          // forward output

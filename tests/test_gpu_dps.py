@@ -94,7 +94,7 @@ def test_config4_bf16_T1024():
 
 @pytest.mark.parametrize("seq_len", [1, 33, 100, 257])
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 def test_mfma_ragged_lengths(seq_len, causal, D):
     """16-bit tensors take the MFMA kernels (forced, so a silent fall-back would fail)."""
     inputs = orc.make_inputs(1, 2, seq_len, D, torch.bfloat16, seed=20 + seq_len)
@@ -109,9 +109,10 @@ def test_mfma_ragged_lengths(seq_len, causal, D):
             assert util.rel_err(a, b) <= 3e-2, (name, util.rel_err(a, b))
 
 
+@pytest.mark.parametrize("D", [32, 64])
 @pytest.mark.parametrize("k_diff", [0, 3, 40, 1000])
-def test_mfma_k_diff_band(k_diff):
-    inputs = orc.make_inputs(2, 2, 150, 64, torch.float16, seed=31)
+def test_mfma_k_diff_band(k_diff, D):
+    inputs = orc.make_inputs(2, 2, 150, D, torch.float16, seed=31)
     z, lse, grads = util.oracle_dps(inputs, 1 / 8, True, k_diff)
     out, m, g = util.run_dps(inputs, 1 / 8, True, k_diff, flags=2)
     util.assert_close("out", out, z, **LOWP)
