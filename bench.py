@@ -114,6 +114,7 @@ def main():
                          "tdp: triple-dot forward+backward at --B --H --T --D with --windows (secondary shapes: "
                          "D=128, windowed masks)")
     ap.add_argument("--windows", default="", help="k1_window,k2_window,kk_left,kk_right for --mode tdp (empty: full)")
+    ap.add_argument("--dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="tensor type for --mode tdp")
     ap.add_argument("--B", type=int, default=4)
     ap.add_argument("--H", type=int, default=8)
     ap.add_argument("--T", type=int, default=1024)
@@ -186,7 +187,8 @@ def main():
                           "io_gbs_fwd": (6 * B * H * T * D * 2) / ms_f / 1e6,
                           "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} bf16 causal"}}), flush=True)
         return
-    q, k1, k2, v1, v2, do = (t.to(dev) for t in orc.make_inputs(B, H, T, D, torch.bfloat16, seed=0))
+    tdtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype if args.mode == "tdp" else "bf16"]
+    q, k1, k2, v1, v2, do = (t.to(dev) for t in orc.make_inputs(B, H, T, D, tdtype, seed=0))
     leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
     kw = dict(softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True)
 
@@ -220,7 +222,7 @@ def main():
         ms_bwd = time_events(bwd_only, args.steps, args.warmup, torch)
         print(json.dumps({"metric": "triple-dot trittention fwd / bwd", "unit": "ms", "fwd_ms": ms_fwd, "bwd_ms": ms_bwd,
                           "fwd_tflops": f_fwd / ms_fwd / 1e9, "bwd_tflops": f_bwd / ms_bwd / 1e9, "valid_triples": n,
-                          "config": {"workload": f"triple-dot fwd+bwd B={B} H={H} T={T} D={D} bf16 causal",
+                          "config": {"workload": f"triple-dot fwd+bwd B={B} H={H} T={T} D={D} {args.dtype} causal",
                                      "windows": win}}), flush=True)
         return
 
