@@ -1,5 +1,6 @@
 // C ABI of libtrittention_hip.so: argument checks, scratch layout, dispatch.
 // Declarations and the contract of each entry point: include/trittention_hip.h.
+#include <cstdint>
 #include "../../include/trittention_hip.h"
 
 #include "common.hpp"
@@ -276,6 +277,13 @@ bool any_null(std::initializer_list<const void*> ps) {
     return false;
 }
 
+// the kernels move 16 bytes per lane: every [B,H,T,D] tensor must start on a 16-byte boundary
+bool any_misaligned(std::initializer_list<const void*> ps) {
+    for (const void* p : ps)
+        if (reinterpret_cast<uintptr_t>(p) & 15) return true;
+    return false;
+}
+
 }  // namespace
 }  // namespace tritt
 
@@ -288,7 +296,7 @@ int tritt_version(void) { return 100; }
 const char* tritt_status_string(int status) {
     switch (status) {
         case TRITT_OK: return "ok";
-        case TRITT_ERR_INVALID: return "invalid argument (null pointer, non-positive size, negative window or unknown dtype)";
+        case TRITT_ERR_INVALID: return "invalid argument (null or misaligned pointer, non-positive size, negative window or unknown dtype)";
         case TRITT_ERR_HEAD_DIM: return "head dimension must be 16, 32, 64 or 128";
         case TRITT_ERR_WORKSPACE: return "workspace missing or too small";
         case TRITT_ERR_UNSUPPORTED: return "requested implementation does not support this configuration";
@@ -315,6 +323,7 @@ int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1,
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o})) return TRITT_ERR_INVALID;
     if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
     const bool mfma = use_mfma_fwd(T, D, dtype, causal, w1, w2, kl, kr, flags);
@@ -355,6 +364,7 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
     if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
     const bool mfma = use_mfma_bwd(T, D, dtype, causal, w1, w2, kl, kr, flags);
@@ -392,6 +402,7 @@ int tritt_dps_fwd(const void* q, const void* k1, const void* k2, const void* v1,
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o})) return TRITT_ERR_INVALID;
     if (causal && k_diff < 0) return TRITT_ERR_INVALID;
     const bool mfma = use_mfma_dps(D, dtype, flags);
     if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;
@@ -426,6 +437,7 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
     if (causal && k_diff < 0) return TRITT_ERR_INVALID;
     const bool mfma = use_mfma_dps(D, dtype, flags);
     if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;

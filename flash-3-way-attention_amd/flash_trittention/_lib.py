@@ -82,6 +82,15 @@ def require_gpu(t: torch.Tensor, what: str):
                            "this library has no CPU implementation")
 
 
+def dense(t):
+    """Contiguous and 16-byte aligned (what the library requires of every [B,H,T,D] tensor): a
+    contiguous view that starts in the middle of a storage is copied."""
+    t = t.contiguous()
+    if t.data_ptr() % 16:
+        t = t.clone(memory_format=torch.contiguous_format)
+    return t
+
+
 def ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 

@@ -35,7 +35,7 @@ class TrittentionTritonFunction(torch.autograd.Function):
             raise ValueError(f"head_dim must be one of 16, 32, 64, 128, got {D}")
         code = _lib.dtype_code(q.dtype)
         _lib.require_gpu(q, "TrittentionTriton")
-        q, k1, k2, v1, v2 = (t.contiguous() for t in (q, k1, k2, v1, v2))
+        q, k1, k2, v1, v2 = (_lib.dense(t) for t in (q, k1, k2, v1, v2))
         k_diff = T if k_diff is None else int(k_diff)
         flags = TrittentionTritonFunction.impl_flags
         lib = _lib.lib()
@@ -62,7 +62,7 @@ class TrittentionTritonFunction(torch.autograd.Function):
         assert grad_output.shape == o.shape, f"Shape mismatch: O={o.shape}, dO={grad_output.shape}"
         assert o.device == grad_output.device, "O and dO must be on the same device"
         assert o.dtype == grad_output.dtype, "O and dO must have the same dtype"
-        grad_output = grad_output.contiguous()
+        grad_output = _lib.dense(grad_output)
         lib = _lib.lib()
         code = _lib.dtype_code(q.dtype)
         dq, dk1, dk2, dv1, dv2 = (torch.empty_like(q) for _ in range(5))

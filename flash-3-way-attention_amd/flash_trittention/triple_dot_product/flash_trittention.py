@@ -42,7 +42,7 @@ class FlashTrittention(torch.autograd.Function):
         _validate(Q, (("K1", K1), ("K2", K2), ("V1", V1), ("V2", V2)))
         _lib.require_gpu(Q, "flash_trittention")
         B, H, T, D = Q.shape
-        Q, K1, K2, V1, V2 = (t.contiguous() for t in (Q, K1, K2, V1, V2))
+        Q, K1, K2, V1, V2 = (_lib.dense(t) for t in (Q, K1, K2, V1, V2))
         k1_window, k2_window, kk_left, kk_right = process_masking_variables(T, k1_window, k2_window, kk_left, kk_right)
         causal = bool(causal)
         flags = FlashTrittention.impl_flags
@@ -72,7 +72,7 @@ class FlashTrittention(torch.autograd.Function):
         B, H, T, D = Q.shape
         if dO.dtype != Q.dtype:
             dO = dO.to(Q.dtype)
-        dO = dO.contiguous()
+        dO = _lib.dense(dO)
         k1_window, k2_window, kk_left, kk_right = ctx.windows
         lib = _lib.lib()
         code = _lib.dtype_code(Q.dtype)

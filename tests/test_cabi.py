@@ -57,6 +57,10 @@ def test_argument_rejection_happens_before_any_launch():
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 1, null) == -3  # no workspace
     assert lib.tritt_dps_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, 16, null, 0, 0, null) == -3
     assert lib.tritt_dps_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, -2, one, 1 << 30, 0, null) == -1
+    odd = ctypes.c_void_p(258)  # not on a 16-byte boundary
+    assert lib.tritt_tdp_fwd(odd, *args7[1:], 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
+    assert lib.tritt_dps_fwd(*args7[:3], odd, *args7[4:], 1, 1, 16, 32, 0, 0.1, 1, 16, null, 0, 0, null) == -1
+    assert b"misaligned" in lib.tritt_status_string(-1)
 
 
 def test_python_host_validation_matches_reference_errors():

@@ -315,6 +315,24 @@ def test_mfma_windows_fp16_batched(D):
         assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
 
 
+def test_unaligned_views_are_copied():
+    """Contiguous views that start in the middle of a storage (2-byte aligned) are accepted: the host side
+    copies them to aligned memory before the library sees them."""
+    inputs = orc.make_inputs(1, 2, 70, 64, torch.bfloat16, seed=79)
+    z, _, grads = util.oracle_tdp(inputs, 1 / 8, True)
+    shifted = []
+    for t in inputs:
+        buf = torch.empty(t.numel() + 1, dtype=t.dtype, device="cuda")
+        view = buf[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 != 0 and view.is_contiguous()
+        shifted.append(view)
+    out, g = util.run_tdp(shifted, 1 / 8, True, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+
+
 def test_mfma_windows_ignored_without_causal():
     """causal=False ignores the windows (as the naive reference module does)."""
     inputs = orc.make_inputs(1, 2, 100, 64, torch.bfloat16, seed=78)
