@@ -166,3 +166,35 @@ def test_rejects_mismatched_shapes():
     q, k1, k2, v1, v2, _ = (t.cuda() for t in orc.make_inputs(2, 2, 32, 32))
     with pytest.raises(ValueError):
         TrittentionTriton()(q, k1, k2, v1, v2[:, :, :16, :].contiguous())
+
+
+# ------------------------------------------------- full-size properties (config 4: B=4 H=8 T=1024 D=64 bf16)
+def test_config4_heads_are_independent_bitwise():
+    """Every output element has one owner (no atomics): permuting the (batch, head) slices permutes
+    the output, the LSE and all five gradients bit for bit."""
+    inputs = orc.make_inputs(4, 8, 1024, 64, torch.bfloat16, seed=41)
+    out, m, g = util.run_dps(inputs, 1 / 8, True, 1024)
+    perm = torch.randperm(32, generator=torch.Generator().manual_seed(2))
+    shuffled = [t.reshape(32, 1024, 64)[perm].reshape(4, 8, 1024, 64).contiguous() for t in inputs]
+    out2, m2, g2 = util.run_dps(shuffled, 1 / 8, True, 1024)
+    inv = torch.argsort(perm)
+    unperm = lambda t: t.reshape(32, 1024, -1)[inv].reshape(t.shape)
+    assert torch.equal(unperm(out2), out)
+    assert torch.equal(unperm(m2.reshape(4, 8, 1024, 1)).reshape(4, 8, 1024), m)
+    for a, b in zip(g, g2):
+        assert torch.equal(unperm(b), a)
+
+
+def test_config4_linear_in_v2_and_do():
+    """O is linear in V2 and the gradients in dO; power-of-two factors commute with the 16-bit rounding
+    of every intermediate, so the relations are exact."""
+    inputs = orc.make_inputs(4, 8, 1024, 64, torch.bfloat16, seed=42)
+    out, m, g = util.run_dps(inputs, 1 / 8, True, 1024)
+    scaled = list(inputs)
+    scaled[4] = inputs[4] * 4
+    scaled[5] = inputs[5] * 0.5
+    out2, m2, g2 = util.run_dps(scaled, 1 / 8, True, 1024)
+    assert torch.equal(out2, out * 4)
+    assert torch.equal(m2, m)
+    for name, a, b, f in zip(util.NAMES, g, g2, (2, 2, 2, 2, 0.5)):
+        util.assert_close(name, b, a * f, rtol=1e-2, atol=1e-3 * f)

@@ -391,3 +391,51 @@ def test_config3_headline_backward_subset():
         for name, a, ref in zip(util.NAMES, g, grads):
             util.assert_close(f"{name}[{b},{h}]", a[b, h], ref, **LOWP)
             assert util.rel_err(a[b, h], ref) <= 2e-2, (name, util.rel_err(a[b, h], ref))
+
+
+# ------------------------------------------------- full-size properties (no oracle: every head is checked)
+def _headline_inputs(seed=5):
+    return orc.make_inputs(4, 8, 1024, 64, torch.bfloat16, seed=seed)
+
+
+def test_config3_heads_are_independent_and_order_free():
+    """Permuting the (batch, head) slices permutes outputs and gradients bit for bit in the forward and
+    in dQ (owner-computes), and to rounding in the atomically accumulated gradients."""
+    inputs = _headline_inputs()
+    out, g = util.run_tdp(inputs, 1 / 8, True)
+    perm = torch.randperm(32, generator=torch.Generator().manual_seed(1))
+    shuffled = [t.reshape(32, 1024, 64)[perm].reshape(4, 8, 1024, 64).contiguous() for t in inputs]
+    out2, g2 = util.run_tdp(shuffled, 1 / 8, True)
+    unperm = lambda t: t.reshape(32, 1024, 64)[torch.argsort(perm)].reshape(4, 8, 1024, 64)
+    assert torch.equal(unperm(out2), out)
+    assert torch.equal(unperm(g2[0]), g[0])
+    for name, a, b in zip(util.NAMES[1:], g[1:], g2[1:]):
+        util.assert_close(name, unperm(b), a, rtol=2e-2, atol=2e-3)
+
+
+def test_config3_linear_in_v2_and_do():
+    """O is linear in V2; every gradient is linear in dO (same softmax): checked with power-of-two
+    factors, which commute with 16-bit rounding, so the forward relation is exact."""
+    inputs = _headline_inputs(seed=6)
+    out, g = util.run_tdp(inputs, 1 / 8, True)
+    scaled = list(inputs)
+    scaled[4] = inputs[4] * 4                      # V2 -> 4 V2
+    scaled[5] = inputs[5] * 0.5                    # dO -> dO / 2
+    out2, g2 = util.run_tdp(scaled, 1 / 8, True)
+    assert torch.equal(out2, out * 4)
+    # dQ, dK1, dK2, dV1 scale by 4 * 0.5 = 2; dV2 by 0.5
+    for name, a, b, f in zip(util.NAMES, g, g2, (2, 2, 2, 2, 0.5)):
+        util.assert_close(name, b, a * f, rtol=2e-2, atol=2e-3 * f)
+
+
+def test_config3_rows_sum_to_one():
+    """With V2 = 1 and SiLU(V1) = c (a constant column pattern) the output of every query is c: the
+    softmax weights of each of the 4*8*1024 rows sum to one over its (j, k) plane."""
+    inputs = _headline_inputs(seed=7)
+    c = torch.linspace(-2, 2, 64)
+    v1 = torch.empty_like(inputs[3]).copy_(c.expand_as(inputs[3]))
+    inputs[3] = v1
+    inputs[4] = torch.ones_like(inputs[4])
+    out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False)
+    want = torch.nn.functional.silu(v1.float()).to(torch.bfloat16).float()
+    util.assert_close("out", out, want, rtol=2e-2, atol=2e-2)
