@@ -12,6 +12,7 @@
 //   launch 1: rows = (K2, V2), streamed = (K1, U):  dQ (owner-computes), dK2, dV2
 //   launch 2: rows = (K1, U),  streamed = (K2, V2): dK1, dU
 // See the comment above the kernel.
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <type_traits>
@@ -33,6 +34,10 @@ struct BwdParams {
     const float *lse, *delta;  // [BH][T]
     E* dq;                     // written only by the WITH_DQ instantiation
     float *acc_k, *acc_v;      // [BH][T][D] fp32 gradients of row_k / row_v, zero on entry
+    // general kernel only: the rows of a query tile are dealt out to `splits` workgroups; with more than
+    // one, dQ / alpha is accumulated into acc_q (fp32, zero on entry) instead of being written to dq
+    float* acc_q;
+    int splits;
     int T, Tp, BH, nqt;
     float alpha;
     int causal;
@@ -437,7 +442,8 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
                                                        E* __restrict__ k2t, E* __restrict__ v2t,
                                                        float* __restrict__ delta, float* __restrict__ zero_a,
                                                        float* __restrict__ zero_b, float* __restrict__ zero_c,
-                                                       float* __restrict__ zero_d, int T, int Tp, int D) {
+                                                       float* __restrict__ zero_d, float* __restrict__ zero_e, int T,
+                                                       int Tp, int D) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * Tp;
     for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
@@ -464,6 +470,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
             zero_b[off] = 0.f;
             zero_c[off] = 0.f;
             zero_d[off] = 0.f;
+            if (zero_e) zero_e[off] = 0.f;
         }
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -483,7 +490,9 @@ template <typename E>
 __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict__ dk1acc,
                                                          const float* __restrict__ duacc,
                                                          const float* __restrict__ dk2acc,
-                                                         const float* __restrict__ dv2acc, const E* __restrict__ v1,
+                                                         const float* __restrict__ dv2acc,
+                                                         const float* __restrict__ dqacc, float alpha,
+                                                         E* __restrict__ dq, const E* __restrict__ v1,
                                                          E* __restrict__ dk1, E* __restrict__ dv1, E* __restrict__ dk2,
                                                          E* __restrict__ dv2, size_t n) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
@@ -491,11 +500,12 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
         dv1[i] = (E)(duacc[i] * silu_grad_f((float)v1[i]));
         dk2[i] = (E)dk2acc[i];
         dv2[i] = (E)dv2acc[i];
+        if (dqacc) dq[i] = (E)(dqacc[i] * alpha);
     }
 }
 
 struct BwdLayout {
-    size_t u, ut, k1t, k2t, v2t, delta, dk1acc, duacc, dk2acc, dv2acc, total;
+    size_t u, ut, k1t, k2t, v2t, delta, dk1acc, duacc, dk2acc, dv2acc, dqacc, total;
 };
 static BwdLayout bwd_layout(int BH, int T, int D) {
     const size_t Tp = (size_t)(T + 63) / 64 * 64, n = (size_t)BH * T * D;
@@ -517,6 +527,7 @@ static BwdLayout bwd_layout(int BH, int T, int D) {
     l.duacc = take(n * 4);
     l.dk2acc = take(n * 4);
     l.dv2acc = take(n * 4);
+    l.dqacc = take(n * 4);  // used when the rows of a query tile are split over workgroups (small grids)
     l.total = (off + 255) & ~size_t(255);
     return l;
 }
@@ -531,10 +542,19 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     float *dk1acc = (float*)(ws + l.dk1acc), *duacc = (float*)(ws + l.duacc);
     float *dk2acc = (float*)(ws + l.dk2acc), *dv2acc = (float*)(ws + l.dv2acc);
 
+    // A workgroup owns a 32-query tile and walks all of its rows.  When that leaves most of the chip idle
+    // (few heads, short sequences) the rows of a tile are dealt out to several workgroups of the general
+    // kernel, and dQ is accumulated in fp32 like the row gradients.
+    const int tiles = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32);
+    int splits = 1;
+    if (tiles < 512) splits = std::min(8, std::max(1, 768 / tiles));
+    if (const char* v = getenv("TRITT_BWD_SPLITS")) splits = std::max(1, std::min(16, atoi(v)));  // tuning sweeps
+    float* dqacc = splits > 1 ? (float*)(ws + l.dqacc) : nullptr;
+
     hipLaunchKernelGGL(bwd_prep_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (const E*)a.k1,
                        (const E*)a.k2, (const E*)a.v2, (const E*)a.o, (const E*)a.d_o, (E*)(ws + l.u),
                        (E*)(ws + l.ut), (E*)(ws + l.k1t), (E*)(ws + l.k2t), (E*)(ws + l.v2t),
-                       (float*)(ws + l.delta), dk1acc, duacc, dk2acc, dv2acc, a.T, Tp, D);
+                       (float*)(ws + l.delta), dk1acc, duacc, dk2acc, dv2acc, dqacc, a.T, Tp, D);
 
     BwdParams<E> p;
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o;
@@ -542,6 +562,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.dq = (E*)a.dq;
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
+    p.acc_q = dqacc; p.splits = splits;
 
     // D = 64, full windows: three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO
     // tiles (twice: operand and epilogue layout), four dQ slices.  Otherwise: tdp_bwd_rows_general.hpp
@@ -554,7 +575,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         smem = bwdg_smem(32, 8, 32, true);
         kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true>;
         kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true>;
-    } else if (a.windowed) {
+    } else if (a.windowed || (D == 64 && splits > 1)) {
+        // (full windows are windows of T: the banded kernel is also the one that can split a tile's rows)
         smem = bwdg_smem(D, 8, 64, true);
         kern_dq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), true, 8, 64, true>;
         kern_nodq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), false, 8, 64, true>;
@@ -594,7 +616,9 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         if (e != hipSuccess) return e;
     }
     const int groups = (a.BH + 7) / 8;
-    const dim3 grid(8 * groups * p.nqt * col_parts);
+    const bool general = D != 64 || a.windowed || splits > 1;
+    if (!general) p.splits = 1;
+    const dim3 grid(8 * groups * p.nqt * col_parts * (general ? p.splits : 1));
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
@@ -612,8 +636,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     size_t gridf = (n + 255) / 256;
     if (gridf > 4096) gridf = 4096;
     hipLaunchKernelGGL(bwd_finish_kernel<E>, dim3((unsigned)gridf), dim3(256), 0, st, (const float*)dk1acc,
-                       (const float*)duacc, (const float*)dk2acc, (const float*)dv2acc, (const E*)a.v1, (E*)a.dk1,
-                       (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n);
+                       (const float*)duacc, (const float*)dk2acc, (const float*)dv2acc, (const float*)dqacc, a.alpha,
+                       (E*)a.dq, (const E*)a.v1, (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n);
     return hipGetLastError();
 }
 

@@ -105,6 +105,8 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
         c0 = (slot & 1) * DH;
         slot >>= 1;
     }
+    const int split = slot % p.splits;  // which share of the tile's rows (rounds) this workgroup walks
+    slot /= p.splits;
     const int bh = (slot % groups) * 8 + xcd;
     const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
     if (bh >= p.BH) return;
@@ -128,6 +130,10 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     const int m_first = banded ? max(0, max(q0 - p.wb, q0 - p.wa - p.rab)) / NW : 0;
     auto step_lo = [&](int m) { return banded ? max(0, max(q0 - p.wa, m * NW - p.lab)) / 32 : 0; };
     auto step_hi = [&](int m) { return banded ? min(jend, m * NW + NW - 1 + p.rab) / 32 : nsteps - 1; };
+    // this workgroup's rounds
+    const int per_split = (nrounds - m_first + p.splits - 1) / p.splits;
+    const int m_lo = m_first + split * per_split, m_hi = min(nrounds, m_lo + per_split);
+    if (m_lo >= m_hi) return;  // fewer rounds than shares (uniform over the workgroup, before any barrier)
     const int q = q0 + n;
     const bool q_ok = q < T;
     const int jq = p.causal ? min(q, T - 1) : T - 1;
@@ -208,16 +214,16 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     }
     // (round, step) of the stage fetched next: the sequence the main loop walks, wrapping to the first
     // round after the last (those fetches are never used)
-    int m_ahead = m_first, st_ahead = step_lo(m_first);
+    int m_ahead = m_lo, st_ahead = step_lo(m_lo);
     auto advance = [&]() {
         if (st_ahead < step_hi(m_ahead)) {
             ++st_ahead;
         } else {
-            m_ahead = m_ahead + 1 < nrounds ? m_ahead + 1 : m_first;
+            m_ahead = m_ahead + 1 < m_hi ? m_ahead + 1 : m_lo;
             st_ahead = step_lo(m_ahead);
         }
     };
-    issue_round(m_first, m_first & 1);
+    issue_round(m_lo, m_lo & 1);
     issue_stage(st_ahead, 0);
     advance();
     issue_stage(st_ahead, 1);
@@ -231,7 +237,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     const int krow_off = key_of_row(n);
     const int fperm = D == 32 ? swz_t(krow_off) : swz_perm(krow_off);
 
-    for (int m = m_first; m < nrounds; ++m) {
+    for (int m = m_lo; m < m_hi; ++m) {
         const int mb = m & 1;
         const int k = m * NW + wave;
         const int st_first = step_lo(m), st_last = step_hi(m);
@@ -260,7 +266,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             // rows) has landed; after the barrier that holds for every wave's part, and every wave is
             // done with the buffer the next fetch overwrites
             barrier_keep_loads<LW>();
-            if (st == st_first && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
+            if (st == st_first && m + 1 < m_hi) issue_round(m + 1, mb ^ 1);  // older than the stage loads
             issue_stage(st_ahead, (gstage + 2) % NBUF);
             advance();
             if (!built) {
@@ -462,7 +468,11 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             const float out[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                if (q0 + r0 + e < T) p.dq[base + (size_t)(q0 + r0 + e) * D + d] = (E)(out[e] * p.alpha);
+                if (q0 + r0 + e < T) {
+                    const size_t off = base + (size_t)(q0 + r0 + e) * D + d;
+                    if (p.splits > 1) unsafeAtomicAdd(p.acc_q + off, out[e]);  // scaled by alpha when converted
+                    else p.dq[off] = (E)(out[e] * p.alpha);
+                }
         }
     }
 }

@@ -315,6 +315,23 @@ def test_mfma_windows_fp16_batched(D):
         assert util.rel_err(a, b) <= 5e-2, (name, util.rel_err(a, b))
 
 
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("splits", [2, 5, 16])
+def test_mfma_backward_row_splits(splits, D, monkeypatch):
+    """The rows of a query tile dealt out to several workgroups (what small grids get): dQ then goes
+    through an fp32 accumulator like the row gradients.  Windowed and full masks, ragged length."""
+    monkeypatch.setenv("TRITT_BWD_SPLITS", str(splits))
+    alpha = 1 / math.sqrt(D)
+    for windows in ((None,) * 4, (40, 100, 20, 7)):
+        inputs = orc.make_inputs(1, 3, 203, D, torch.bfloat16, seed=splits + D)
+        z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
+        out, g = util.run_tdp(inputs, alpha, True, windows, flags=FORCE_MFMA)
+        util.assert_close("out", out, z, **LOWP)
+        for name, a, b in zip(util.NAMES, g, grads):
+            util.assert_mostly_close(name, a, b, **LOWP)
+            assert util.rel_err(a, b) <= 5e-2, (name, windows, util.rel_err(a, b))
+
+
 def test_unaligned_views_are_copied():
     """Contiguous views that start in the middle of a storage (2-byte aligned) are accepted: the host side
     copies them to aligned memory before the library sees them."""
