@@ -547,7 +547,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     // kernel, and dQ is accumulated in fp32 like the row gradients.
     const int tiles = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32);
     int splits = 1;
-    if (tiles < 512) splits = std::min(8, std::max(1, 768 / tiles));
+    if (tiles < 1024) splits = std::min(16, (1024 + tiles - 1) / tiles);  // 512 tiles: the tuned kernel's tail costs more than the general kernel does
     if (const char* v = getenv("TRITT_BWD_SPLITS")) splits = std::max(1, std::min(16, atoi(v)));  // tuning sweeps
     float* dqacc = splits > 1 ? (float*)(ws + l.dqacc) : nullptr;
 
