@@ -104,7 +104,10 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     E* sOe = sQe + DT * 64 * 16;
 
     const int groups = (p.BH + 7) / 8;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int xcd = blockIdx.x & 7;
+    int slot = blockIdx.x >> 3;
+    const int split = slot % p.splits;  // which share of the tile's rounds this workgroup walks (small grids)
+    slot /= p.splits;
     const int bh = (slot % groups) * 8 + xcd;
     const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
     if (bh >= p.BH) return;
@@ -125,6 +128,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     const int jend = p.causal ? qlast : T - 1;  // last j (and last k) any query of the tile needs
     const int jfull = p.causal ? q0 : T - 1;    // keys / rows 0 .. jfull are valid for every column
     const int nst = jend / 64 + 1, nrounds = jend / 8 + 1;
+    const int per_split = (nrounds + p.splits - 1) / p.splits;
+    const int m_lo = split * per_split, m_hi = min(nrounds, m_lo + per_split);
+    if (m_lo >= m_hi) return;  // fewer rounds than shares (uniform over the workgroup, before any barrier)
     const int q = q0 + n;                        // this lane's column
     const bool q_ok = q < T;
     const int jq = p.causal ? min(q, T - 1) : T - 1;  // per-lane bound on j and k
@@ -191,7 +197,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         float* all = reinterpret_cast<float*>(sOb + BQ * LDK);
         for (int idx = tid; idx < (NW / 2) * BQ * D; idx += NTH) all[idx] = 0.f;
     }
-    issue_round(0, 0);
+    issue_round(m_lo, m_lo & 1);
     issue_stage(0, 0);
     issue_stage(1 % nst, 1);
     barrier_keep_loads<0>();  // stages 0 and 1 and the first round have landed for every wave
@@ -233,7 +239,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     const bool late = (wave >> 2) & 1;  // second wave of its SIMD (waves w and w + 4 share one)
     int gstage = 0;          // running stage index; buffer = gstage % NBUF
     int st_ahead = 2 % nst;  // stage number of running index gstage + 2
-    for (int m = 0; m < nrounds; ++m) {
+    for (int m = m_lo; m < m_hi; ++m) {
         const int mb = m & 1;
         const int k = m * 8 + wave;  // this wave's K2/V2 row
 
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 if (half == 1) {
                     // the buffer two stages ahead was last read in the previous stage, and every wave is
                     // past that (this stage's barrier was crossed in the first half): fetch it now
-                    if (st == 0 && m + 1 < nrounds) issue_round(m + 1, mb ^ 1);  // older than the stage loads
+                    if (st == 0 && m + 1 < m_hi) issue_round(m + 1, mb ^ 1);  // older than the stage loads
                     issue_stage(st_ahead, (gstage + 2) % NBUF);
                     st_ahead = st_ahead + 1 < nst ? st_ahead + 1 : 0;
                 }
@@ -426,7 +432,11 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         const float out[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            if (q0 + r0 + e < T) p.dq[base + (size_t)(q0 + r0 + e) * D + d] = (E)(out[e] * p.alpha);
+            if (q0 + r0 + e < T) {
+                const size_t off = base + (size_t)(q0 + r0 + e) * D + d;
+                if (p.splits > 1) unsafeAtomicAdd(p.acc_q + off, out[e]);  // scaled by alpha when converted
+                else p.dq[off] = (E)(out[e] * p.alpha);
+            }
     }
 }
 
@@ -542,12 +552,12 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     float *dk1acc = (float*)(ws + l.dk1acc), *duacc = (float*)(ws + l.duacc);
     float *dk2acc = (float*)(ws + l.dk2acc), *dv2acc = (float*)(ws + l.dv2acc);
 
-    // A workgroup owns a 32-query tile and walks all of its rows.  When that leaves most of the chip idle
-    // (few heads, short sequences) the rows of a tile are dealt out to several workgroups of the general
-    // kernel, and dQ is accumulated in fp32 like the row gradients.
+    // A workgroup owns a 32-query tile and walks all of its rows.  When that leaves most of the chip idle, or
+    // ends in a long tail (few heads, short sequences), the rows of a tile are dealt out to several
+    // workgroups, and dQ is accumulated in fp32 like the row gradients.
     const int tiles = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32);
     int splits = 1;
-    if (tiles < 1024) splits = std::min(16, (1024 + tiles - 1) / tiles);  // 512 tiles: the tuned kernel's tail costs more than the general kernel does
+    if (tiles < 1024) splits = std::min(16, (1024 + tiles - 1) / tiles);
     if (const char* v = getenv("TRITT_BWD_SPLITS")) splits = std::max(1, std::min(16, atoi(v)));  // tuning sweeps
     float* dqacc = splits > 1 ? (float*)(ws + l.dqacc) : nullptr;
 
@@ -575,8 +585,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         smem = bwdg_smem(32, 8, 32, true);
         kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true>;
         kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true>;
-    } else if (a.windowed || (D == 64 && splits > 1)) {
-        // (full windows are windows of T: the banded kernel is also the one that can split a tile's rows)
+    } else if (a.windowed) {
         smem = bwdg_smem(D, 8, 64, true);
         kern_dq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), true, 8, 64, true>;
         kern_nodq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), false, 8, 64, true>;
@@ -616,9 +625,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         if (e != hipSuccess) return e;
     }
     const int groups = (a.BH + 7) / 8;
-    const bool general = D != 64 || a.windowed || splits > 1;
-    if (!general) p.splits = 1;
-    const dim3 grid(8 * groups * p.nqt * col_parts * (general ? p.splits : 1));
+    const dim3 grid(8 * groups * p.nqt * col_parts * p.splits);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
