@@ -49,6 +49,15 @@ def windowed_triples(T, w1, w2, kl, kr):
     return total
 
 
+def make_inputs(B, H, T, D, dtype, seed=0, n=6):
+    """Seeded synthetic inputs: N(0,1) draws from a CPU generator in the order Q, K1, K2, V1, V2, dO, drawn in
+    fp32 and then cast (the same draws the parity tests use)."""
+    import torch
+
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return [torch.randn(B, H, T, D, generator=g, dtype=torch.float32).to(dtype) for _ in range(n)]
+
+
 def time_events(fn, iters, warmup, torch):
     """Average milliseconds per call, HIP events on the stream the kernels run on
     (torch's current stream, which is the stream handed to the library)."""
@@ -106,13 +115,15 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "dps", "tdp"], default="both",
+    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "dps", "tdp", "published"], default="both",
                     help="fwd: time only the forward (for profiling runs); copy: a plain 256 MiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against; "
                          "sweep: triple-dot forward at B=1 H=16 D=128 bf16 over T in 512..4096; "
                          "dps: dot-product-sum forward+backward at --B --H --T --D; "
                          "tdp: triple-dot forward+backward at --B --H --T --D with --windows (secondary shapes: "
-                         "D=128, windowed masks)")
+                         "D=128, windowed masks); "
+                         "published: the forward cases the reference publishes timings for (B=2 H=8 D=64 fp16 causal: "
+                         "T=256/512/1024 full windows, T=2048 windows 128,128,32,32), its best H100 / B200 figures beside ours")
     ap.add_argument("--windows", default="", help="k1_window,k2_window,kk_left,kk_right for --mode tdp (empty: full)")
     ap.add_argument("--dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="tensor type for --mode tdp")
     ap.add_argument("--B", type=int, default=4)
@@ -128,8 +139,6 @@ def main():
 
     from flash_trittention import _lib
     from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
-    from oracle import trittention_oracle as orc
-
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     _lib.lib()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
@@ -146,7 +155,7 @@ def main():
     if args.mode == "sweep":
         rows = []
         for Ts in (512, 1024, 2048, 4096):
-            ins = [t.to(dev) for t in orc.make_inputs(1, 16, Ts, 128, torch.bfloat16, seed=0, n=5)]
+            ins = [t.to(dev) for t in make_inputs(1, 16, Ts, 128, torch.bfloat16, seed=0, n=5)]
             torch.cuda.reset_peak_memory_stats()
             base_mem = torch.cuda.memory_allocated()
 
@@ -163,10 +172,33 @@ def main():
         print(json.dumps({"metric": "triple-dot trittention fwd TFLOP/s vs T", "unit": "TFLOP/s",
                           "config": {"workload": "triple-dot fwd B=1 H=16 D=128 bf16 causal"}, "rows": rows}), flush=True)
         return
+    if args.mode == "published":
+        # the reference's own forward table (h100/README.md:50-53, b200/README.md:53-56): milliseconds of its
+        # best kernel on each machine; B=2 H=8 D=64 fp16 causal, softmax_scale 1/8
+        cases = [(256, None, 0.298, 0.461), (512, None, 1.451, 2.111), (1024, None, 8.748, 11.61),
+                 (2048, (128, 128, 32, 32), 1.163, 1.074)]
+        rows = []
+        for Ts, win, h100_ms, b200_ms in cases:
+            ins = [t.to(dev) for t in make_inputs(2, 8, Ts, 64, torch.float16, seed=1, n=5)]
+            w = win or (None, None, None, None)
+
+            def f():
+                with torch.no_grad():
+                    return flash_trittention(*ins, softmax_scale=1 / 8, k1_window=w[0], k2_window=w[1], kk_left=w[2],
+                                             kk_right=w[3], causal=True)
+
+            ms = time_events(f, max(args.steps, 20), max(args.warmup, 5), torch)
+            nt = 16 * (windowed_triples(Ts, *win) if win else triples(1, 1, Ts))
+            rows.append({"T": Ts, "windows": win, "ms": ms, "tflops": 4 * 64 * nt / ms / 1e9,
+                         "reference_h100_ms": h100_ms, "reference_b200_ms": b200_ms,
+                         "speedup_vs_best_published": min(h100_ms, b200_ms) / ms})
+        print(json.dumps({"metric": "triple-dot trittention fwd ms on the reference's published cases", "unit": "ms",
+                          "config": {"workload": "triple-dot fwd B=2 H=8 D=64 fp16 causal"}, "rows": rows}), flush=True)
+        return
     if args.mode == "dps":
         from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
 
-        ins = [t.to(dev) for t in orc.make_inputs(B, H, T, D, torch.bfloat16, seed=0)]
+        ins = [t.to(dev) for t in make_inputs(B, H, T, D, torch.bfloat16, seed=0)]
         lv = [t.clone().requires_grad_(True) for t in ins[:5]]
         mod = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=T)
         hold = {}
@@ -188,7 +220,7 @@ def main():
                           "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} bf16 causal"}}), flush=True)
         return
     tdtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype if args.mode == "tdp" else "bf16"]
-    q, k1, k2, v1, v2, do = (t.to(dev) for t in orc.make_inputs(B, H, T, D, tdtype, seed=0))
+    q, k1, k2, v1, v2, do = (t.to(dev) for t in make_inputs(B, H, T, D, tdtype, seed=0))
     leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
     kw = dict(softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True)
 

@@ -177,20 +177,25 @@ def dps_forward_backward(q, k1, k2, v1, v2, d_out, alpha, causal=True, k_diff=No
 
 
 def tdp_forward_backward_chunked(q, k1, k2, v1, v2, d_out, alpha, causal=True,
-                                 q_chunk: int = 64, need_grads: bool = True):
+                                 q_chunk: int = 64, need_grads: bool = True, rows=None):
     """Same as ``tdp_forward_backward`` for ONE head ([T, D] inputs), full
     windows only, evaluated in chunks of query rows so the [q, j, k] slab
     stays small (T=1024: 64 x 1024 x 1024 fp32 = 268 MB).  For a causal chunk
-    only j,k <= last query of the chunk are touched.
+    only j,k <= last query of the chunk are touched.  ``rows=(lo, hi)``
+    (forward only) evaluates just the query rows lo..hi-1 and returns
+    [hi - lo, ...] tensors: spot checks at sequence lengths whose full plane
+    is out of reach.
     """
     assert q.dim() == 2
     T, D = q.shape
+    r_lo, r_hi = rows if rows is not None else (0, T)
+    assert rows is None or not need_grads
     leaves = [t.detach().clone().requires_grad_(need_grads) for t in (q, k1, k2, v1, v2)]
     ql, k1l, k2l, v1l, v2l = leaves
-    z_out = torch.empty_like(q)
-    lse_out = torch.empty(T, dtype=q.dtype)
-    for lo in range(0, T, q_chunk):
-        hi = min(T, lo + q_chunk)
+    z_out = torch.empty_like(q[r_lo:r_hi])
+    lse_out = torch.empty(r_hi - r_lo, dtype=q.dtype)
+    for lo in range(r_lo, r_hi, q_chunk):
+        hi = min(r_hi, lo + q_chunk)
         n = hi if causal else T          # keys beyond the chunk's last query are masked
         with torch.set_grad_enabled(need_grads):
             u = F.silu(v1l[:n])
@@ -206,8 +211,8 @@ def tdp_forward_backward_chunked(q, k1, k2, v1, v2, d_out, alpha, causal=True,
             z = (t1 * v2l[None, :n, :]).sum(1)
             if need_grads:
                 z.backward(d_out[lo:hi])
-        z_out[lo:hi] = z.detach()
-        lse_out[lo:hi] = lse.detach()
+        z_out[lo - r_lo:hi - r_lo] = z.detach()
+        lse_out[lo - r_lo:hi - r_lo] = lse.detach()
     grads = [t.grad for t in leaves] if need_grads else None
     return z_out, lse_out, grads
 

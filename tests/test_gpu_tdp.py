@@ -250,6 +250,38 @@ def test_config3_headline_forward_subset():
         util.assert_close(f"out[{b},{h}]", out[b, h], z, **LOWP)
 
 
+@pytest.mark.parametrize("seq_len,row_blocks", [(512, [(0, 512)]), (1024, [(0, 64), (480, 544), (960, 1024)]),
+                                                (2048, [(0, 32), (1000, 1032), (2016, 2048)]),
+                                                (4096, [(2040, 2056), (4080, 4096)])])
+def test_config5_long_sequence_forward(seq_len, row_blocks):
+    """B=1 H=16 D=128 bf16 causal, alpha = 1/sqrt(D), T = 512 .. 4096: blocks of query rows of two heads
+    against the chunked dense oracle, and device memory beyond the inputs stays O(B H T D): the output,
+    the log-sum-exp and one transposed copy of SiLU(V1), never a score plane."""
+    print(f"case config5 forward T={seq_len}", flush=True)
+    alpha = 1 / math.sqrt(128)
+    inputs = orc.make_inputs(1, 16, seq_len, 128, torch.bfloat16, seed=5, n=5)
+    dev = [t.cuda() for t in inputs]
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    with torch.no_grad():
+        out = flash_trittention(*dev, softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None,
+                                kk_right=None, causal=True)
+    torch.cuda.synchronize()
+    extra = torch.cuda.max_memory_allocated() - before
+    one_tensor = 16 * seq_len * 128 * 2
+    assert extra <= 2.5 * one_tensor + (1 << 20), (extra, one_tensor)
+    out = out.cpu()
+    for h in (3, 15):
+        for lo, hi in row_blocks:
+            z, _, _ = orc.tdp_forward_backward_chunked(*(t[0, h].float() for t in inputs), None, alpha, True,
+                                                       q_chunk=16 if seq_len > 2048 else 64, need_grads=False,
+                                                       rows=(lo, hi))
+            util.assert_close(f"out[{h}, {lo}:{hi}]", out[0, h, lo:hi].float(), z, **LOWP)
+
+
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("seq_len", [1, 33, 100, 256, 300])
 def test_mfma_backward_bf16(seq_len, causal):

@@ -181,6 +181,17 @@ def test_chunked_equals_dense(causal):
         assert torch.allclose(a, b, atol=1e-11)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_chunked_row_range_equals_dense_rows(causal):
+    T, D, alpha = 40, 8, 0.35
+    q, k1, k2, v1, v2 = (rnd(T, D, seed=85 + s) for s in range(5))
+    z, lse = orc.tdp_forward_dense(q, k1, k2, v1, v2, alpha=alpha, causal=causal)
+    zr, lser, g = orc.tdp_forward_backward_chunked(q, k1, k2, v1, v2, None, alpha, causal, q_chunk=7,
+                                                   need_grads=False, rows=(11, 30))
+    assert g is None and zr.shape == (19, D)
+    assert torch.allclose(z[11:30], zr, atol=1e-12) and torch.allclose(lse[11:30], lser, atol=1e-12)
+
+
 def test_batched_heads_are_independent():
     B, H, T, D = 2, 3, 9, 4
     ins = [rnd(B, H, T, D, seed=90 + s) for s in range(5)]
