@@ -305,11 +305,23 @@ const char* tritt_status_string(int status) {
     return "unknown status";
 }
 
+// the fields of MfmaFwdArgs that describe the problem (no pointers)
+static MfmaFwdArgs mfma_fwd_shape(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,
+                                  int kk_left, int kk_right) {
+    const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
+    MfmaFwdArgs a{};
+    a.BH = B * H; a.T = T; a.D = D; a.causal = causal ? 1 : 0;
+    a.is_bf16 = dtype == TRITT_BF16;
+    a.windowed = full_windows(T, causal, w1, w2, kl, kr) ? 0 : 1;
+    a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+    return a;
+}
+
 size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,
                                      int kk_left, int kk_right, unsigned flags) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
     if (use_mfma_fwd(T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags))
-        return mfma_tdp_fwd_workspace(B * H, T, D);
+        return mfma_tdp_fwd_workspace(mfma_fwd_shape(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right));
     Arena ar(nullptr);
     tdp_fwd_generic(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f,
                     causal, k1_window, k2_window, kk_left, kk_right, nullptr);
@@ -331,12 +343,9 @@ int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1,
     const size_t need = tritt_tdp_fwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
     if (need && (!workspace || workspace_bytes < need)) return TRITT_ERR_WORKSPACE;
     if (mfma) {
-        MfmaFwdArgs a{};
+        MfmaFwdArgs a = mfma_fwd_shape(B, H, T, D, dtype, causal, w1, w2, kl, kr);
         a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.lse = lse; a.ut = workspace;
-        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0;
-        a.is_bf16 = dtype == TRITT_BF16;
-        a.windowed = full_windows(T, causal, w1, w2, kl, kr) ? 0 : 1;
-        a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+        a.alpha = alpha;
         return (int)mfma_tdp_fwd(a, (hipStream_t)stream);
     }
     Arena ar(workspace);

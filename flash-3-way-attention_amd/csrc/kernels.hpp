@@ -51,7 +51,8 @@ struct MfmaFwdArgs {
     int windowed;  // some window can exclude a pair with j, k <= q: the banded instantiation
     int k1_window, k2_window, kk_left, kk_right;
 };
-size_t mfma_tdp_fwd_workspace(int BH, int T, int D);
+// needs BH, T, D, causal, windowed and the four windows of `a`
+size_t mfma_tdp_fwd_workspace(const MfmaFwdArgs& a);
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st);
 

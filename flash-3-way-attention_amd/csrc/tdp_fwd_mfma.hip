@@ -42,6 +42,11 @@ struct FwdParams {
     // windowed instantiation only: (q, j, k) takes part iff j <= q, k <= q, q - j <= wa, q - k <= wb,
     // k - j <= lab, j - k <= rab
     int wa, wb, lab, rab;
+    // splits > 1 (small grids): the k-tiles of a query tile are dealt out to `splits` workgroups; each writes
+    // its unnormalised output, reference maximum and row sum to part[((bh T + q) splits + s) (D + 2)]
+    // (O[D], M, L; M in log2 units, -inf: nothing in this part) and fwd_merge_kernel joins them
+    int splits;
+    float* part;
 };
 
 constexpr float kLazyThreshold = 8.0f;
@@ -80,7 +85,10 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     // every XCD its own set of heads (their K/V stay in that XCD's L2) and hand out the
     // longest query tiles first.
     const int groups = (p.BH + 7) / 8;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int xcd = blockIdx.x & 7;
+    int slot = blockIdx.x >> 3;
+    const int split = slot % p.splits;
+    slot /= p.splits;
     const int bh = (slot % groups) * 8 + xcd;
     const int qt = p.nqt - 1 - slot / groups;
     if (bh >= p.BH) return;
@@ -98,11 +106,23 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 
     const int q0 = qt * BQ;
     const int jend = p.causal ? min(T - 1, q0 + BQ - 1) : T - 1;  // last key any query here needs
-    const int nst = jend / JS + 1, nkt = jend / 32 + 1;
+    const int nst = jend / JS + 1;
+    int nkt = jend / 32 + 1;
     // WIN: the first k-tile any query here can use (k >= q - wb, and some j with q - wa <= j <= k + rab),
     // and per k-tile the stages that hold keys j any (q, k) of it can use
     const bool banded = WIN && p.causal;
-    const int kt_lo = banded ? max(0, max(q0 - p.wb, q0 - p.wa - p.rab)) / 32 : 0;
+    int kt_lo = banded ? max(0, max(q0 - p.wb, q0 - p.wa - p.rab)) / 32 : 0;
+    if (p.splits > 1) {  // this workgroup's share of the k-tiles
+        const int per = (nkt - kt_lo + p.splits - 1) / p.splits;
+        kt_lo += split * per;
+        nkt = min(nkt, kt_lo + per);
+        if (kt_lo >= nkt) {  // nothing left for this part: say so and leave
+            const int q = q0 + (int)(threadIdx.x >> 6) * NT + (int)(threadIdx.x & 63);
+            if ((threadIdx.x & 63) < NT && q < p.T)
+                p.part[(((size_t)bh * p.T + q) * p.splits + split) * (D + 2) + D] = -INFINITY;
+            return;
+        }
+    }
     auto first_stage = [&](int kt) { return banded ? max(0, max(q0 - p.wa, kt * 32 - p.lab)) / JS : 0; };
     auto last_stage = [&](int kt) { return banded ? min(jend, kt * 32 + 31 + p.rab) / JS : nst - 1; };
 
@@ -680,6 +700,19 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int q = qrow[t];
+        if (p.splits > 1) {
+            float* dst = p.part + (((size_t)bh * T + q) * p.splits + split) * (D + 2);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const float o = Orun[t][dt] + __shfl_xor(Orun[t][dt], 32, 64);
+                if (q < T && g == 0) dst[dt * 32 + n] = o;
+            }
+            if (q < T && lane == 0) {
+                dst[D] = Mrun[t];
+                dst[D + 1] = Lrun[t];
+            }
+            continue;
+        }
         const float inv = 1.0f / Lrun[t];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -688,6 +721,28 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
         }
         if (q < T && lane == 0) p.lse[(size_t)bh * T + q] = (Mrun[t] + fast_log2(Lrun[t])) * kLn2;
     }
+}
+
+// Joins the parts a split forward left behind: one thread per (row, d).
+template <typename E>
+__global__ __launch_bounds__(256) void fwd_merge_kernel(const float* __restrict__ part, E* __restrict__ o,
+                                                        float* __restrict__ lse, int rows, int D, int splits) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    const int row = idx / D, d = idx % D;
+    if (row >= rows) return;
+    const float* src = part + (size_t)row * splits * (D + 2);
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, src[s * (D + 2) + D]);
+    float l = 0.f, acc = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float ms = src[s * (D + 2) + D];
+        if (ms == -INFINITY) continue;  // an empty part: its other fields were never written
+        const float w = fast_exp2(ms - m);
+        l += w * src[s * (D + 2) + D + 1];
+        acc += w * src[s * (D + 2) + d];
+    }
+    o[(size_t)row * D + d] = (E)(acc / l);
+    if (d == 0) lse[row] = (m + fast_log2(l)) * kLn2;
 }
 
 // U^T[bh][d][j] = SiLU(V1[bh][j][d]) for j < T, 0 for T <= j < Tp
@@ -713,12 +768,41 @@ constexpr size_t fwd_smem_bytes() {
 
 constexpr int kTpad = 128;  // U^T rows are padded to a multiple of the largest stage
 
+// Small grids split the k-tiles of every query tile over several workgroups: a causal grid ends in its heaviest
+// query tiles, three times the average, and one workgroup fills a CU.  Measured optimum: enough parts for about
+// 768 workgroups, no more than 4 (every part pays the prologue and a tail), and parts of at least 2 k-tiles
+// (4 under a windowed mask, whose k-tiles see only a few steps of j each).
+constexpr int kFwdSplitTarget = 768, kAutoFwdSplits = 4, kMaxFwdSplits = 8;
+
+static int fwd_variant();
+
+// queries per workgroup of the instantiation mfma_tdp_fwd() picks
+static int fwd_tile_queries(int D, int windowed) { return (D == 64 && !windowed && fwd_variant() != 2) ? 16 : 8; }
+
+static size_t ut_bytes(int BH, int T, int D) {
+    const size_t Tp = (size_t)(T + kTpad - 1) / kTpad * kTpad;
+    return ((size_t)BH * D * Tp * 2 + 255) / 256 * 256;
+}
+
+// TRITT_FWD_SPLITS overrides the count (tests, tuning sweeps); read per call, so the workspace query and
+// the launch that follows it must see the same value
+static int fwd_splits(const MfmaFwdArgs& a, int bq) {
+    if (const char* e = getenv("TRITT_FWD_SPLITS")) return max(1, min(atoi(e), kMaxFwdSplits));
+    const int wgs = a.BH * ((a.T + bq - 1) / bq);
+    const bool banded = a.windowed && a.causal;
+    // keys k the heaviest query tile walks
+    const int span = banded ? min(a.T, max(a.k2_window, a.k1_window + a.kk_right) + bq) : a.T;
+    const int by_size = (kFwdSplitTarget + wgs - 1) / wgs, by_tiles = (span + 31) / 32 / (banded ? 4 : 2);
+    return max(1, min(kAutoFwdSplits, min(by_size, by_tiles)));
+}
+
 template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false>
 static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
                        a.T, Tp, D);
     constexpr int BQ = WAVES * NT;
+    if (BQ != fwd_tile_queries(D, a.windowed)) return hipErrorInvalidValue;  // the workspace was sized for another shape
     FwdParams<E> p;
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
     p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse;
@@ -726,6 +810,8 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     p.scale_log2 = a.alpha * kLog2e;
     p.causal = a.causal;
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
+    p.splits = fwd_splits(a, BQ);
+    p.part = reinterpret_cast<float*>(static_cast<char*>(a.ut) + ut_bytes(a.BH, a.T, D));
     constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS>();
     auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN>;
     {
@@ -735,13 +821,19 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
         if (e != hipSuccess) return e;
     }
     const int groups = (a.BH + 7) / 8;
-    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(64 * WAVES), smem, st, p);
+    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt * p.splits), dim3(64 * WAVES), smem, st, p);
+    if (p.splits > 1) {
+        const int rows = a.BH * a.T;
+        hipLaunchKernelGGL(fwd_merge_kernel<E>, dim3((rows * D + 255) / 256), dim3(256), 0, st, p.part, (E*)a.o, a.lse,
+                           rows, D, p.splits);
+    }
     return hipGetLastError();
 }
 
-size_t mfma_tdp_fwd_workspace(int BH, int T, int D) {
-    const size_t Tp = (size_t)(T + kTpad - 1) / kTpad * kTpad;
-    return (size_t)BH * D * Tp * 2;
+// U^T, then the parts of a split forward
+size_t mfma_tdp_fwd_workspace(const MfmaFwdArgs& a) {
+    const int splits = fwd_splits(a, fwd_tile_queries(a.D, a.windowed));
+    return ut_bytes(a.BH, a.T, a.D) + (splits > 1 ? (size_t)a.BH * a.T * splits * (a.D + 2) * sizeof(float) : 0);
 }
 
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }

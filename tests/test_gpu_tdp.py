@@ -364,6 +364,60 @@ def test_mfma_backward_row_splits(splits, D, monkeypatch):
             assert util.rel_err(a, b) <= 5e-2, (name, windows, util.rel_err(a, b))
 
 
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("splits", [2, 3, 8])
+def test_mfma_forward_k_splits(splits, D, monkeypatch):
+    """The k-tiles of a query tile dealt out to several workgroups and joined by the merge kernel (what
+    small grids get): full, non-causal and windowed masks at a ragged length.  Parts with no k-tile at all
+    (early query tiles) must drop out of the merge.  The backward reads the merged log-sum-exp."""
+    monkeypatch.setenv("TRITT_FWD_SPLITS", str(splits))
+    alpha = 1 / math.sqrt(D)
+    inputs = orc.make_inputs(1, 3, 203, D, torch.bfloat16, seed=splits + D)
+    for causal, windows in ((True, (None,) * 4), (False, (None,) * 4), (True, (40, 100, 20, 7))):
+        z, _, grads = util.oracle_tdp(inputs, alpha, causal, windows)
+        out, g = util.run_tdp(inputs, alpha, causal, windows, flags=FORCE_MFMA)
+        util.assert_close("out", out, z, **LOWP)
+        for name, a, b in zip(util.NAMES, g, grads):
+            util.assert_mostly_close(name, a, b, **LOWP)
+
+
+@pytest.mark.parametrize("splits", [1, 4])
+def test_mfma_forward_k_splits_large_logits(splits, monkeypatch):
+    """Scores spanning hundreds with the k-tiles split: every part goes through the repeat sweep with its own
+    reference maximum, and the merge must bring them to a common one.  Same statistical bound as the
+    unsplit large-logit case; split and unsplit runs must agree far more closely than either does with the
+    oracle (they round the same products)."""
+    inputs = orc.make_inputs(1, 2, 160, 64, torch.bfloat16, seed=22)
+    inputs[1] = (inputs[1].float() * 6).bfloat16()
+    inputs[2] = (inputs[2].float() * 6).bfloat16()
+    z, _, _ = util.oracle_tdp(inputs, 1 / 8, True)
+    monkeypatch.setenv("TRITT_FWD_SPLITS", "1")
+    whole, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
+    monkeypatch.setenv("TRITT_FWD_SPLITS", str(splits))
+    out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
+    assert torch.isfinite(out).all()
+    err = (out - z).abs()
+    assert (err > 5e-2).float().mean() < 0.01 and err.max() < 0.5, (err.max(), (err > 5e-2).float().mean())
+    assert (out - whole).abs().max() <= 2e-2, (out - whole).abs().max()
+
+
+def test_small_grid_forward_splits_by_itself():
+    """B=1 H=2 T=256 D=64: 32 query tiles, far below the split threshold, so the launcher splits four ways
+    by itself; output and (through the backward, which reads the log-sum-exp) gradients against the oracle,
+    and the workspace query covers the parts."""
+    from flash_trittention import _lib
+
+    alpha = 1 / 8
+    inputs = orc.make_inputs(1, 2, 256, 64, torch.bfloat16, seed=77)
+    z, _, grads = util.oracle_tdp(inputs, alpha, True)
+    out, g = util.run_tdp(inputs, alpha, True, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+    need = _lib.lib().tritt_tdp_fwd_workspace_bytes(1, 2, 256, 64, _lib.TRITT_BF16, 1, 256, 256, 256, 256, FORCE_MFMA)
+    assert need == 2 * 64 * 256 * 2 + 2 * 256 * 4 * 66 * 4, need
+
+
 def test_unaligned_views_are_copied():
     """Contiguous views that start in the middle of a storage (2-byte aligned) are accepted: the host side
     copies them to aligned memory before the library sees them."""
