@@ -766,6 +766,10 @@ constexpr size_t fwd_smem_bytes() {
            sizeof(float) * (WAVES * NT * (D + 4) + WAVES * 32) + 16;
 }
 
+}  // namespace tritt
+#include "tdp_fwd_band.hpp"
+namespace tritt {
+
 constexpr int kTpad = 128;  // U^T rows are padded to a multiple of the largest stage
 
 // Small grids split the k-tiles of every query tile over several workgroups: a causal grid ends in its heaviest
@@ -786,7 +790,45 @@ static size_t ut_bytes(int BH, int T, int D) {
 
 // TRITT_FWD_SPLITS overrides the count (tests, tuning sweeps); read per call, so the workspace query and
 // the launch that follows it must see the same value
+// The band-resident kernel takes windowed causal masks whose band fits in LDS (with room to spare for the
+// compiler's own use).  TRITT_FWD_BAND=0 switches it off (A/B runs).
+constexpr size_t kBandSmemLimit = 156 * 1024;
+static bool use_band_kernel(const MfmaFwdArgs& a) {
+    if (!(a.windowed && a.causal)) return false;
+    if (const char* e = getenv("TRITT_FWD_BAND"))
+        if (atoi(e) == 0) return false;
+    const int nr = band_rows(a.k1_window, a.k2_window);
+    const size_t smem = a.D == 32 ? band_smem_bytes<32>(nr) : a.D == 64 ? band_smem_bytes<64>(nr) : band_smem_bytes<128>(nr);
+    return smem <= kBandSmemLimit;
+}
+
+template <typename E, int D>
+static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
+    const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
+    hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
+                       a.T, Tp, D);
+    FwdParams<E> p;
+    p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
+    p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse;
+    p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + kBandQ - 1) / kBandQ;
+    p.scale_log2 = a.alpha * kLog2e;
+    p.causal = 1;
+    p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
+    p.splits = 1;
+    p.part = nullptr;
+    const int nr = band_rows(p.wa, p.wb);
+    const size_t smem = band_smem_bytes<D>(nr);
+    auto kern = tdp_fwd_band_kernel<E, D>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)smem);
+    if (e != hipSuccess) return e;
+    const int groups = (a.BH + 7) / 8;
+    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p, nr);
+    return hipGetLastError();
+}
+
 static int fwd_splits(const MfmaFwdArgs& a, int bq) {
+    if (use_band_kernel(a)) return 1;
     if (const char* e = getenv("TRITT_FWD_SPLITS")) return max(1, min(atoi(e), kMaxFwdSplits));
     const int wgs = a.BH * ((a.T + bq - 1) / bq);
     const bool banded = a.windowed && a.causal;
@@ -864,6 +906,18 @@ static hipError_t launch_d64(const MfmaFwdArgs& a, hipStream_t st) {
 }
 
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
+    if (use_band_kernel(a)) {
+        if (a.is_bf16) {
+            if (a.D == 32) return launch_band<__bf16, 32>(a, st);
+            if (a.D == 64) return launch_band<__bf16, 64>(a, st);
+            if (a.D == 128) return launch_band<__bf16, 128>(a, st);
+        } else {
+            if (a.D == 32) return launch_band<_Float16, 32>(a, st);
+            if (a.D == 64) return launch_band<_Float16, 64>(a, st);
+            if (a.D == 128) return launch_band<_Float16, 128>(a, st);
+        }
+        return hipErrorInvalidValue;
+    }
     if (a.windowed) {
         // one tile per wave, eight waves: the stages inside the band run the two-step interleaved loop,
         // the stages on its edges the general one

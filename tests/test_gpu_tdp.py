@@ -91,18 +91,24 @@ def test_lse_matches_oracle():
     util.assert_close("lse", ctx.saved[6].cpu(), lse, rtol=1e-5, atol=1e-5)
 
 
-def test_reproducible():
-    """Forward and dQ have a single owner per element and a fixed summation order: bitwise equal
-    from run to run.  dK1/dV1/dK2/dV2 of the MFMA path are summed over query tiles with fp32
-    atomics, so they are only reproducible to rounding; the fp32 VALU path is bitwise reproducible
-    throughout."""
+def test_reproducible(monkeypatch):
+    """Forward and (one workgroup per query tile) dQ have a single owner per element and a fixed summation
+    order: bitwise equal from run to run.  dK1/dV1/dK2/dV2 of the MFMA path are summed over query tiles with
+    fp32 atomics, and so is dQ when a small grid deals the rows of a tile out to several workgroups: those are
+    reproducible to rounding only.  The fp32 VALU path is bitwise reproducible throughout."""
     inputs = orc.make_inputs(1, 2, 96, 64, torch.bfloat16, seed=5)
+    monkeypatch.setenv("TRITT_BWD_SPLITS", "1")
     a = util.run_tdp(inputs, 1 / 8, True)
     b = util.run_tdp(inputs, 1 / 8, True)
     assert torch.equal(a[0], b[0])
     assert torch.equal(a[1][0], b[1][0]), "dq"
     for i in (1, 2, 3, 4):
         util.assert_close(util.NAMES[i], a[1][i], b[1][i], rtol=1e-2, atol=1e-2)
+    monkeypatch.delenv("TRITT_BWD_SPLITS")
+    e = util.run_tdp(inputs, 1 / 8, True)  # this grid is small: rows split, dQ accumulated atomically
+    assert torch.equal(a[0], e[0])
+    for i in range(5):
+        util.assert_close(util.NAMES[i], a[1][i], e[1][i], rtol=1e-2, atol=1e-2)
     c = util.run_tdp(inputs, 1 / 8, True, flags=1)
     d = util.run_tdp(inputs, 1 / 8, True, flags=1)
     assert torch.equal(c[0], d[0])
@@ -416,6 +422,40 @@ def test_small_grid_forward_splits_by_itself():
         util.assert_mostly_close(name, a, b, **LOWP)
     need = _lib.lib().tritt_tdp_fwd_workspace_bytes(1, 2, 256, 64, _lib.TRITT_BF16, 1, 256, 256, 256, 256, FORCE_MFMA)
     assert need == 2 * 64 * 256 * 2 + 2 * 256 * 4 * 66 * 4, need
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("windows", [(128, 128, 32, 32), (64, 64, 16, 16), (32, 90, 8, 60), (90, 32, 33, 0), (17, 5, 40, 40),
+                                     (3, 100, 1, 2)])
+def test_band_resident_forward_matches_streaming_and_oracle(windows, D, monkeypatch):
+    """Narrow windows take the band-resident forward (the whole band of a 32-query tile in LDS); switched off,
+    the streaming windowed kernel takes the same problem.  Both against the oracle, and against each other
+    far more tightly (they round the same products).  T = 333: eleven query tiles, the last one ragged;
+    where the band of a head dimension does not fit in LDS both runs are the streaming kernel."""
+    alpha = 1 / math.sqrt(D)
+    inputs = orc.make_inputs(1, 2, 333, D, torch.bfloat16, seed=D + windows[0])
+    z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
+    out, g = util.run_tdp(inputs, alpha, True, windows, flags=FORCE_MFMA)
+    monkeypatch.setenv("TRITT_FWD_BAND", "0")
+    ref, _ = util.run_tdp(inputs, alpha, True, windows, backward=False, flags=FORCE_MFMA)
+    util.assert_close("out", out, z, **LOWP)
+    util.assert_close("out vs streaming", out, ref, rtol=1e-2, atol=4e-3)
+    for name, a, b in zip(util.NAMES, g, grads):  # the backward reads the band kernel's log-sum-exp
+        util.assert_mostly_close(name, a, b, **LOWP)
+
+
+def test_band_resident_forward_large_logits():
+    """Scores spanning hundreds under a narrow window: single waves leave the fast sweep and repeat their
+    k-tile with the online softmax, and k-tiles with different reference maxima meet in the merge."""
+    inputs = orc.make_inputs(1, 2, 160, 64, torch.bfloat16, seed=23)
+    inputs[1] = (inputs[1].float() * 6).bfloat16()
+    inputs[2] = (inputs[2].float() * 6).bfloat16()
+    windows = (70, 50, 20, 30)
+    z, _, _ = util.oracle_tdp(inputs, 1 / 8, True, windows)
+    out, _ = util.run_tdp(inputs, 1 / 8, True, windows, backward=False, flags=FORCE_MFMA)
+    assert torch.isfinite(out).all()
+    err = (out - z).abs()
+    assert (err > 5e-2).float().mean() < 0.01 and err.max() < 0.5, (err.max(), (err > 5e-2).float().mean())
 
 
 def test_unaligned_views_are_copied():
