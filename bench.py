@@ -58,6 +58,22 @@ def make_inputs(B, H, T, D, dtype, seed=0, n=6):
     return [torch.randn(B, H, T, D, generator=g, dtype=torch.float32).to(dtype) for _ in range(n)]
 
 
+def nominal_clock_mhz():
+    """The device's nominal shader clock (hipDeviceAttributeClockRate = 5, kHz) from the HIP runtime the
+    process already has loaded; None if the runtime cannot be reached."""
+    import ctypes
+
+    for name in ("libamdhip64.so", "libamdhip64.so.7", "libamdhip64.so.6"):
+        try:
+            hip = ctypes.CDLL(name)
+            v = ctypes.c_int(0)
+            if hip.hipDeviceGetAttribute(ctypes.byref(v), 5, 0) == 0 and v.value > 0:
+                return v.value / 1e3
+        except OSError:
+            continue
+    return None
+
+
 def time_events(fn, iters, warmup, torch):
     """Average milliseconds per call, HIP events on the stream the kernels run on
     (torch's current stream, which is the stream handed to the library)."""
@@ -303,7 +319,8 @@ def main():
         "fwd_ms": ms_fwd, "bwd_ms": ms_bwd, "fwd_tflops": fwd_tf, "bwd_tflops": bwd_tf,
         "fwd_hbm_gbs": bytes_fwd / ms_fwd / 1e6, "bwd_hbm_gbs": bytes_bwd / ms_bwd / 1e6,
         "device": {"name": props.name, "cus": props.multi_processor_count,
-                   "clock_mhz": getattr(props, "clock_rate", 0) / 1e3},
+                   "nominal_clock_mhz": nominal_clock_mhz(),
+                   "peak_used": "2.5 PFLOP/s bf16 dense (256 CUs x 4096 flop/clk x 2.4 GHz nominal)"},
         # dominant kernel by time: tdp_bwd_rows_kernel, launched twice per backward (dQ,dK2,dV2 then
         # dK1,dU).  Each launch is credited half of the backward's algorithmic flops (6*D*N) and
         # half of the event-timed backward (the prep/finish kernels in that time are < 1 %).
