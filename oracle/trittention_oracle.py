@@ -58,17 +58,20 @@ def _windows(T: int, k1_window, k2_window, kk_left, kk_right):
 
 
 def tdp_mask(T: int, k1_window=None, k2_window=None, kk_left=None, kk_right=None,
-             q_lo: int = 0, q_hi: Optional[int] = None) -> torch.Tensor:
+             q_lo: int = 0, q_hi: Optional[int] = None, key_lo: int = 0,
+             key_hi: Optional[int] = None) -> torch.Tensor:
     """Boolean [q, j, k] tensor, True = masked OUT (trittention_pytorch.py:68-75).
 
     Axis order here is (q, j, k) — the reference stores (j, k, q); the
-    predicate is the same.  ``q_lo:q_hi`` selects a chunk of query rows.
+    predicate is the same.  ``q_lo:q_hi`` selects a chunk of query rows,
+    ``key_lo:key_hi`` the range of both key axes.
     """
     k1w, k2w, kl, kr = _windows(T, k1_window, k2_window, kk_left, kk_right)
     q_hi = T if q_hi is None else q_hi
+    key_hi = T if key_hi is None else key_hi
     q = torch.arange(q_lo, q_hi).view(-1, 1, 1)
-    j = torch.arange(T).view(1, -1, 1)
-    k = torch.arange(T).view(1, 1, -1)
+    j = torch.arange(key_lo, key_hi).view(1, -1, 1)
+    k = torch.arange(key_lo, key_hi).view(1, 1, -1)
     return ((j > q) | (k > q) | (q > j + k1w) | (q > k + k2w)
             | (j + kl < k) | (k + kr < j))
 
@@ -177,11 +180,14 @@ def dps_forward_backward(q, k1, k2, v1, v2, d_out, alpha, causal=True, k_diff=No
 
 
 def tdp_forward_backward_chunked(q, k1, k2, v1, v2, d_out, alpha, causal=True,
-                                 q_chunk: int = 64, need_grads: bool = True, rows=None):
-    """Same as ``tdp_forward_backward`` for ONE head ([T, D] inputs), full
-    windows only, evaluated in chunks of query rows so the [q, j, k] slab
-    stays small (T=1024: 64 x 1024 x 1024 fp32 = 268 MB).  For a causal chunk
-    only j,k <= last query of the chunk are touched.  ``rows=(lo, hi)``
+                                 q_chunk: int = 64, need_grads: bool = True, rows=None, **windows):
+    """Same as ``tdp_forward_backward`` for ONE head ([T, D] inputs),
+    evaluated in chunks of query rows so the [q, j, k] slab stays small
+    (T=1024: 64 x 1024 x 1024 fp32 = 268 MB).  For a causal chunk only
+    j,k <= last query of the chunk are touched, and under windows only keys
+    from (first query of the chunk - the larger query window) on: the keys
+    left out are masked for every query of the chunk, and a masked score
+    contributes an exact zero to the dense softmax.  ``rows=(lo, hi)``
     (forward only) evaluates just the query rows lo..hi-1 and returns
     [hi - lo, ...] tensors: spot checks at sequence lengths whose full plane
     is out of reach.
@@ -194,21 +200,23 @@ def tdp_forward_backward_chunked(q, k1, k2, v1, v2, d_out, alpha, causal=True,
     ql, k1l, k2l, v1l, v2l = leaves
     z_out = torch.empty_like(q[r_lo:r_hi])
     lse_out = torch.empty(r_hi - r_lo, dtype=q.dtype)
+    k1w, k2w, _, _ = _windows(T, windows.get("k1_window"), windows.get("k2_window"), None, None)
     for lo in range(r_lo, r_hi, q_chunk):
         hi = min(r_hi, lo + q_chunk)
         n = hi if causal else T          # keys beyond the chunk's last query are masked
+        ks = max(0, lo - max(k1w, k2w)) if causal else 0
         with torch.set_grad_enabled(need_grads):
-            u = F.silu(v1l[:n])
-            qk1 = ql[lo:hi, None, :] * k1l[None, :n, :]              # [c, n, D]
-            score = qk1 @ k2l[:n].t()                                # [c, j, k]
+            u = F.silu(v1l[ks:n])
+            qk1 = ql[lo:hi, None, :] * k1l[None, ks:n, :]            # [c, n - ks, D]
+            score = qk1 @ k2l[ks:n].t()                              # [c, j, k]
             if causal:
-                masked = tdp_mask(T, q_lo=lo, q_hi=hi)[:, :n, :n]
+                masked = tdp_mask(T, q_lo=lo, q_hi=hi, key_lo=ks, key_hi=n, **windows)
                 score = score.masked_fill(masked, MASK_FILL)
             flat = score.flatten(-2) * alpha
             lse = torch.logsumexp(flat, dim=-1)
             p = torch.softmax(flat, dim=-1).view(score.shape)
             t1 = torch.einsum("qjk,jd->qkd", p, u)
-            z = (t1 * v2l[None, :n, :]).sum(1)
+            z = (t1 * v2l[None, ks:n, :]).sum(1)
             if need_grads:
                 z.backward(d_out[lo:hi])
         z_out[lo - r_lo:hi - r_lo] = z.detach()

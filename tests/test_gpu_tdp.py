@@ -458,6 +458,24 @@ def test_band_resident_forward_large_logits():
     assert (err > 5e-2).float().mean() < 0.01 and err.max() < 0.5, (err.max(), (err > 5e-2).float().mean())
 
 
+@pytest.mark.parametrize("T,D,windows", [(8192, 64, (128, 128, 32, 32)), (8192, 128, (64, 64, 32, 32)),
+                                         (4096, 64, (300, 300, 64, 64)), (6000, 32, (200, 90, 17, 50))])
+def test_long_sequences_under_windows(T, D, windows):
+    """Windowed masks are how long sequences become affordable: forward and all five gradients at T = 4096 ..
+    8192 (band-resident forward where the band fits in LDS, streaming forward otherwise, banded backward)
+    against the oracle evaluated in chunks of query rows over the keys their windows can reach."""
+    print(f"case long windows T={T} D={D} {windows}", flush=True)
+    alpha = 1 / math.sqrt(D)
+    kw = dict(zip(("k1_window", "k2_window", "kk_left", "kk_right"), windows))
+    inputs = orc.make_inputs(1, 2, T, D, torch.bfloat16, seed=T % 1000 + D)
+    out, g = util.run_tdp(inputs, alpha, True, windows, flags=FORCE_MFMA)
+    for h in range(2):
+        z, _, grads = orc.tdp_forward_backward_chunked(*(t[0, h].float() for t in inputs), alpha, True, q_chunk=128, **kw)
+        util.assert_close(f"out[{h}]", out[0, h], z, **LOWP)
+        for name, a, b in zip(util.NAMES, g, grads):
+            util.assert_mostly_close(f"{name}[{h}]", a[0, h], b, **LOWP)
+
+
 def test_unaligned_views_are_copied():
     """Contiguous views that start in the middle of a storage (2-byte aligned) are accepted: the host side
     copies them to aligned memory before the library sees them."""

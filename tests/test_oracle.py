@@ -192,6 +192,18 @@ def test_chunked_row_range_equals_dense_rows(causal):
     assert torch.allclose(z[11:30], zr, atol=1e-12) and torch.allclose(lse[11:30], lser, atol=1e-12)
 
 
+@pytest.mark.parametrize("windows", [(5, 3, 4, 1), (2, 30, 0, 3), (12, 12, 40, 40)])
+def test_chunked_with_windows_equals_dense(windows):
+    T, D, alpha = 40, 8, 0.35
+    kw = dict(zip(("k1_window", "k2_window", "kk_left", "kk_right"), windows))
+    q, k1, k2, v1, v2, do = (rnd(T, D, seed=70 + s) for s in range(6))
+    z, lse, g = orc.tdp_forward_backward(q, k1, k2, v1, v2, do, alpha, True, **kw)
+    zc, lsec, gc = orc.tdp_forward_backward_chunked(q, k1, k2, v1, v2, do, alpha, True, q_chunk=7, **kw)
+    assert torch.allclose(z, zc, atol=1e-12) and torch.allclose(lse, lsec, atol=1e-12)
+    for a, b in zip(g, gc):
+        assert torch.allclose(a, b, atol=1e-11)
+
+
 def test_batched_heads_are_independent():
     B, H, T, D = 2, 3, 9, 4
     ins = [rnd(B, H, T, D, seed=90 + s) for s in range(5)]
