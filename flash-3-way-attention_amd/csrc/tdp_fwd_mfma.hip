@@ -55,7 +55,10 @@ constexpr float kLazyThreshold = 8.0f;
 // WIN: windowed causal masks.  The k-tile and stage loops run over the band only, every step goes
 // through the general (per tile, element-wise masked) loop, and the CAREFUL sweep tolerates rows whose
 // first valid key comes late.
-template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false>
+// MDIAG (NT = 1 only): the stages on the causal diagonal run the interleaved loop too, masked through the C
+// operand, instead of the general loop.  Pays on short sequences, where those stages are a large share of the
+// work; costs registers (a few more scratch reloads at D = 128), so long sequences keep the general loop.
+template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false>
 __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -555,7 +558,11 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                         general_until(min(st_hi + 1, max(st_lo, min(in_lo, nfull))));
                     }
                 }
-                for (; st < nfull; ++st, ++gstage) {
+                // MASKED (MDIAG: the stages that straddle the causal bound of this wave's query, or lie past it
+                // while other waves still need them): a key past the bound starts its score at -3e4, so its P
+                // is exactly 0.  Element i of a lane is key jb + key_of(0, i) + 8 g.
+                auto stage_nt1 = [&](auto masked_tag) {
+                    constexpr bool MASKED = decltype(masked_tag)::value;
                     const int sb = gstage & 1;
                     issue_stage(st < st_hi ? st + 1 : st_next);
                     if (st == st_lo && kt + 1 < nkt) issue_ktile(kt + 1);
@@ -563,10 +570,11 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     const E* utp = sUT + (sb * D + n) * LDU + g * 8;
                     v8 ka[KS], ua[DT][2], pa[2][2];
                     f32x16 sc[2];
+                    [[maybe_unused]] const int room = jmax[0] - st * JS - 8 * g;  // keys of this stage inside the bound
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
-                        sc[0][i] = 0.f;
-                        sc[1][i] = 0.f;
+                        sc[0][i] = (MASKED && key_of(0, i) > room) ? -3.0e4f : 0.f;
+                        sc[1][i] = (MASKED && key_of(0, i) + 32 > room) ? -3.0e4f : 0.f;
                     }
                     auto load_k = [&](int half) {
 #pragma unroll
@@ -622,6 +630,10 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     __builtin_amdgcn_sched_barrier(0);
                     commit_stage(sb ^ 1);
                     __syncthreads();
+                };
+                for (; st < nfull; ++st, ++gstage) stage_nt1(std::false_type{});
+                if constexpr (MDIAG && !WIN) {
+                    for (; st <= st_hi; ++st, ++gstage) stage_nt1(std::true_type{});
                 }
             }
             general_until(st_hi + 1);
@@ -838,7 +850,7 @@ static int fwd_splits(const MfmaFwdArgs& a, int bq) {
     return max(1, min(kAutoFwdSplits, min(by_size, by_tiles)));
 }
 
-template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false>
+template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false>
 static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
@@ -855,7 +867,7 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     p.splits = fwd_splits(a, BQ);
     p.part = reinterpret_cast<float*>(static_cast<char*>(a.ut) + ut_bytes(a.BH, a.T, D));
     constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS>();
-    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN>;
+    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG>;
     {
         // per call: the attribute belongs to the current device, and a process may drive several
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -905,6 +917,9 @@ static hipError_t launch_d64(const MfmaFwdArgs& a, hipStream_t st) {
     }
 }
 
+// D = 128: sequences up to this length run the diagonal stages in the interleaved loop (MDIAG)
+constexpr int kMaskedDiagonalUpTo = 768;
+
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
     if (use_band_kernel(a)) {
         if (a.is_bf16) {
@@ -935,11 +950,15 @@ hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
     if (a.is_bf16) {
         if (a.D == 32) return launch<__bf16, 32, 1, 8, 2, 64>(a, st);
         if (a.D == 64) return launch_d64<__bf16>(a, st);
-        if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64>(a, st);
+        if (a.D == 128)
+            return a.T <= kMaskedDiagonalUpTo ? launch<__bf16, 128, 1, 8, 2, 64, false, true>(a, st)
+                                               : launch<__bf16, 128, 1, 8, 2, 64>(a, st);
     } else {
         if (a.D == 32) return launch<_Float16, 32, 1, 8, 2, 64>(a, st);
         if (a.D == 64) return launch_d64<_Float16>(a, st);
-        if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64>(a, st);
+        if (a.D == 128)
+            return a.T <= kMaskedDiagonalUpTo ? launch<_Float16, 128, 1, 8, 2, 64, false, true>(a, st)
+                                               : launch<_Float16, 128, 1, 8, 2, 64>(a, st);
     }
     return hipErrorInvalidValue;
 }
