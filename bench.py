@@ -180,7 +180,7 @@ def main():
                     return flash_trittention(*ins, softmax_scale=1 / math.sqrt(128), k1_window=None, k2_window=None,
                                              kk_left=None, kk_right=None, causal=True)
 
-            ms = time_events(f, max(2, min(args.steps, 32768 // Ts)), 1, torch)
+            ms = time_events(f, max(3, min(4 * args.steps, 65536 // Ts)), 3 if Ts <= 2048 else 1, torch)
             fl = 4 * 128 * triples(1, 16, Ts)
             rows.append({"T": Ts, "ms": ms, "tflops": fl / ms / 1e9, "frac_of_bf16_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS,
                          "extra_device_bytes": torch.cuda.max_memory_allocated() - base_mem,

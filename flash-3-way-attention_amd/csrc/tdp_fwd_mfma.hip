@@ -21,7 +21,6 @@
 // by more than 2^8 ("lazy" max).  P is packed to 16 bit in the registers it already occupies
 // and fed straight back as the A operand of Tv += P * U.
 #include <stdlib.h>
-#include <string.h>
 
 #include <type_traits>
 
@@ -790,10 +789,9 @@ constexpr int kTpad = 128;  // U^T rows are padded to a multiple of the largest 
 // (4 under a windowed mask, whose k-tiles see only a few steps of j each).
 constexpr int kFwdSplitTarget = 768, kAutoFwdSplits = 4, kMaxFwdSplits = 8;
 
-static int fwd_variant();
-
-// queries per workgroup of the instantiation mfma_tdp_fwd() picks
-static int fwd_tile_queries(int D, int windowed) { return (D == 64 && !windowed && fwd_variant() != 2) ? 16 : 8; }
+// queries per workgroup of the instantiation mfma_tdp_fwd() picks: D = 64 without windows runs two queries per
+// wave, everything else one
+static int fwd_tile_queries(int D, int windowed) { return (D == 64 && !windowed) ? 16 : 8; }
 
 static size_t ut_bytes(int BH, int T, int D) {
     const size_t Tp = (size_t)(T + kTpad - 1) / kTpad * kTpad;
@@ -892,31 +890,6 @@ size_t mfma_tdp_fwd_workspace(const MfmaFwdArgs& a) {
 
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
 
-// Tile shape used for D = 64.  TRITT_FWD_VARIANT (read once) selects another instantiation for
-// tuning sweeps: "nt2w8" (default), "nt1w16", "nt1w8".
-static int fwd_variant() {
-    static int v = -1;
-    if (v < 0) {
-        const char* e = getenv("TRITT_FWD_VARIANT");
-        v = 0;
-        if (e) {
-            const char* names[] = {"nt2w8", "nt1w16", "nt1w8"};
-            for (int i = 0; i < 3; ++i)
-                if (!strcmp(e, names[i])) v = i;
-        }
-    }
-    return v;
-}
-
-template <typename E>
-static hipError_t launch_d64(const MfmaFwdArgs& a, hipStream_t st) {
-    switch (fwd_variant()) {
-        case 1: return launch<E, 64, 1, 16, 4, 64>(a, st);
-        case 2: return launch<E, 64, 1, 8, 4, 64>(a, st);
-        default: return launch<E, 64, 2, 8, 2, 64>(a, st);
-    }
-}
-
 // D = 128: sequences up to this length run the diagonal stages in the interleaved loop (MDIAG)
 constexpr int kMaskedDiagonalUpTo = 768;
 
@@ -949,13 +922,13 @@ hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
     }
     if (a.is_bf16) {
         if (a.D == 32) return launch<__bf16, 32, 1, 8, 2, 64>(a, st);
-        if (a.D == 64) return launch_d64<__bf16>(a, st);
+        if (a.D == 64) return launch<__bf16, 64, 2, 8, 2, 64>(a, st);
         if (a.D == 128)
             return a.T <= kMaskedDiagonalUpTo ? launch<__bf16, 128, 1, 8, 2, 64, false, true>(a, st)
                                                : launch<__bf16, 128, 1, 8, 2, 64>(a, st);
     } else {
         if (a.D == 32) return launch<_Float16, 32, 1, 8, 2, 64>(a, st);
-        if (a.D == 64) return launch_d64<_Float16>(a, st);
+        if (a.D == 64) return launch<_Float16, 64, 2, 8, 2, 64>(a, st);
         if (a.D == 128)
             return a.T <= kMaskedDiagonalUpTo ? launch<_Float16, 128, 1, 8, 2, 64, false, true>(a, st)
                                                : launch<_Float16, 128, 1, 8, 2, 64>(a, st);
