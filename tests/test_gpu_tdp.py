@@ -476,6 +476,55 @@ def test_long_sequences_under_windows(T, D, windows):
             util.assert_mostly_close(f"{name}[{h}]", a[0, h], b, **LOWP)
 
 
+@pytest.mark.parametrize("shape", [(2, 4, 256, 64, (None,) * 4), (1, 3, 200, 128, (None,) * 4), (1, 2, 300, 64, (64, 64, 16, 16))])
+def test_forward_and_backward_replay_from_a_hip_graph(shape):
+    """The library only launches kernels on the stream it is given (no allocation, copy, memset or
+    synchronisation inside), so a forward + backward can be captured into a HIP graph once and replayed for
+    launch-bound small problems.  Three replays on fresh inputs, with eager work and synchronisations in between,
+    each against the eager result of the same inputs: bitwise for O, to rounding for the gradients
+    (atomically accumulated)."""
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    B, H, T, D, windows = shape
+    alpha = 1 / math.sqrt(D)
+    kw = dict(softmax_scale=alpha, k1_window=windows[0], k2_window=windows[1], kk_left=windows[2], kk_right=windows[3],
+              causal=True)
+    static = [t.cuda().requires_grad_(True) for t in orc.make_inputs(B, H, T, D, torch.bfloat16, seed=1)[:5]]
+    static_do = torch.zeros(B, H, T, D, dtype=torch.bfloat16, device="cuda")
+
+    def step():
+        out = flash_trittention(*static, **kw)
+        grads = torch.autograd.grad(out, static, static_do)
+        return out, grads
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_out, g_grads = step()
+    for rep in range(3):
+        fresh = orc.make_inputs(B, H, T, D, torch.bfloat16, seed=10 + rep)
+        with torch.no_grad():
+            for dst, src in zip(static, fresh[:5]):
+                dst.copy_(src)
+            static_do.copy_(fresh[5])
+        graph.replay()
+        torch.cuda.synchronize()
+        got_out, got_grads = g_out.clone(), [g.clone() for g in g_grads]
+        e_out, e_grads = step()   # eager, same inputs
+        torch.cuda.synchronize()
+        assert torch.equal(got_out, e_out), rep
+        for name, a, b in zip(util.NAMES, got_grads, e_grads):
+            util.assert_close(f"{name} replay {rep}", a.float().cpu(), b.float().cpu(), rtol=2e-2, atol=2e-2)
+        z, _, ref = util.oracle_tdp(fresh, alpha, True, windows)
+        util.assert_close("out vs oracle", got_out.float().cpu(), z, **LOWP)
+
+
 def test_unaligned_views_are_copied():
     """Contiguous views that start in the middle of a storage (2-byte aligned) are accepted: the host side
     copies them to aligned memory before the library sees them."""
