@@ -20,6 +20,11 @@
 // CAREFUL sweep: online softmax whose reference maximum is raised only when a score exceeds it
 // by more than 2^8 ("lazy" max).  P is packed to 16 bit in the registers it already occupies
 // and fed straight back as the A operand of Tv += P * U.
+//
+// Small grids: the k-tiles of a query tile are dealt out to several workgroups (FwdParams::splits), each
+// writes its unnormalised output, reference maximum and row sum, and fwd_merge_kernel joins them.
+// Narrow windowed masks take another kernel altogether (tdp_fwd_band.hpp): the whole band of a query
+// tile resident in LDS, waves independent after one barrier.
 #include <stdlib.h>
 
 #include <type_traits>
