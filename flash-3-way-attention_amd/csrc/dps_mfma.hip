@@ -41,6 +41,17 @@ __device__ __forceinline__ int row_of_key(int k) {
     const int i = 8 * (k >> 4) + (k & 7), g = (k >> 3) & 1;
     return ((i >> 2) << 3) | (g << 2) | (i & 3);
 }
+// XCD-aware block order of a 1-D grid of 8 * ceil(BH / 8) * ntiles workgroups: consecutive block ids go to
+// different XCDs, so every XCD gets its own (batch, head) slices and their packed operands stay in that
+// XCD's L2.  `tile` counts 0 .. ntiles-1 in launch order.  False: a padding block (BH not a multiple of 8).
+__device__ __forceinline__ bool block_to_tile(int BH, int& bh, int& tile) {
+    const int groups = (BH + 7) / 8;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    bh = (slot % groups) * 8 + xcd;
+    tile = slot / groups;
+    return bh < BH;
+}
+
 // element offsets of (row, d) in the two packings
 template <int D>
 __device__ __forceinline__ size_t p1_index(int row, int d) {
@@ -107,6 +118,7 @@ struct AttnFwdP {
     E* outm_p2;         // out * mul, packing P2, or null
     float* lse;         // [BH][lse_stride]
     int lse_stride;
+    int BH;
     float lse_scale;    // lse = lse_scale * log2-sum-exp2
     int T, Tp;
     float scale_log2;
@@ -123,7 +135,9 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     float* sM = sO + kW * D * kLdr;                  // [kW][32]
     float* sL = sM + kW * 32;                        // [kW][32]
 
-    const int bh = blockIdx.y, r0 = (gridDim.x - 1 - blockIdx.x) * 32;  // longest rows first
+    int bh, tile;
+    if (!block_to_tile(p.BH, bh, tile)) return;
+    const int r0 = (p.Tp / 32 - 1 - tile) * 32;  // longest rows first
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T, Tp = p.Tp;
@@ -315,7 +329,7 @@ struct AttnBwdP {
     const float* bias;       // [BH][Tp] log2 units or null
     const float* lse2;       // [BH][Tp] log2 units
     const float* delta;      // [BH][Tp]
-    int T, Tp;
+    int BH, T, Tp;
     float alpha;
     int causal, k_diff;
     // row kernel output: dx = alpha * sum + addend
@@ -342,7 +356,9 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
     extern __shared__ __align__(16) char smem_raw[];
     float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
 
-    const int bh = blockIdx.y, r0 = (gridDim.x - 1 - blockIdx.x) * 32;
+    int bh, tile;
+    if (!block_to_tile(p.BH, bh, tile)) return;
+    const int r0 = (p.Tp / 32 - 1 - tile) * 32;
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T, Tp = p.Tp;
@@ -479,7 +495,9 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     float* sB = sO + kW * D * kLdr;                  // [kW][32]  dbias partials
     float* sR = sB + kW * 32;                        // [8][32]   delta1 partials
 
-    const int bh = blockIdx.y, c0 = blockIdx.x * 32;  // lowest key rows are the longest
+    int bh, tile;
+    if (!block_to_tile(p.BH, bh, tile)) return;
+    const int c0 = tile * 32;  // lowest key rows are the longest
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T, Tp = p.Tp;
@@ -708,13 +726,15 @@ struct PrepP {
     E *up1, *k1p1, *k2p1, *qp1, *dop1;  // packing P1
     E *up2, *k1p2, *k2p2, *qp2, *dop2;  // packing P2
     float *lse2, *delta;
-    int T, Tp;
+    int BH, T, Tp;
 };
 
 template <typename E, int D>
 __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
     using v8 = typename Mma<E>::v8;
-    const int bh = blockIdx.y, j0 = blockIdx.x * 32, T = p.T, Tp = p.Tp;
+    int bh, tile;
+    if (!block_to_tile(p.BH, bh, tile)) return;
+    const int j0 = tile * 32, T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp;
     // one 16-byte piece (8 consecutive d of one row) per step: it is one piece of P1 and 8 elements of P2
     for (int idx = threadIdx.x; idx < 32 * (D / 8); idx += 256) {
@@ -822,7 +842,7 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, for_bwd);
     char* ws = static_cast<char*>(a.workspace);
-    const dim3 grid(Tp / 32, a.BH);
+    const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
     auto kern = attn_fwd_mfma_kernel<E, D>;
     hipError_t e = allow_smem(kern, fwd_smem<D>());
     if (e != hipSuccess) return e;
@@ -832,7 +852,7 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
         PrepP<E> pp{};
         pp.v1 = (const E*)a.v1; pp.k1 = (const E*)a.k1; pp.k2 = (const E*)a.k2;
         pp.up2 = (E*)(ws + l.up2); pp.k1p1 = (E*)(ws + l.k1p1); pp.k2p1 = (E*)(ws + l.k2p1);
-        pp.T = a.T; pp.Tp = Tp;
+        pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp;
         hipLaunchKernelGGL((dps_prep_kernel<E, D>), grid, dim3(256), 0, st, pp);
     }
     // inner: rows K2[t], keys K1, values U; R (fp32, backward only), W = R * V2 and W^T, lse1 (log2)
@@ -843,14 +863,14 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     p.outm_p1 = for_bwd ? (E*)(ws + l.wp1) : nullptr;
     p.outm_p2 = (E*)(ws + l.wp2);
     p.lse = (float*)(ws + l.lse1); p.lse_stride = Tp; p.lse_scale = 1.0f;
-    p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff;
+    p.BH = a.BH; p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff;
     hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, p);
     if (for_bwd) return hipGetLastError();
     // outer: rows Q[q], keys K2 with bias lse1, values W; O and LSE (natural log)
     AttnFwdP<E> o{};
     o.x = (const E*)a.q; o.kp = (const E*)(ws + l.k2p1); o.vp2 = (const E*)(ws + l.wp2); o.bias = (const float*)(ws + l.lse1);
     o.out = (E*)a.o_out; o.lse = a.lse_out; o.lse_stride = a.T; o.lse_scale = kLn2;
-    o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T;
+    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T;
     hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, o);
     return hipGetLastError();
 }
@@ -860,7 +880,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, true);
     char* ws = static_cast<char*>(a.workspace);
-    const dim3 grid(Tp / 32, a.BH);
+    const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
     auto krow = attn_bwd_row_mfma_kernel<E, D>;
     auto kcol_link = attn_bwd_col_mfma_kernel<E, D, true>;
     auto kcol = attn_bwd_col_mfma_kernel<E, D, false>;
@@ -878,7 +898,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     pp.up2 = (E*)(ws + l.up2); pp.k1p2 = (E*)(ws + l.k1p2); pp.k2p2 = (E*)(ws + l.k2p2);
     pp.qp2 = (E*)(ws + l.qp2); pp.dop2 = (E*)(ws + l.dop2);
     pp.lse2 = (float*)(ws + l.lse2); pp.delta = (float*)(ws + l.delta);
-    pp.T = a.T; pp.Tp = Tp;
+    pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp;
     hipLaunchKernelGGL((dps_prep_kernel<E, D>), grid, dim3(256), 0, st, pp);
     // recompute the inner pass: R, W, W^T, lse1
     e = run_fwd<E, D>(a, st, true);
@@ -891,7 +911,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     o.xp = (const E*)(ws + l.qp1); o.gp = (const E*)(ws + l.dop1);
     o.xp2 = (const E*)(ws + l.qp2); o.gp2 = (const E*)(ws + l.dop2);
     o.bias = (const float*)(ws + l.lse1); o.lse2 = (const float*)(ws + l.lse2); o.delta = (const float*)(ws + l.delta);
-    o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T;
+    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T;
     o.dx = (E*)a.dq;
     o.dk_f32 = (float*)(ws + l.dk2p);
     o.r_f32 = (const float*)(ws + l.r); o.v2 = (const E*)a.v2; o.dv2 = (E*)a.dv2;
@@ -906,7 +926,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     i.xp = (const E*)(ws + l.k2p1); i.gp = (const E*)(ws + l.drp1);
     i.xp2 = (const E*)(ws + l.k2p2); i.gp2 = (const E*)(ws + l.drp2);
     i.lse2 = (const float*)(ws + l.lse1); i.delta = (const float*)(ws + l.delta1);
-    i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff;
+    i.BH = a.BH; i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff;
     i.addend = (const float*)(ws + l.dk2p); i.dx = (E*)a.dk2;
     i.dk = (E*)a.dk1; i.v1 = (const E*)a.v1; i.dv = (E*)a.dv1;
     hipLaunchKernelGGL(krow, grid, dim3(64 * kW), row_smem<D>(), st, i);
