@@ -12,8 +12,8 @@
 //   attn_bwd_row_mfma_kernel   owner = 32 query-like rows;  dX
 //   attn_bwd_col_mfma_kernel   owner = 32 key-like rows;    dK, dV, dbias (+ the element-wise link
 //                              between the two passes when it runs the outer pass)
-// A workgroup is 4 waves that share one owner tile and split the streamed 32-row tiles between
-// them round-robin (their partial results meet in LDS), so T = 1024 already gives 4096 waves.
+// A workgroup is kW (2 or 4) waves that share one owner tile and split the streamed 32-row tiles between
+// them round-robin (their partial results meet in LDS).
 // Every tile is computed transposed where needed so that the owner index sits on the MFMA column
 // (= lane) axis: softmax statistics, LSE and Delta stay lane-local, and with the permuted row order
 // of mfma.hpp the probabilities leave one MFMA in exactly the operand layout of the next.
@@ -32,7 +32,6 @@
 namespace tritt {
 namespace {
 
-constexpr int kW = 4;     // waves per workgroup
 constexpr int kLdr = 33;  // LDS row stride (floats) of the cross-wave reduction tiles
 constexpr float kLazyRaise = 8.0f;  // log2 units a score may exceed the running reference before it is raised
 
@@ -125,7 +124,8 @@ struct AttnFwdP {
     int causal, k_diff;
 };
 
-template <typename E, int D>
+// kW: waves per workgroup (they split the streamed tiles of one owner tile)
+template <typename E, int D, int kW>
 __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     const float inv = 1.0f / ll;
     if (dg == 0 && row < T) p.lse[(size_t)bh * p.lse_stride + row] = (mm + fast_log2(ll)) * p.lse_scale;
 #pragma unroll
-    for (int c = dg; c < D / 8; c += 8) {  // 16-byte pieces dg, dg + 8, ... of the row
+    for (int c = dg; c < D / 8; c += 2 * kW) {  // 16-byte pieces dg, dg + 2 kW, ... of the row
         const int d0 = 8 * c;
         float o[8];
 #pragma unroll
@@ -348,7 +348,7 @@ struct AttnBwdP {
     float* delta1;           // [BH][Tp]
 };
 
-template <typename E, int D>
+template <typename E, int D, int kW>
 __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -467,7 +467,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
     const int rr = tid & 31, dg = tid >> 5, row = r0 + rr;
     if (row >= T) return;
 #pragma unroll
-    for (int c = dg; c < D / 8; c += 8) {  // 16-byte pieces dg, dg + 8, ... of the row
+    for (int c = dg; c < D / 8; c += 2 * kW) {  // 16-byte pieces dg, dg + 2 kW, ... of the row
         const int d0 = 8 * c;
         const size_t off = base + (size_t)row * D + d0;
         v8 ov;
@@ -485,7 +485,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
 }
 
 // --------------------------------------------------------------------------- backward, columns
-template <typename E, int D, bool LINK>
+template <typename E, int D, int kW, bool LINK>
 __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -493,7 +493,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     extern __shared__ __align__(16) char smem_raw[];
     float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
     float* sB = sO + kW * D * kLdr;                  // [kW][32]  dbias partials
-    float* sR = sB + kW * 32;                        // [8][32]   delta1 partials
+    float* sR = sB + kW * 32;                        // [2 kW][32]   delta1 partials
 
     int bh, tile;
     if (!block_to_tile(p.BH, bh, tile)) return;
@@ -625,7 +625,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     __syncthreads();
     if (row < T) {
 #pragma unroll
-        for (int c = dg; c < D / 8; c += 8) {
+        for (int c = dg; c < D / 8; c += 2 * kW) {
             const int d0 = 8 * c;
             const size_t off = base + (size_t)row * D + d0;
             float o[8];
@@ -654,7 +654,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     __syncthreads();
     float part = 0.f;
 #pragma unroll
-    for (int c = dg; c < D / 8; c += 8) {  // 16-byte pieces dg, dg + 8, ... of the row
+    for (int c = dg; c < D / 8; c += 2 * kW) {  // 16-byte pieces dg, dg + 2 kW, ... of the row
         const int d0 = 8 * c;
         const size_t off = base + (size_t)row * D + d0;
         float o[8];
@@ -706,7 +706,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
         if (tid < 32) {
             float d1 = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) d1 += sR[j * 32 + tid];
+            for (int j = 0; j < 2 * kW; ++j) d1 += sR[j * 32 + tid];
 #pragma unroll
             for (int w = 0; w < kW; ++w) d1 -= sB[w * 32 + tid];
             p.delta1[vb + c0 + tid] = (c0 + tid < T) ? d1 : 0.f;
@@ -825,11 +825,11 @@ Layout layout(int BH, int T, int D, bool bwd) {
     return l;
 }
 
-template <int D>
+template <int D, int kW>
 constexpr size_t fwd_smem() { return 4 * (size_t)(kW * D * kLdr + 2 * kW * 32); }
-template <int D>
-constexpr size_t col_smem() { return 4 * (size_t)(kW * D * kLdr + kW * 32 + 8 * 32); }
-template <int D>
+template <int D, int kW>
+constexpr size_t col_smem() { return 4 * (size_t)(kW * D * kLdr + kW * 32 + 2 * kW * 32); }
+template <int D, int kW>
 constexpr size_t row_smem() { return 4 * (size_t)(kW * D * kLdr); }
 
 template <typename F>
@@ -837,14 +837,14 @@ hipError_t allow_smem(F kern, size_t bytes) {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
-template <typename E, int D>
+template <typename E, int D, int kW>
 hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, for_bwd);
     char* ws = static_cast<char*>(a.workspace);
     const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
-    auto kern = attn_fwd_mfma_kernel<E, D>;
-    hipError_t e = allow_smem(kern, fwd_smem<D>());
+    auto kern = attn_fwd_mfma_kernel<E, D, kW>;
+    hipError_t e = allow_smem(kern, fwd_smem<D, kW>());
     if (e != hipSuccess) return e;
     const float sl2 = a.alpha * kLog2e;
 
@@ -864,29 +864,29 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     p.outm_p2 = (E*)(ws + l.wp2);
     p.lse = (float*)(ws + l.lse1); p.lse_stride = Tp; p.lse_scale = 1.0f;
     p.BH = a.BH; p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff;
-    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, p);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), (fwd_smem<D, kW>()), st, p);
     if (for_bwd) return hipGetLastError();
     // outer: rows Q[q], keys K2 with bias lse1, values W; O and LSE (natural log)
     AttnFwdP<E> o{};
     o.x = (const E*)a.q; o.kp = (const E*)(ws + l.k2p1); o.vp2 = (const E*)(ws + l.wp2); o.bias = (const float*)(ws + l.lse1);
     o.out = (E*)a.o_out; o.lse = a.lse_out; o.lse_stride = a.T; o.lse_scale = kLn2;
     o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T;
-    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), fwd_smem<D>(), st, o);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), (fwd_smem<D, kW>()), st, o);
     return hipGetLastError();
 }
 
-template <typename E, int D>
+template <typename E, int D, int kW>
 hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, true);
     char* ws = static_cast<char*>(a.workspace);
     const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
-    auto krow = attn_bwd_row_mfma_kernel<E, D>;
-    auto kcol_link = attn_bwd_col_mfma_kernel<E, D, true>;
-    auto kcol = attn_bwd_col_mfma_kernel<E, D, false>;
-    hipError_t e = allow_smem(krow, row_smem<D>());
-    if (e == hipSuccess) e = allow_smem(kcol_link, col_smem<D>());
-    if (e == hipSuccess) e = allow_smem(kcol, col_smem<D>());
+    auto krow = attn_bwd_row_mfma_kernel<E, D, kW>;
+    auto kcol_link = attn_bwd_col_mfma_kernel<E, D, kW, true>;
+    auto kcol = attn_bwd_col_mfma_kernel<E, D, kW, false>;
+    hipError_t e = allow_smem(krow, row_smem<D, kW>());
+    if (e == hipSuccess) e = allow_smem(kcol_link, col_smem<D, kW>());
+    if (e == hipSuccess) e = allow_smem(kcol, col_smem<D, kW>());
     if (e != hipSuccess) return e;
 
     PrepP<E> pp{};
@@ -901,7 +901,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp;
     hipLaunchKernelGGL((dps_prep_kernel<E, D>), grid, dim3(256), 0, st, pp);
     // recompute the inner pass: R, W, W^T, lse1
-    e = run_fwd<E, D>(a, st, true);
+    e = run_fwd<E, D, kW>(a, st, true);
     if (e != hipSuccess) return e;
 
     // outer pass: X = Q, G = dO, K = K2 (bias lse1), V = W
@@ -916,8 +916,8 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     o.dk_f32 = (float*)(ws + l.dk2p);
     o.r_f32 = (const float*)(ws + l.r); o.v2 = (const E*)a.v2; o.dv2 = (E*)a.dv2;
     o.dr = (E*)(ws + l.dr); o.dr_p1 = (E*)(ws + l.drp1); o.dr_p2 = (E*)(ws + l.drp2); o.delta1 = (float*)(ws + l.delta1);
-    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), row_smem<D>(), st, o);
-    hipLaunchKernelGGL(kcol_link, grid, dim3(64 * kW), col_smem<D>(), st, o);
+    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), (row_smem<D, kW>()), st, o);
+    hipLaunchKernelGGL(kcol_link, grid, dim3(64 * kW), (col_smem<D, kW>()), st, o);
 
     // inner pass: X = K2, G = dR, K = K1, V = U
     AttnBwdP<E> i{};
@@ -929,8 +929,8 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     i.BH = a.BH; i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff;
     i.addend = (const float*)(ws + l.dk2p); i.dx = (E*)a.dk2;
     i.dk = (E*)a.dk1; i.v1 = (const E*)a.v1; i.dv = (E*)a.dv1;
-    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), row_smem<D>(), st, i);
-    hipLaunchKernelGGL(kcol, grid, dim3(64 * kW), col_smem<D>(), st, i);
+    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), (row_smem<D, kW>()), st, i);
+    hipLaunchKernelGGL(kcol, grid, dim3(64 * kW), (col_smem<D, kW>()), st, i);
     return hipGetLastError();
 }
 
@@ -940,18 +940,31 @@ bool mfma_dps_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D
 size_t mfma_dps_fwd_workspace(int BH, int T, int D) { return layout(BH, T, D, false).total; }
 size_t mfma_dps_bwd_workspace(int BH, int T, int D) { return layout(BH, T, D, true).total; }
 
-hipError_t mfma_dps_fwd(const MfmaDpsArgs& a, hipStream_t st) {
-    if (a.D == 32) return a.is_bf16 ? run_fwd<__bf16, 32>(a, st, false) : run_fwd<_Float16, 32>(a, st, false);
-    if (a.D == 64) return a.is_bf16 ? run_fwd<__bf16, 64>(a, st, false) : run_fwd<_Float16, 64>(a, st, false);
-    if (a.D == 128) return a.is_bf16 ? run_fwd<__bf16, 128>(a, st, false) : run_fwd<_Float16, 128>(a, st, false);
+// Waves per workgroup, measured: two at D = 128 and for long sequences at D = 64 (fewer partial results to
+// merge, longer-lived waves), four otherwise (short sequences and D = 32 want the parallelism).
+static bool two_waves(const MfmaDpsArgs& a) { return a.D == 128 || (a.D == 64 && a.T >= 1024); }
+
+template <typename E>
+static hipError_t dps_fwd_typed(const MfmaDpsArgs& a, hipStream_t st) {
+    if (a.D == 32) return run_fwd<E, 32, 4>(a, st, false);
+    if (a.D == 64) return two_waves(a) ? run_fwd<E, 64, 2>(a, st, false) : run_fwd<E, 64, 4>(a, st, false);
+    if (a.D == 128) return run_fwd<E, 128, 2>(a, st, false);
+    return hipErrorInvalidValue;
+}
+template <typename E>
+static hipError_t dps_bwd_typed(const MfmaDpsArgs& a, hipStream_t st) {
+    if (a.D == 32) return run_bwd<E, 32, 4>(a, st);
+    if (a.D == 64) return two_waves(a) ? run_bwd<E, 64, 2>(a, st) : run_bwd<E, 64, 4>(a, st);
+    if (a.D == 128) return run_bwd<E, 128, 2>(a, st);
     return hipErrorInvalidValue;
 }
 
+hipError_t mfma_dps_fwd(const MfmaDpsArgs& a, hipStream_t st) {
+    return a.is_bf16 ? dps_fwd_typed<__bf16>(a, st) : dps_fwd_typed<_Float16>(a, st);
+}
+
 hipError_t mfma_dps_bwd(const MfmaDpsArgs& a, hipStream_t st) {
-    if (a.D == 32) return a.is_bf16 ? run_bwd<__bf16, 32>(a, st) : run_bwd<_Float16, 32>(a, st);
-    if (a.D == 64) return a.is_bf16 ? run_bwd<__bf16, 64>(a, st) : run_bwd<_Float16, 64>(a, st);
-    if (a.D == 128) return a.is_bf16 ? run_bwd<__bf16, 128>(a, st) : run_bwd<_Float16, 128>(a, st);
-    return hipErrorInvalidValue;
+    return a.is_bf16 ? dps_bwd_typed<__bf16>(a, st) : dps_bwd_typed<_Float16>(a, st);
 }
 
 }  // namespace tritt
