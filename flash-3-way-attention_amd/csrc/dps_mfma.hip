@@ -732,18 +732,21 @@ struct PrepP {
 template <typename E, int D>
 __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
     using v8 = typename Mma<E>::v8;
-    int bh, tile;
-    if (!block_to_tile(p.BH, bh, tile)) return;
-    const int j0 = tile * 32, T = p.T, Tp = p.Tp;
+    int bh, tile_id;
+    if (!block_to_tile(p.BH, bh, tile_id)) return;
+    const int j0 = tile_id * 32, T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp;
-    // one 16-byte piece (8 consecutive d of one row) per step: it is one piece of P1 and 8 elements of P2
-    for (int idx = threadIdx.x; idx < 32 * (D / 8); idx += 256) {
-        const int j = j0 + idx / (D / 8), d0 = (idx % (D / 8)) * 8;
-        const bool in = j < T;
-        const size_t off = base + (size_t)(in ? j : 0) * D + d0;
-        const size_t o1 = tb + p1_index<D>(j, d0);
-        auto emit = [&](const E* src, E* dst1, E* dst2, bool silu) {
-            if (!dst1 && !dst2 && !(silu && p.u)) return;
+    // One 16-byte piece (8 consecutive d of one row) per thread and step: it is one piece of P1 as it stands.
+    // P2 wants 8 consecutive rows of one column in a piece, so the 32 x D tile goes through LDS and comes
+    // back out transposed, again as whole 16-byte pieces (element-wise 2-byte stores were most of this
+    // kernel's time).
+    __shared__ E sT[32][D + 2];
+    auto emit = [&](const E* src, E* dst1, E* dst2, bool silu) {
+        if (!dst1 && !dst2 && !(silu && p.u)) return;  // uniform over the workgroup
+        for (int idx = threadIdx.x; idx < 32 * (D / 8); idx += 256) {
+            const int jj = idx / (D / 8), j = j0 + jj, d0 = (idx % (D / 8)) * 8;
+            const bool in = j < T;
+            const size_t off = base + (size_t)(in ? j : 0) * D + d0;
             v8 x;
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = (E)0.f;
@@ -753,17 +756,30 @@ __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
                 for (int e = 0; e < 8; ++e) x[e] = (E)(in ? silu_f((float)x[e]) : 0.f);
                 if (p.u && in) *reinterpret_cast<v8*>(p.u + off) = x;
             }
-            if (dst1) *reinterpret_cast<v8*>(dst1 + o1) = x;
-            if (dst2)
+            if (dst1) *reinterpret_cast<v8*>(dst1 + tb + p1_index<D>(j, d0)) = x;
+            if (dst2) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) dst2[tb + p2_index<D>(j, d0 + e)] = x[e];
-        };
-        emit(p.v1, p.up1, p.up2, true);
-        emit(p.k1, p.k1p1, p.k1p2, false);
-        emit(p.k2, p.k2p1, p.k2p2, false);
-        if (p.q) emit(p.q, p.qp1, p.qp2, false);
-        if (p.d_o) emit(p.d_o, p.dop1, p.dop2, false);
-    }
+                for (int e = 0; e < 8; ++e) sT[jj][d0 + e] = x[e];
+            }
+        }
+        if (dst2) {
+            __syncthreads();
+            for (int idx = threadIdx.x; idx < (D / 32) * 2 * 64; idx += 256) {
+                const int ln = idx & 63, kk = (idx >> 6) & 1, dt = idx >> 7;
+                const int r = kk * 16 + (ln >> 5) * 8, d = dt * 32 + (ln & 31);
+                v8 y;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) y[e] = sT[r + e][d];
+                *reinterpret_cast<v8*>(dst2 + tb + ((size_t)((tile_id * (D / 32) + dt) * 2 + kk) * 64 + ln) * 8) = y;
+            }
+            __syncthreads();
+        }
+    };
+    emit(p.v1, p.up1, p.up2, true);
+    emit(p.k1, p.k1p1, p.k1p2, false);
+    emit(p.k2, p.k2p1, p.k2p2, false);
+    if (p.q) emit(p.q, p.qp1, p.qp2, false);
+    if (p.d_o) emit(p.d_o, p.dop1, p.dop2, false);
     if (p.delta) {
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         for (int jj = wave; jj < 32; jj += 4) {
