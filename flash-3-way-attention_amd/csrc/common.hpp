@@ -55,6 +55,47 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// One 64-row block of a row-major [T][D] tensor, transposed into dst[d][Tp] (rows past T become zeros), through
+// an LDS tile so that both the reads (8 consecutive d of a row) and the writes (8 consecutive rows of a column)
+// are whole 16-byte pieces: an element-wise transposed copy touches one cache line per lane and is bound by the
+// address traffic of the vector memory path.  256 threads; `tile` holds 64 x (D + 2) elements; the caller
+// synchronises the workgroup between transpose_load and transpose_store (and again before reusing the tile).
+// SILU applies x -> SiLU(x) on the way and, with `rows` non-null, also stores the result row-major.
+template <typename E, bool SILU>
+__device__ __forceinline__ void transpose_load(const E* __restrict__ src, E* __restrict__ rows, E* tile, int j0, int T,
+                                               int D) {
+    typedef __attribute__((ext_vector_type(8))) E e8;
+    const int ld = D + 2, cpr = D / 8;
+    for (int idx = threadIdx.x; idx < 64 * cpr; idx += 256) {
+        const int jj = idx / cpr, c = idx % cpr, j = j0 + jj;
+        e8 x;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = (E)0.f;
+        if (j < T) {
+            x = *reinterpret_cast<const e8*>(src + (size_t)j * D + c * 8);
+            if (SILU) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (E)silu_f((float)x[e]);
+                if (rows) *reinterpret_cast<e8*>(rows + (size_t)j * D + c * 8) = x;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) tile[jj * ld + c * 8 + e] = x[e];
+    }
+}
+template <typename E>
+__device__ __forceinline__ void transpose_store(E* __restrict__ dst, const E* tile, int j0, int Tp, int D) {
+    typedef __attribute__((ext_vector_type(8))) E e8;
+    const int ld = D + 2;
+    for (int idx = threadIdx.x; idx < D * 8; idx += 256) {
+        const int d = idx >> 3, cj = idx & 7;
+        e8 y;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = tile[(cj * 8 + e) * ld + d];
+        *reinterpret_cast<e8*>(dst + (size_t)d * Tp + j0 + cj * 8) = y;
+    }
+}
+
 // Window parameters of the triple-dot causal mask, expressed for a "staged"
 // index a and an "owner" index b (a = j, b = k in the natural orientation):
 //   valid  <=>  a<=q, b<=q, q<=a+wa, q<=b+wb, b<=a+lab, a<=b+rab

@@ -456,42 +456,46 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
                                                        int Tp, int D) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * Tp;
-    for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
-        const int d = idx >> 6, jj = idx & 63, j = j0 + jj;
-        float uv = 0.f, kv = 0.f, k2v = 0.f, v2v = 0.f;
+    // two tiles at a time (static LDS stays under 64 KB at D = 128): their loads are in flight together
+    constexpr int kTile = 64 * (128 + 2);
+    __shared__ E tiles[2 * kTile];
+    transpose_load<E, true>(v1 + base, u + base, tiles, j0, T, D);
+    transpose_load<E, false>(k1 + base, nullptr, tiles + kTile, j0, T, D);
+    __syncthreads();
+    transpose_store<E>(ut + tbase, tiles, j0, Tp, D);
+    transpose_store<E>(k1t + tbase, tiles + kTile, j0, Tp, D);
+    __syncthreads();
+    transpose_load<E, false>(k2 + base, nullptr, tiles, j0, T, D);
+    transpose_load<E, false>(v2 + base, nullptr, tiles + kTile, j0, T, D);
+    __syncthreads();
+    transpose_store<E>(k2t + tbase, tiles, j0, Tp, D);
+    transpose_store<E>(v2t + tbase, tiles + kTile, j0, Tp, D);
+    const float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int idx = threadIdx.x; idx < 64 * (D / 4); idx += 256) {
+        const int j = j0 + idx / (D / 4);
         if (j < T) {
-            const size_t off = base + (size_t)j * D + d;
-            uv = silu_f((float)v1[off]);
-            kv = (float)k1[off];
-            k2v = (float)k2[off];
-            v2v = (float)v2[off];
-        }
-        ut[tbase + (size_t)d * Tp + j] = (E)uv;
-        k1t[tbase + (size_t)d * Tp + j] = (E)kv;
-        k2t[tbase + (size_t)d * Tp + j] = (E)k2v;
-        v2t[tbase + (size_t)d * Tp + j] = (E)v2v;
-    }
-    for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
-        const int jj = idx / D, d = idx % D, j = j0 + jj;
-        if (j < T) {
-            const size_t off = base + (size_t)j * D + d;
-            u[off] = (E)silu_f((float)v1[off]);
-            zero_a[off] = 0.f;
-            zero_b[off] = 0.f;
-            zero_c[off] = 0.f;
-            zero_d[off] = 0.f;
-            if (zero_e) zero_e[off] = 0.f;
+            const size_t off = base + (size_t)j * D + (idx % (D / 4)) * 4;
+            *reinterpret_cast<float4*>(zero_a + off) = z4;
+            *reinterpret_cast<float4*>(zero_b + off) = z4;
+            *reinterpret_cast<float4*>(zero_c + off) = z4;
+            *reinterpret_cast<float4*>(zero_d + off) = z4;
+            if (zero_e) *reinterpret_cast<float4*>(zero_e + off) = z4;
         }
     }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int jj = wave; jj < 64; jj += 4) {
-        const int j = j0 + jj;
-        if (j >= T) break;
+    // Delta[j] = dO[j] . O[j]: the D / 8 lanes that hold a row's 16-byte pieces sit next to each other
+    typedef __attribute__((ext_vector_type(8))) E e8;
+    const int cpr = D / 8;
+    for (int idx = threadIdx.x; idx < 64 * cpr; idx += 256) {
+        const int j = j0 + idx / cpr, c = idx % cpr;
         float part = 0.f;
-        for (int d = lane; d < D; d += 64)
-            part += (float)o[base + (size_t)j * D + d] * (float)d_o[base + (size_t)j * D + d];
-        part = wave_sum(part);
-        if (lane == 0) delta[(size_t)bh * T + j] = part;
+        if (j < T) {
+            const size_t off = base + (size_t)j * D + c * 8;
+            const e8 a = *reinterpret_cast<const e8*>(o + off), b = *reinterpret_cast<const e8*>(d_o + off);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) part += (float)a[e] * (float)b[e];
+        }
+        for (int off = cpr >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if (c == 0 && j < T) delta[(size_t)bh * T + j] = part;
     }
 }
 

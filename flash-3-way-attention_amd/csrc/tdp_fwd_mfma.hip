@@ -766,14 +766,10 @@ template <typename E>
 __global__ __launch_bounds__(256) void silu_transpose_kernel(const E* __restrict__ v1, E* __restrict__ ut, int T,
                                                              int Tp, int D) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
-    const E* src = v1 + (size_t)bh * T * D;
-    E* dst = ut + (size_t)bh * D * Tp;
-    for (int idx = threadIdx.x; idx < D * 64; idx += 256) {
-        const int d = idx >> 6, jj = idx & 63, j = j0 + jj;
-        float v = 0.f;
-        if (j < T) v = silu_f((float)src[(size_t)j * D + d]);
-        dst[(size_t)d * Tp + j] = (E)v;
-    }
+    __shared__ E tile[64 * (128 + 2)];
+    transpose_load<E, true>(v1 + (size_t)bh * T * D, nullptr, tile, j0, T, D);
+    __syncthreads();
+    transpose_store<E>(ut + (size_t)bh * D * Tp, tile, j0, Tp, D);
 }
 
 template <int D, int NT, int WAVES, int JS>
