@@ -781,15 +781,20 @@ __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
     if (p.q) emit(p.q, p.qp1, p.qp2, false);
     if (p.d_o) emit(p.d_o, p.dop1, p.dop2, false);
     if (p.delta) {
-        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        for (int jj = wave; jj < 32; jj += 4) {
-            const int j = j0 + jj;
+        // Delta[j] = dO[j] . O[j]: the D / 8 lanes that hold a row's 16-byte pieces sit next to each other
+        constexpr int cpr = D / 8;
+        for (int idx = threadIdx.x; idx < 32 * cpr; idx += 256) {
+            const int j = j0 + idx / cpr, c = idx % cpr;
             float part = 0.f;
-            if (j < T)
-                for (int d = lane; d < D; d += 64)
-                    part += (float)p.o[base + (size_t)j * D + d] * (float)p.d_o[base + (size_t)j * D + d];
-            part = wave_sum(part);
-            if (lane == 0) {
+            if (j < T) {
+                const size_t off = base + (size_t)j * D + c * 8;
+                const v8 a = *reinterpret_cast<const v8*>(p.o + off), b = *reinterpret_cast<const v8*>(p.d_o + off);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) part += (float)a[e] * (float)b[e];
+            }
+#pragma unroll
+            for (int off = cpr >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+            if (c == 0) {
                 p.delta[(size_t)bh * Tp + j] = part;
                 p.lse2[(size_t)bh * Tp + j] = j < T ? p.lse[(size_t)bh * T + j] * kLog2e : 0.f;
             }
