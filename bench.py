@@ -27,8 +27,10 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by a plain 256 MiB copy (see the summaries under profiles/); not measured live
-TRAFFIC_FWD = 25.6e6        # 20.3 MiB fetched + 4.1 MiB written
-TRAFFIC_BWD_ROWS = 336e6     # average of the two launches: 33-75 MiB fetched, 264-268 MiB of fp32 atomics written
+TRAFFIC_FWD = 27.0e6        # 21.6 MiB fetched + 4.1 MiB written
+# average of the two launches: 264-268 MiB of fp32 atomics written; 50 MiB fetched by the second launch, and by the
+# first either 34 MiB or (most runs) ~500 MiB: its atomically accumulated row gradients then fall out of their XCD's L2
+TRAFFIC_BWD_ROWS = 565e6
 
 
 def triples(B, H, T, causal=True):
