@@ -440,7 +440,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 __syncthreads();
             }
             };
-            if constexpr (NT == 2 && !CAREFUL && !WIN) {
+            if constexpr (NT == 2 && !CAREFUL) {
                 // Stages whose 64 keys lie inside the causal bound of both tiles of this wave: a loop
                 // without branches on tile validity, so the accumulators stay in place (no copies
                 // at control-flow joins) and the wave itself overlaps matrix and vector work.  The
@@ -450,10 +450,26 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 // tile's value product in between that of the second.  K1 and U^T operands are
                 // read once for both tiles; the K1 operands of a block are fetched during the
                 // previous block of the same stage.
-                const int nfull = min(nst, (min(jmax[0], jmax[1]) + 1) / JS);
-                // MASKED (the stages that straddle the causal bound): a key past the bound of its tile
-                // starts its score at -3e4 (C operand of the first k-step), so its P is exactly 0.
-                // Element i of a lane is key jb + key_of(0, i) + 8 g.
+                // Interior stages [in_lo, in_hi): all 64 keys valid for every (q, k) of both tiles.
+                int in_lo = st_lo, in_hi = min(nst, (min(jmax[0], jmax[1]) + 1) / JS);
+                if constexpr (WIN) {
+                    if (banded) {
+                        const int k0 = kt * 32;
+                        bool rows_in = true;
+                        int lo_key = 0, hi_key = jend;
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) {
+                            rows_in = rows_in && (k0 + 31 <= jmax[t]) && (qrow[t] <= k0 + p.wb);
+                            lo_key = max(lo_key, max(qrow[t] - p.wa, k0 + 31 - p.lab));
+                            hi_key = min(hi_key, min(jmax[t], k0 + p.rab));
+                        }
+                        in_lo = min(st_hi + 1, max(st_lo, (lo_key + JS - 1) / JS));
+                        in_hi = rows_in ? min(st_hi + 1, max(in_lo, (hi_key + 1) / JS)) : in_lo;
+                    }
+                }
+                // MASKED (the stages that straddle the causal bound or an edge of the band): a key that is
+                // not valid for its (q, k) starts its score at -3e4 (C operand of the first k-step), so its P
+                // is exactly 0.  Element i of a lane is key jb + key_of(0, i) + 8 g.
                 auto fused = [&](auto masked_tag, const E* utp, const E* k1_next, v8 (&kn)[KS], int jb) {
                 constexpr bool MASKED = decltype(masked_tag)::value;
                 v8 ka[KS], ua[DT][2];
@@ -462,8 +478,14 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 f32x16 s0, s1;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    s0[i] = (MASKED && key_of(0, i) > jmax[0] - jb - 8 * g) ? -3.0e4f : 0.f;
-                    s1[i] = (MASKED && key_of(0, i) > jmax[1] - jb - 8 * g) ? -3.0e4f : 0.f;
+                    if constexpr (WIN) {
+                        const int j = jb + key_of(0, i) + 8 * g;
+                        s0[i] = (MASKED && (j < wlo[0] || j > whi[0])) ? -3.0e4f : 0.f;
+                        s1[i] = (MASKED && (j < wlo[1] || j > whi[1])) ? -3.0e4f : 0.f;
+                    } else {
+                        s0[i] = (MASKED && key_of(0, i) > jmax[0] - jb - 8 * g) ? -3.0e4f : 0.f;
+                        s1[i] = (MASKED && key_of(0, i) > jmax[1] - jb - 8 * g) ? -3.0e4f : 0.f;
+                    }
                 }
                 v8 pa0[2], pa1[2];
                 // quarter r of a tile's exp2 / pack / row-sum work: 4 exp2, 2 packs, 2 dot2
@@ -513,35 +535,25 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 for (int r = 0; r < 4; ++r) acc[1][r & 1] = M::mma(pa1[r >> 1], ua[r & 1][r >> 1], acc[1][r & 1]);
                 __builtin_amdgcn_sched_barrier(0);
                 };
-                for (; st < nfull; ++st, ++gstage) {
+                auto stage_nt2 = [&](auto masked_tag) {
+                    constexpr bool MASKED = decltype(masked_tag)::value;
                     const int sb = gstage & 1;
-                    issue_stage(st + 1 < nst ? st + 1 : 0);
-                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
+                    issue_stage(st < st_hi ? st + 1 : st_next);
+                    if (st == st_lo && kt + 1 < nkt) issue_ktile(kt + 1);
                     const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
                     const E* utp = sUT + (sb * D + n) * LDU + g * 8;
                     v8 kn[KS];
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
                     static_assert(JS == 64 || NT != 2, "two blocks per stage");
-                    fused(std::false_type{}, utp, k1p + 32 * LDK, kn, 0);
-                    fused(std::false_type{}, utp + 32, nullptr, kn, 0);
+                    fused(masked_tag, utp, k1p + 32 * LDK, kn, st * JS);
+                    if (!MASKED || st * JS + 32 <= jend) fused(masked_tag, utp + 32, nullptr, kn, st * JS + 32);
                     commit_stage(sb ^ 1);
                     __syncthreads();
-                }
-                for (; st < nst; ++st, ++gstage) {  // the one or two stages on the diagonal
-                    const int sb = gstage & 1;
-                    issue_stage(st + 1 < nst ? st + 1 : 0);
-                    if (st == 0 && kt + 1 < nkt) issue_ktile(kt + 1);
-                    const E* k1p = sK1 + (sb * JS + krow_off) * LDK + g * 8;
-                    const E* utp = sUT + (sb * D + n) * LDU + g * 8;
-                    v8 kn[KS];
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) kn[ks] = *reinterpret_cast<const v8*>(k1p + ks * 16);
-                    fused(std::true_type{}, utp, k1p + 32 * LDK, kn, st * JS);
-                    if (st * JS + 32 <= jend) fused(std::true_type{}, utp + 32, nullptr, kn, st * JS + 32);
-                    commit_stage(sb ^ 1);
-                    __syncthreads();
-                }
+                };
+                for (; st < in_lo; ++st, ++gstage) stage_nt2(std::true_type{});   // leading edge of the band
+                for (; st < in_hi; ++st, ++gstage) stage_nt2(std::false_type{});
+                for (; st <= st_hi; ++st, ++gstage) stage_nt2(std::true_type{});  // the diagonal / trailing edge
             }
             if constexpr (NT == 1 && !CAREFUL) {
                 // The same for one tile per wave (D = 128: two tiles do not fit the register file).
@@ -790,9 +802,8 @@ constexpr int kTpad = 128;  // U^T rows are padded to a multiple of the largest 
 // (4 under a windowed mask, whose k-tiles see only a few steps of j each).
 constexpr int kFwdSplitTarget = 768, kAutoFwdSplits = 4, kMaxFwdSplits = 8;
 
-// queries per workgroup of the instantiation mfma_tdp_fwd() picks: D = 64 without windows runs two queries per
-// wave, everything else one
-static int fwd_tile_queries(int D, int windowed) { return (D == 64 && !windowed) ? 16 : 8; }
+// queries per workgroup of the instantiation mfma_tdp_fwd() picks: D = 64 runs two queries per wave, the others one
+static int fwd_tile_queries(int D, int /*windowed*/) { return D == 64 ? 16 : 8; }
 
 static size_t ut_bytes(int BH, int T, int D) {
     const size_t Tp = (size_t)(T + kTpad - 1) / kTpad * kTpad;
@@ -912,11 +923,11 @@ hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
         // the stages on its edges the general one
         if (a.is_bf16) {
             if (a.D == 32) return launch<__bf16, 32, 1, 8, 2, 64, true>(a, st);
-            if (a.D == 64) return launch<__bf16, 64, 1, 8, 2, 64, true>(a, st);
+            if (a.D == 64) return launch<__bf16, 64, 2, 8, 2, 64, true>(a, st);
             if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64, true>(a, st);
         } else {
             if (a.D == 32) return launch<_Float16, 32, 1, 8, 2, 64, true>(a, st);
-            if (a.D == 64) return launch<_Float16, 64, 1, 8, 2, 64, true>(a, st);
+            if (a.D == 64) return launch<_Float16, 64, 2, 8, 2, 64, true>(a, st);
             if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64, true>(a, st);
         }
         return hipErrorInvalidValue;
