@@ -661,15 +661,12 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
             bool bad = false;
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
+                // every P is at most its row sum, so a row sum inside this range keeps the value accumulators
+                // (P times SiLU(V1), a handful of terms) finite as well
                 const float lk = lsum[t] + __shfl_xor(lsum[t], 32, 64);
-                float mag = 0.f;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) mag += fabsf(acc[t][dt][i]);
                 bool kval = (kt * 32 + n) <= jmax[t];
                 if constexpr (WIN) kval = whi[t] >= 0;
-                bad |= (kval && !(lk > 1e-30f && lk < 1e30f)) || !(mag < 1e30f);
+                bad |= kval && !(lk > 1e-30f && lk < 1e25f);
             }
             if (__any(bad) && lane == 0) *sFlag = 1;
             __syncthreads();

@@ -231,6 +231,24 @@ def test_mfma_forward_large_logits():
     assert (err > 5e-2).float().mean() < 0.01 and err.max() < 0.5, (err.max(), (err > 5e-2).float().mean())
 
 
+def test_mfma_forward_large_values_and_logits():
+    """Values in the thousands together with scores spanning hundreds: the fast sweep judges its exponent range
+    by the row sums alone (every P is at most its row sum), so the value accumulators must stay finite whenever
+    it is accepted, and the repeat sweep must take over where it is not."""
+    inputs = orc.make_inputs(1, 2, 160, 64, torch.bfloat16, seed=31)
+    inputs[1] = (inputs[1].float() * 5).bfloat16()
+    inputs[2] = (inputs[2].float() * 5).bfloat16()
+    inputs[3] = (inputs[3].float() * 2048).bfloat16()
+    inputs[4] = (inputs[4].float() * 64).bfloat16()
+    z, _, _ = util.oracle_tdp(inputs, 1 / 8, True)
+    for flags in (FORCE_MFMA,):
+        out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=flags)
+        assert torch.isfinite(out).all()
+        scale = z.abs().max()
+        err = (out - z).abs() / scale
+        assert (err > 2e-2).float().mean() < 0.01 and err.max() < 0.2, (err.max(), (err > 2e-2).float().mean())
+
+
 def test_mfma_and_generic_agree_bf16():
     inputs = orc.make_inputs(1, 2, 192, 64, torch.bfloat16, seed=23)
     a, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
