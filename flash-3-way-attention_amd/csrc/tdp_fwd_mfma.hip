@@ -233,7 +233,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
         const int r = idx / D, d = idx % D;
         sQ[r * LDQ + d] = (float)Q[(size_t)min(q0 + r, T - 1) * D + d] * p.scale_log2;
     }
-    if (tid == 0) *sFlag = 0;
+    if (tid < 2) sFlag[tid] = 0;  // two flags, used by alternate k-tiles
     issue_ktile(kt_lo);
     issue_stage(first_stage(kt_lo));
     commit_ktile(0);
@@ -668,12 +668,14 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 if constexpr (WIN) kval = whi[t] >= 0;
                 bad |= kval && !(lk > 1e-30f && lk < 1e25f);
             }
-            if (__any(bad) && lane == 0) *sFlag = 1;
+            // One barrier per k-tile: this k-tile's flag is read after it; the other flag was read by every
+            // wave before it arrived here, is cleared now, and is next written after the barriers of the
+            // following k-tile's sweep.
+            if (__any(bad) && lane == 0) sFlag[kb] = 1;
             __syncthreads();
-            const bool redo = *sFlag != 0;
-            __syncthreads();
+            const bool redo = sFlag[kb] != 0;
+            if (tid == 0) sFlag[kb ^ 1] = 0;
             if (redo) {
-                if (tid == 0) *sFlag = 0;
                 if constexpr (WIN) {
                     if (st_next != st_lo) {  // the stage fetched ahead belongs to the next k-tile: fetch this one's
                         issue_stage(st_lo);
