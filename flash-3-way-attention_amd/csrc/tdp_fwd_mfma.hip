@@ -672,6 +672,10 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
             // wave before it arrived here, is cleared now, and is next written after the barriers of the
             // following k-tile's sweep.
             if (__any(bad) && lane == 0) sFlag[kb] = 1;
+            // The next k-tile's K2 / V2 rows go to LDS here too (their buffer was last read in the previous
+            // k-tile, and every wave has crossed a stage barrier of this one since), so the same barrier
+            // publishes them and the k-tile needs none at its end.
+            if (kt + 1 < nkt) commit_ktile(kb ^ 1);
             __syncthreads();
             const bool redo = sFlag[kb] != 0;
             if (tid == 0) sFlag[kb ^ 1] = 0;
@@ -719,8 +723,6 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
             }
         }
 
-        if (kt + 1 < nkt) commit_ktile(kb ^ 1);
-        __syncthreads();
     }
 
     // ---- epilogue ---------------------------------------------------------------------------
