@@ -28,9 +28,10 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by a plain 256 MiB copy (see the summaries under profiles/); not measured live
 TRAFFIC_FWD = 27.0e6        # 21.6 MiB fetched + 4.1 MiB written
-# average of the two launches: 264-268 MiB of fp32 atomics written; 50 MiB fetched by the second launch, and by the
-# first either 34 MiB or (most runs) ~500 MiB: its atomically accumulated row gradients then fall out of their XCD's L2
-TRAFFIC_BWD_ROWS = 565e6
+# average of the two launches: 264-268 MiB of fp32 atomics written and 34-90 MiB fetched; in some dispatches (most of
+# them on some boxes) the first launch fetches ~500 MiB instead: its atomically accumulated row gradients then fall
+# out of their XCD's L2 (same duration either way)
+TRAFFIC_BWD_ROWS = 350e6
 
 
 def triples(B, H, T, causal=True):
