@@ -94,13 +94,16 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][4 tensors: K1, U, K1^T, U^T][TILE]
     E* sKr = sStage + NBUF * 4 * TILE;       // [2][8][D]  K2 rows of a round (one per wave), dense
     E* sVr = sKr + 2 * 8 * D;                // [2][8][D]  V2 rows
-    E* sQb = sVr + 2 * 8 * D;                // [BQ][LDK]  Q tile (operand build)
-    E* sOb = sQb + BQ * LDK;                 // [BQ][LDK]  dO tile
+    // Q * alpha*log2(e) and dO as fp32 (operand build: one conversion and one multiply per product, and S is
+    // rounded exactly as the forward rounded it)
+    constexpr int LDQ = D + 4;
+    float* sQb = reinterpret_cast<float*>(sVr + 2 * 8 * D);  // [BQ][LDQ]
+    float* sOb = sQb + BQ * LDQ;                              // [BQ][LDQ]
     // dQ / alpha of the tile, summed over rounds: one slice per pair of waves, element (dt, i) of a
     // lane at [((dt * 4 + i / 4) * 64 + lane) * 4 + i % 4] (the accumulator layout, 16 bytes per access)
-    float* sDQ = reinterpret_cast<float*>(sOb + BQ * LDK) + (wave_of(threadIdx.x) >> 1) * (BQ * D);
+    float* sDQ = sOb + BQ * LDQ + (wave_of(threadIdx.x) >> 1) * (BQ * D);
     // Q and dO once more, in accumulator layout for the round epilogue: [dt][lane][i] = X[c_row(lane / 32, i)][32 dt + lane % 32]
-    E* sQe = reinterpret_cast<E*>(reinterpret_cast<float*>(sOb + BQ * LDK) + (NW / 2) * (BQ * D));
+    E* sQe = reinterpret_cast<E*>(sOb + BQ * LDQ + (NW / 2) * (BQ * D));
     E* sOe = sQe + DT * 64 * 16;
 
     const int groups = (p.BH + 7) / 8;
@@ -184,8 +187,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         const int r = idx / D, d = idx % D;
         const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
         const E qv = p.q[off], ov = p.d_o[off];
-        sQb[r * LDK + d] = qv;
-        sOb[r * LDK + d] = ov;
+        sQb[r * LDQ + d] = (float)qv * scale_log2;
+        sOb[r * LDQ + d] = (float)ov;
     }
     for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
         const int i = idx & 15, ln = (idx >> 4) & 63, dt = idx >> 10;
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         sOe[idx] = p.d_o[off];
     }
     if constexpr (WITH_DQ) {
-        float* all = reinterpret_cast<float*>(sOb + BQ * LDK);
+        float* all = sOb + BQ * LDQ;
         for (int idx = tid; idx < (NW / 2) * BQ * D; idx += NTH) all[idx] = 0.f;
     }
     issue_round(m_lo, m_lo & 1);
@@ -249,14 +252,17 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
             const int off = ks * 16 + g * 8;
             const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * 8 + wave) * D + off);
             const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * 8 + wave) * D + off);
-            const v8 qv = *reinterpret_cast<const v8*>(sQb + n * LDK + off);
-            const v8 dv = *reinterpret_cast<const v8*>(sOb + n * LDK + off);
+            const float4 qa = *reinterpret_cast<const float4*>(sQb + n * LDQ + off);
+            const float4 qb = *reinterpret_cast<const float4*>(sQb + n * LDQ + off + 4);
+            const float4 da = *reinterpret_cast<const float4*>(sOb + n * LDQ + off);
+            const float4 db = *reinterpret_cast<const float4*>(sOb + n * LDQ + off + 4);
+            const float qv[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+            const float dv[8] = {da.x, da.y, da.z, da.w, db.x, db.y, db.z, db.w};
             v8 a, b;
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
-                const v2 pa = M::pack((float)kv[e] * (float)qv[e] * scale_log2,
-                                      (float)kv[e + 1] * (float)qv[e + 1] * scale_log2);
-                const v2 pb = M::pack((float)vv[e] * (float)dv[e], (float)vv[e + 1] * (float)dv[e + 1]);
+                const v2 pa = M::pack((float)kv[e] * qv[e], (float)kv[e + 1] * qv[e + 1]);
+                const v2 pb = M::pack((float)vv[e] * dv[e], (float)vv[e + 1] * dv[e + 1]);
                 a[e] = pa[0]; a[e + 1] = pa[1];
                 b[e] = pb[0]; b[e + 1] = pb[1];
             }
@@ -421,7 +427,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     if constexpr (WITH_DQ) {
         // ---- dQ: sum the pairs' slices; thread (wave, lane) owns accumulator registers 4*(wave%4) .. +3
         // of d-tile wave/4, i.e. four consecutive query rows of column d
-        const float* all = reinterpret_cast<const float*>(sOb + BQ * LDK);
+        const float* all = sOb + BQ * LDQ;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int sl = 0; sl < NW / 2; ++sl) {
@@ -615,8 +621,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
             nthreads = 256;
         }
     } else {
-        smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * 64 + 2 * 32 * (64 + 8) + 2 * (64 / 32) * 64 * 16) +
-               4 * (size_t)(4 * 32 * 64);
+        smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * 64 + 2 * (64 / 32) * 64 * 16) +
+               4 * (size_t)(2 * 32 * (64 + 4) + 4 * 32 * 64);
         kern_dq = tdp_bwd_rows_kernel<E, 64, true>;
         kern_nodq = tdp_bwd_rows_kernel<E, 64, false>;
     }
