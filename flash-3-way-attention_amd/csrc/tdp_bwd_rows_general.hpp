@@ -61,7 +61,7 @@ constexpr int bwdg_round_rows(int d, int nw) { return nw > 512 / d ? nw : 512 / 
 constexpr size_t bwdg_smem(int d, int nw, int ncol, bool with_dq) {
     return 3 * (size_t)bwdg_stage_bytes(d, ncol)               // stage buffers
            + 2 * (2 * bwdg_round_rows(d, nw) * d * 2)           // K2 / V2 rows of two rounds
-           + 2 * (32 * (d + 8) * 2)                             // Q and dO tiles
+           + (d == 64 ? 2 * (32 * (d + 4) * 4) : 2 * (32 * (d + 8) * 2))  // Q and dO tiles (D = 64: fp32)
            + (with_dq ? (nw / 2) * (32 * ncol * 4) : 0)         // dQ slices (one per pair of waves)
            + (ncol == 64 ? 2 * (2 * 64 * 16 * 2) : 0);          // Q and dO in accumulator layout (NCOL = 64)
 }
@@ -90,9 +90,16 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows 4096 | U rows 4096 | K1^T 2048 | U^T 2048]
     E* sKr = sStage + NBUF * STAGE;          // [2][RR][D]
     E* sVr = sKr + 2 * RR * D;
-    E* sQb = sVr + 2 * RR * D;               // [BQ][LDK]
-    E* sOb = sQb + BQ * LDK;
-    float* sDQall = reinterpret_cast<float*>(sOb + BQ * LDK);  // [NW/2][BQ * DH], accumulator layout (WITH_DQ)
+    // Q and dO tiles for the operand build.  D = 64 (where LDS has the room): Q * alpha*log2(e) and dO in fp32, so a
+    // product is one conversion and one multiply and S is rounded exactly as the forward rounded it.
+    constexpr bool QF = D == 64;
+    constexpr int LDQ = D + 4, QT_BYTES = QF ? BQ * LDQ * 4 : BQ * LDK * 2;
+    char* qtiles = reinterpret_cast<char*>(sVr + 2 * RR * D);
+    E* sQb = reinterpret_cast<E*>(qtiles);              // [BQ][LDK]   (!QF)
+    E* sOb = reinterpret_cast<E*>(qtiles + QT_BYTES);
+    [[maybe_unused]] float* sQf = reinterpret_cast<float*>(qtiles);  // [BQ][LDQ]   (QF)
+    [[maybe_unused]] float* sOf = reinterpret_cast<float*>(qtiles + QT_BYTES);
+    float* sDQall = reinterpret_cast<float*>(qtiles + 2 * QT_BYTES);  // [NW/2][BQ * DH], accumulator layout (WITH_DQ)
     float* sDQ = sDQall + (wave_of(threadIdx.x) >> 1) * (BQ * DH);
     E* sQe = reinterpret_cast<E*>(sDQall + (WITH_DQ ? (NW / 2) * (BQ * DH) : 0));  // [DT][64][16] (EPI_TILES)
     E* sOe = sQe + DT * 64 * 16;
@@ -198,8 +205,13 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     for (int idx = tid; idx < BQ * D; idx += NTH) {
         const int r = idx / D, d = idx % D;
         const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
-        sQb[r * LDK + d] = p.q[off];
-        sOb[r * LDK + d] = p.d_o[off];
+        if constexpr (QF) {
+            sQf[r * LDQ + d] = (float)p.q[off] * scale_log2;
+            sOf[r * LDQ + d] = (float)p.d_o[off];
+        } else {
+            sQb[r * LDK + d] = p.q[off];
+            sOb[r * LDK + d] = p.d_o[off];
+        }
     }
     if constexpr (EPI_TILES) {
         for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
@@ -277,14 +289,28 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                     const int off = ks * 16 + g * 8;
                     const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * RR + wave) * D + off);
                     const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * RR + wave) * D + off);
-                    const v8 qv = *reinterpret_cast<const v8*>(sQb + n * LDK + off);
-                    const v8 dv = *reinterpret_cast<const v8*>(sOb + n * LDK + off);
+                    float qf[8], df[8];
+                    if constexpr (QF) {
+                        const float4 qa = *reinterpret_cast<const float4*>(sQf + n * LDQ + off);
+                        const float4 qb = *reinterpret_cast<const float4*>(sQf + n * LDQ + off + 4);
+                        const float4 da = *reinterpret_cast<const float4*>(sOf + n * LDQ + off);
+                        const float4 db = *reinterpret_cast<const float4*>(sOf + n * LDQ + off + 4);
+                        qf[0] = qa.x; qf[1] = qa.y; qf[2] = qa.z; qf[3] = qa.w; qf[4] = qb.x; qf[5] = qb.y; qf[6] = qb.z; qf[7] = qb.w;
+                        df[0] = da.x; df[1] = da.y; df[2] = da.z; df[3] = da.w; df[4] = db.x; df[5] = db.y; df[6] = db.z; df[7] = db.w;
+                    } else {
+                        const v8 qv = *reinterpret_cast<const v8*>(sQb + n * LDK + off);
+                        const v8 dv = *reinterpret_cast<const v8*>(sOb + n * LDK + off);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            qf[e] = (float)qv[e] * scale_log2;
+                            df[e] = (float)dv[e];
+                        }
+                    }
                     v8 a, b;
 #pragma unroll
                     for (int e = 0; e < 8; e += 2) {
-                        const v2 pa = M::pack((float)kv[e] * (float)qv[e] * scale_log2,
-                                              (float)kv[e + 1] * (float)qv[e + 1] * scale_log2);
-                        const v2 pb = M::pack((float)vv[e] * (float)dv[e], (float)vv[e + 1] * (float)dv[e + 1]);
+                        const v2 pa = M::pack((float)kv[e] * qf[e], (float)kv[e + 1] * qf[e + 1]);
+                        const v2 pb = M::pack((float)vv[e] * df[e], (float)vv[e + 1] * df[e + 1]);
                         a[e] = pa[0]; a[e + 1] = pa[1];
                         b[e] = pb[0]; b[e + 1] = pb[1];
                     }
