@@ -61,7 +61,7 @@ constexpr int bwdg_round_rows(int d, int nw) { return nw > 512 / d ? nw : 512 / 
 constexpr size_t bwdg_smem(int d, int nw, int ncol, bool with_dq) {
     return 3 * (size_t)bwdg_stage_bytes(d, ncol)               // stage buffers
            + 2 * (2 * bwdg_round_rows(d, nw) * d * 2)           // K2 / V2 rows of two rounds
-           + (d == 64 ? 2 * (32 * (d + 4) * 4) : 2 * (32 * (d + 8) * 2))  // Q and dO tiles (D = 64: fp32)
+           + (ncol == 64 ? 2 * (32 * (d + 4) * 4) : 2 * (32 * (d + 8) * 2))  // Q and dO tiles (64 columns: fp32)
            + (with_dq ? (nw / 2) * (32 * ncol * 4) : 0)         // dQ slices (one per pair of waves)
            + (ncol == 64 ? 2 * (2 * 64 * 16 * 2) : 0);          // Q and dO in accumulator layout (NCOL = 64)
 }
@@ -90,9 +90,9 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows 4096 | U rows 4096 | K1^T 2048 | U^T 2048]
     E* sKr = sStage + NBUF * STAGE;          // [2][RR][D]
     E* sVr = sKr + 2 * RR * D;
-    // Q and dO tiles for the operand build.  D = 64 (where LDS has the room): Q * alpha*log2(e) and dO in fp32, so a
-    // product is one conversion and one multiply and S is rounded exactly as the forward rounded it.
-    constexpr bool QF = D == 64;
+    // Q and dO tiles for the operand build.  64-column shapes (where LDS has the room): Q * alpha*log2(e) and dO in
+    // fp32, so a product is one conversion and one multiply and S is rounded exactly as the forward rounded it.
+    constexpr bool QF = NCOL == 64;
     constexpr int LDQ = D + 4, QT_BYTES = QF ? BQ * LDQ * 4 : BQ * LDK * 2;
     char* qtiles = reinterpret_cast<char*>(sVr + 2 * RR * D);
     E* sQb = reinterpret_cast<E*>(qtiles);              // [BQ][LDK]   (!QF)
