@@ -334,13 +334,16 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             }
 
             // row operands in two batches of four k-steps: the second is read under the first products
-            v8 ak[KS], au[KS];
+            // one batch of row operands at a time: the second batch (D = 128) reuses the registers of the first
+            // once its products have been issued
+            constexpr int KB = KS < 4 ? KS : 4;
+            v8 ak[KB], au[KB];
             auto load_rows = [&](int first) {
 #pragma unroll
                 for (int ks = first; ks < min(first + 4, KS); ++ks) {
                     const int roff = ((ks >> 2) * 32 + krow_off) * RW + ((((ks & 3) * 2 + g) ^ fperm) * 8);
-                    ak[ks] = *reinterpret_cast<const v8*>(sK1 + roff);
-                    au[ks] = *reinterpret_cast<const v8*>(sU + roff);
+                    ak[ks & 3] = *reinterpret_cast<const v8*>(sK1 + roff);
+                    au[ks & 3] = *reinterpret_cast<const v8*>(sU + roff);
                 }
             };
             load_rows(0);
@@ -367,15 +370,22 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                 s = M::mma(a_ones, b_lse, c);
             }
             __builtin_amdgcn_sched_barrier(0);
-            load_rows(4);
-            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
+            for (int ks = 0; ks < KB; ++ks) {
                 s = M::mma(ak[ks], bq[ks], s);
                 dp = M::mma(au[ks], bg[ks], dp);
-                if (ks == 3) __builtin_amdgcn_sched_barrier(0);
             }
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (KS > 4) {
+                load_rows(4);  // lands under the products just issued
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 4; ks < KS; ++ks) {
+                    s = M::mma(ak[ks & 3], bq[ks], s);
+                    dp = M::mma(au[ks & 3], bg[ks], dp);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
             v8 bt[DT][2], bk[DT][2];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
