@@ -601,10 +601,11 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         kern_nodq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), false, 8, 64, true>;
         col_parts = D / 64;
     } else if constexpr (D == 128) {
-        // One wave per SIMD with all 128 columns is ~10 % faster once the grid fills the chip several times
-        // over; below that the smaller workgroups of the two-waves-per-SIMD shape balance better.
+        // Two waves per SIMD, 64 gradient columns per workgroup (S and dP computed by both column halves) is the
+        // faster shape at every grid size measured, now that it fits the register file without scratch memory;
+        // the one-wave-per-SIMD shape with all 128 columns stays selectable.
         // TRITT_BWD128_VARIANT=w8 / w4 overrides the choice (read at every call).
-        bool w8 = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32) < 1024;
+        bool w8 = true;
         if (const char* v = getenv("TRITT_BWD128_VARIANT")) {
             if (strcmp(v, "w8") == 0) w8 = true;
             if (strcmp(v, "w4") == 0) w8 = false;
