@@ -34,6 +34,9 @@ int check_common(int B, int H, int T, int D, int dtype) {
     return TRITT_OK;
 }
 
+// An empty batch, head set or sequence: nothing to compute, no pointer is touched.
+bool empty_problem(int B, int H, int T) { return B >= 0 && H >= 0 && T >= 0 && (B == 0 || H == 0 || T == 0); }
+
 // ---------------------------------------------------------------- elementwise helpers
 template <typename T, bool SILU>
 __global__ __launch_bounds__(256) void to_f32_kernel(const T* __restrict__ src, float* __restrict__ dst, size_t n) {
@@ -332,6 +335,7 @@ size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int 
 int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, void* o, float* lse,
                   int B, int H, int T, int D, int dtype, float alpha, int causal, int k1_window, int k2_window,
                   int kk_left, int kk_right, void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
@@ -370,6 +374,7 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
                   const float* lse, const void* d_o, void* dq, void* dk1, void* dk2, void* dv1, void* dv2, int B, int H,
                   int T, int D, int dtype, float alpha, int causal, int k1_window, int k2_window, int kk_left,
                   int kk_right, void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
@@ -408,6 +413,7 @@ size_t tritt_dps_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, unsi
 int tritt_dps_fwd(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, void* o, float* lse,
                   int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff, void* workspace,
                   size_t workspace_bytes, unsigned flags, void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
@@ -443,6 +449,7 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
                   const float* lse, const void* d_o, void* dq, void* dk1, void* dk2, void* dv1, void* dv2, int B, int H,
                   int T, int D, int dtype, float alpha, int causal, int k_diff, void* workspace, size_t workspace_bytes,
                   unsigned flags, void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;

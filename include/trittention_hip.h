@@ -16,7 +16,9 @@
  * these calls: scratch memory is passed in by the caller (`workspace`), its
  * required size is returned by the matching *_workspace_bytes function.
  * Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
- * null stream) and the calls do not synchronise.
+ * null stream) and the calls do not synchronise.  A problem with B, H or T
+ * equal to 0 is a successful no-op: nothing is launched, no pointer is read
+ * (they may be NULL) and its workspace size is 0.
  */
 #ifndef TRITTENTION_HIP_H
 #define TRITTENTION_HIP_H
@@ -32,7 +34,7 @@ enum { TRITT_F32 = 0, TRITT_BF16 = 1, TRITT_F16 = 2 };
 
 enum {
     TRITT_OK = 0,
-    TRITT_ERR_INVALID = -1,     /* null or misaligned pointer, non-positive size, bad dtype */
+    TRITT_ERR_INVALID = -1,     /* null or misaligned pointer, negative size, bad dtype */
     TRITT_ERR_HEAD_DIM = -2,    /* D not one of 16, 32, 64, 128                            */
     TRITT_ERR_WORKSPACE = -3,   /* workspace missing or smaller than *_workspace_bytes     */
     TRITT_ERR_UNSUPPORTED = -4  /* requested implementation cannot run this configuration */

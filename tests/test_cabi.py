@@ -50,7 +50,7 @@ def test_argument_rejection_happens_before_any_launch():
     one = ctypes.c_void_p(256)  # never dereferenced: rejected first
     args7 = [one] * 7
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 24, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -2
-    assert lib.tritt_tdp_fwd(*args7, 0, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
+    assert lib.tritt_tdp_fwd(*args7, -1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 7, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
     assert lib.tritt_tdp_fwd(null, *args7[1:], 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, -1, 16, 16, 16, null, 0, 0, null) == -1
@@ -61,6 +61,22 @@ def test_argument_rejection_happens_before_any_launch():
     assert lib.tritt_tdp_fwd(odd, *args7[1:], 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
     assert lib.tritt_dps_fwd(*args7[:3], odd, *args7[4:], 1, 1, 16, 32, 0, 0.1, 1, 16, null, 0, 0, null) == -1
     assert b"misaligned" in lib.tritt_status_string(-1)
+
+
+def test_empty_problem_is_a_successful_no_op():
+    """B, H or T equal to 0: nothing is launched, null pointers are accepted, the workspace size is 0; the head
+    dimension and the dtype are still checked."""
+    lib = _lib.lib()
+    null = ctypes.c_void_p(0)
+    for B, H, T in [(0, 2, 16), (2, 0, 16), (2, 2, 0)]:
+        assert lib.tritt_tdp_fwd_workspace_bytes(B, H, T, 32, 0, 1, 16, 16, 16, 16, 0) == 0
+        assert lib.tritt_tdp_fwd(*[null] * 7, B, H, T, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == 0
+        assert lib.tritt_tdp_bwd(*[null] * 13, B, H, T, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == 0
+        assert lib.tritt_dps_fwd(*[null] * 7, B, H, T, 32, 0, 0.1, 1, 16, null, 0, 0, null) == 0
+        assert lib.tritt_dps_bwd(*[null] * 13, B, H, T, 32, 0, 0.1, 1, 16, null, 0, 0, null) == 0
+    assert lib.tritt_tdp_fwd(*[null] * 7, 0, 2, 16, 24, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -2
+    assert lib.tritt_dps_fwd(*[null] * 7, 0, 2, 16, 32, 9, 0.1, 1, 16, null, 0, 0, null) == -1
+    assert lib.tritt_tdp_fwd(*[null] * 7, 0, -2, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
 
 
 def test_python_host_validation_matches_reference_errors():

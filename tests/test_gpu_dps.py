@@ -168,6 +168,14 @@ def test_rejects_mismatched_shapes():
         TrittentionTriton()(q, k1, k2, v1, v2[:, :, :16, :].contiguous())
 
 
+@pytest.mark.parametrize("shape", [(0, 2, 16, 32), (2, 0, 16, 32), (2, 2, 0, 32)])
+def test_empty_inputs_give_empty_results(shape):
+    inputs = [torch.zeros(shape, dtype=torch.bfloat16) for _ in range(6)]
+    out, m, grads = util.run_dps(inputs, 0.125, True, 16)
+    assert out.shape == shape and m.shape == shape[:3]
+    assert all(g.shape == shape for g in grads)
+
+
 # ------------------------------------------------- full-size properties (config 4: B=4 H=8 T=1024 D=64 bf16)
 def test_config4_heads_are_independent_bitwise():
     """Every output element has one owner (no atomics): permuting the (batch, head) slices permutes

@@ -494,6 +494,16 @@ def test_long_sequences_under_windows(T, D, windows):
             util.assert_mostly_close(f"{name}[{h}]", a[0, h], b, **LOWP)
 
 
+@pytest.mark.parametrize("shape", [(0, 2, 16, 32), (2, 0, 16, 32), (2, 2, 0, 64)])
+def test_empty_inputs_give_empty_results(shape):
+    inputs = [torch.zeros(shape, dtype=torch.bfloat16) for _ in range(6)]
+    out, grads = util.run_tdp(inputs, 0.125, True, (None,) * 4)
+    assert out.shape == shape
+    assert all(g.shape == shape for g in grads)
+    out, _ = util.run_tdp(inputs, 0.125, True, (4, 4, 2, 2), backward=False)
+    assert out.shape == shape
+
+
 @pytest.mark.parametrize("shape", [(2, 4, 256, 64, (None,) * 4), (1, 3, 200, 128, (None,) * 4), (1, 2, 300, 64, (64, 64, 16, 16))])
 def test_forward_and_backward_replay_from_a_hip_graph(shape):
     """The library only launches kernels on the stream it is given (no allocation, copy, memset or
