@@ -31,6 +31,7 @@ int check_common(int B, int H, int T, int D, int dtype) {
     if (dtype != TRITT_F32 && dtype != TRITT_BF16 && dtype != TRITT_F16) return TRITT_ERR_INVALID;
     if (D != 16 && D != 32 && D != 64 && D != 128) return TRITT_ERR_HEAD_DIM;
     if ((long long)B * H > 65535) return TRITT_ERR_INVALID;
+    if ((long long)B * H * T > 0x7fffffffLL) return TRITT_ERR_INVALID;  // row indices are 32-bit; element offsets are not
     return TRITT_OK;
 }
 

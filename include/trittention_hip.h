@@ -34,7 +34,8 @@ enum { TRITT_F32 = 0, TRITT_BF16 = 1, TRITT_F16 = 2 };
 
 enum {
     TRITT_OK = 0,
-    TRITT_ERR_INVALID = -1,     /* null or misaligned pointer, negative size, bad dtype */
+    TRITT_ERR_INVALID = -1,     /* null or misaligned pointer, negative size, bad dtype,
+                                   B*H above 65535 or B*H*T above 2^31-1                    */
     TRITT_ERR_HEAD_DIM = -2,    /* D not one of 16, 32, 64, 128                            */
     TRITT_ERR_WORKSPACE = -3,   /* workspace missing or smaller than *_workspace_bytes     */
     TRITT_ERR_UNSUPPORTED = -4  /* requested implementation cannot run this configuration */

@@ -52,6 +52,8 @@ def test_argument_rejection_happens_before_any_launch():
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 24, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -2
     assert lib.tritt_tdp_fwd(*args7, -1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 7, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
+    assert lib.tritt_tdp_fwd(*args7, 256, 256, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1  # B*H
+    assert lib.tritt_dps_fwd(*args7, 128, 256, 1 << 16, 32, 1, 0.1, 1, 16, null, 0, 0, null) == -1  # B*H*T
     assert lib.tritt_tdp_fwd(null, *args7[1:], 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 0, null) == -1
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, -1, 16, 16, 16, null, 0, 0, null) == -1
     assert lib.tritt_tdp_fwd(*args7, 1, 1, 16, 32, 0, 0.1, 1, 16, 16, 16, 16, null, 0, 1, null) == -3  # no workspace

@@ -168,6 +168,12 @@ def test_rejects_mismatched_shapes():
         TrittentionTriton()(q, k1, k2, v1, v2[:, :, :16, :].contiguous())
 
 
+def test_tensors_of_more_than_2_31_elements():
+    """Element offsets beyond 32 bits: B*H = 52500 heads of T=640, D=64 (4.3 GB per bf16 tensor)."""
+    print("case beyond 2^31 elements (7, 7500, 640, 64)", flush=True)
+    util.check_offsets_beyond_32_bits("dps", 7, 7500, 640, 64)
+
+
 @pytest.mark.parametrize("shape", [(0, 2, 16, 32), (2, 0, 16, 32), (2, 2, 0, 32)])
 def test_empty_inputs_give_empty_results(shape):
     inputs = [torch.zeros(shape, dtype=torch.bfloat16) for _ in range(6)]

@@ -494,6 +494,15 @@ def test_long_sequences_under_windows(T, D, windows):
             util.assert_mostly_close(f"{name}[{h}]", a[0, h], b, **LOWP)
 
 
+@pytest.mark.parametrize("B,H,T,D,windows", [(7, 7500, 640, 64, (None,) * 4), (5, 8000, 512, 128, (64, 64, 32, 32))])
+def test_tensors_of_more_than_2_31_elements(B, H, T, D, windows):
+    """Element offsets beyond 32 bits (4-5 GB per bf16 tensor, up to ~130 GB of device memory with the
+    backward's workspace): the tuned D=64 kernels on full windows, and the band-resident forward and banded
+    backward at D=128; the heads around element 2^31 and the last one against the oracle."""
+    print(f"case beyond 2^31 elements {B, H, T, D} {windows}", flush=True)
+    util.check_offsets_beyond_32_bits("tdp", B, H, T, D, windows)
+
+
 @pytest.mark.parametrize("shape", [(0, 2, 16, 32), (2, 0, 16, 32), (2, 2, 0, 64)])
 def test_empty_inputs_give_empty_results(shape):
     inputs = [torch.zeros(shape, dtype=torch.bfloat16) for _ in range(6)]

@@ -108,3 +108,40 @@ def assert_mostly_close(name, got, want, rtol, atol, outlier_frac=1e-3, outlier_
     bad = err > tol
     assert bad.float().mean().item() <= outlier_frac, f"{name}: {bad.sum().item()} of {bad.numel()} outside tolerance"
     assert (err <= outlier_scale * tol).all(), f"{name}: max error {err.max().item()}"
+
+
+def check_offsets_beyond_32_bits(variant, B, H, T, D, windows=(None,) * 4, rtol=5e-2, atol=2e-2):
+    """Forward and backward on bf16 tensors of more than 2^31 elements (inputs drawn on the device), checked
+    against the oracle on the first head, the heads either side of element 2^31 and the last head."""
+    import math
+
+    from flash_trittention import TrittentionTriton, flash_trittention
+
+    assert B * H * T * D > 2**31
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    draw = lambda: torch.randn(B, H, T, D, device="cuda", dtype=torch.bfloat16, generator=gen)
+    leaves = [draw().requires_grad_(True) for _ in range(5)]
+    do = draw()
+    alpha = 1 / math.sqrt(D)
+    kw = dict(zip(("k1_window", "k2_window", "kk_left", "kk_right"), windows))
+    if variant == "tdp":
+        out = flash_trittention(*leaves, softmax_scale=alpha, causal=True, **kw)
+    else:
+        out, _ = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=T)(*leaves)
+    out.backward(do)
+    torch.cuda.synchronize()
+    edge = 2**31 // (T * D)  # the head that holds element 2^31
+    try:
+        for hd in sorted({0, edge - 1, edge, edge + 1, B * H - 1}):
+            b, h = divmod(hd, H)
+            ins = [t.detach()[b, h].float().cpu() for t in leaves] + [do[b, h].float().cpu()]
+            if variant == "tdp":
+                z, _, grads = orc.tdp_forward_backward_chunked(*ins, alpha, True, q_chunk=128, **kw)
+            else:
+                z, _, grads = orc.dps_forward_backward(*ins, alpha, True, k_diff=T, factorised=True)
+            assert_close(f"out[{hd}]", out.detach()[b, h].float().cpu(), z, rtol=rtol, atol=atol)
+            for name, leaf, want in zip(NAMES, leaves, grads):
+                assert_mostly_close(f"{name}[{hd}]", leaf.grad[b, h].float().cpu(), want, rtol=rtol, atol=atol)
+    finally:
+        del leaves, do, out
+        torch.cuda.empty_cache()
