@@ -240,7 +240,7 @@ __global__ __launch_bounds__(512, 2) void tdp_fwd_band_kernel(FwdParams<E> p, in
             {
                 // P <= its row sum, so a row sum inside this range keeps the value accumulators finite as well
                 const float lk = lsum + __shfl_xor(lsum, 32, 64);
-                fast_ok = !__any(kval && !(lk > 1e-30f && lk < 1e25f));
+                fast_ok = !__any(kval && !(lk > fast_row_sum_floor<E>() && lk < 1e25f));
             }
             if (!fast_ok) {
                 // ---- CAREFUL sweep: online softmax, reference raised lazily; a row may meet its first

@@ -55,6 +55,14 @@ struct FwdParams {
 
 constexpr float kLazyThreshold = 8.0f;
 
+// Smallest row sum the FAST sweep (P = exp2(score), reference 0) accepts.  bf16 has the exponent range of fp32, so
+// only a vanished sum is refused.  fp16 loses mantissa bits below 2^-14 and flushes below 2^-24: a row whose sum is
+// under 2^-10 was summed from values in that range and is redone with a running maximum.
+template <typename E>
+__device__ __forceinline__ constexpr float fast_row_sum_floor() {
+    return std::is_same<E, _Float16>::value ? 9.765625e-4f : 1e-30f;
+}
+
 // MINW (second launch-bounds argument): waves per SIMD the register allocator must leave room for
 // WIN: windowed causal masks.  The k-tile and stage loops run over the band only, every step goes
 // through the general (per tile, element-wise masked) loop, and the CAREFUL sweep tolerates rows whose
@@ -666,7 +674,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 const float lk = lsum[t] + __shfl_xor(lsum[t], 32, 64);
                 bool kval = (kt * 32 + n) <= jmax[t];
                 if constexpr (WIN) kval = whi[t] >= 0;
-                bad |= kval && !(lk > 1e-30f && lk < 1e25f);
+                bad |= kval && !(lk > fast_row_sum_floor<E>() && lk < 1e25f);
             }
             // One barrier per k-tile: this k-tile's flag is read after it; the other flag was read by every
             // wave before it arrived here, is cleared now, and is next written after the barriers of the
@@ -704,20 +712,29 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
             // WIN: the first k-tiles of the band can hold no valid row for this query yet
             const float f = (WIN && mnew == -INFINITY) ? 1.f : fast_exp2(Mrun[t] - mnew);
             const float w = kval ? fast_exp2(mref[t] - mnew) : 0.f;
-            float wl = w * lk;
+            float wl = kval ? w * lk : 0.f;  // a row past the causal bound was swept unmasked: its sum may be inf
 #pragma unroll
             for (int off = 16; off > 0; off >>= 1) wl += __shfl_xor(wl, off, 64);
             Lrun[t] = Lrun[t] * f + wl;
             Mrun[t] = mnew;
             float wr[16];
             rows_of(w, wr);
+            // wr = 0 for rows outside the mask.  The FAST sweep ran them unmasked and unchecked, so their
+            // accumulators may hold inf or NaN (fp16 tensors: exp2 of a score above 16 is inf) and 0 * inf must
+            // not reach the sum: k-tiles that hold such rows (the diagonal one, the edges of a band) clear them.
+            if (!__all(kval)) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[t][dt][i] = wr[i] == 0.f ? 0.f : acc[t][dt][i];
+            }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 float part = 0.f;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const float v = (float)sV2[(kb * 32 + c_row(g, i)) * LDK + dt * 32 + n];
-                    part += wr[i] * v * acc[t][dt][i];  // wr = 0 for rows past the causal bound
+                    part += wr[i] * v * acc[t][dt][i];
                 }
                 Orun[t][dt] = Orun[t][dt] * f + part;
             }

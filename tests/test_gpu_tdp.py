@@ -249,6 +249,26 @@ def test_mfma_forward_large_values_and_logits():
         assert (err > 2e-2).float().mean() < 0.01 and err.max() < 0.2, (err.max(), (err > 2e-2).float().mean())
 
 
+@pytest.mark.parametrize("B,H,T,D,seed,windows", [(2, 5, 32, 64, 13, (None,) * 4), (1, 9, 64, 128, 50, (None,) * 4),
+                                                  (1, 2, 449, 64, 19, (None,) * 4), (1, 3, 200, 32, 7, (None,) * 4),
+                                                  (1, 3, 300, 64, 5, (100, 64, 33, 16))])
+def test_fp16_scores_beyond_the_half_precision_range(B, H, T, D, seed, windows):
+    """fp16 tensors with Q three times larger: exp2 of a score above 16 is inf in half precision.  The fast
+    sweep also runs the virtual rows (q, k > q) of the diagonal k-tile, which no check looks at; what they
+    leave in their accumulators (inf, NaN) must not reach the output through a zero weight.  Forward and all
+    five gradients against the oracle."""
+    print(f"case fp16 range {B, H, T, D} seed {seed} {windows}", flush=True)
+    inputs = list(orc.make_inputs(B, H, T, D, torch.float16, seed=seed))
+    inputs[0] = (inputs[0].float() * 3).half()
+    alpha = 1 / math.sqrt(D)
+    z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
+    out, g = util.run_tdp(inputs, alpha, True, windows, flags=FORCE_MFMA)
+    assert torch.isfinite(out).all() and all(torch.isfinite(x).all() for x in g)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+
+
 def test_mfma_and_generic_agree_bf16():
     inputs = orc.make_inputs(1, 2, 192, 64, torch.bfloat16, seed=23)
     a, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
