@@ -168,6 +168,35 @@ def test_rejects_mismatched_shapes():
         TrittentionTriton()(q, k1, k2, v1, v2[:, :, :16, :].contiguous())
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_shapes_mfma_against_fp32_kernels(seed):
+    """Seeded random draws of (B, H, T, D, dtype, causal, k_diff): the MFMA kernels against the fp32 kernels
+    of the same library on the same 16-bit inputs; every third case scales Q by 3."""
+    import random
+
+    rng = random.Random(seed)
+    for it in range(12):
+        D = rng.choice([32, 64, 128])
+        T = rng.choice([1, 7, 31, 32, 33, 63, 64, 65, 127, 129, 200, 257, 449, 513, 1000])
+        B, H = rng.choice([(1, 1), (1, 3), (2, 5), (1, 9), (3, 3)])
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        causal = rng.random() < 0.85
+        k_diff = rng.choice([0, 1, 2, 5, 31, 32, 33, 100, T, 2 * T, None])
+        qscale = 3 if it % 3 == 2 else 1
+        print(f"case random {seed}.{it}: {B, H, T, D} {dtype} causal={causal} k_diff={k_diff} q*{qscale}", flush=True)
+        inputs = list(orc.make_inputs(B, H, T, D, dtype, seed=100 * seed + it))
+        inputs[0] = (inputs[0].float() * qscale).to(dtype)
+        alpha = 1 / math.sqrt(D)
+        a, ma, ga = util.run_dps(inputs, alpha, causal, k_diff, flags=2)
+        b, mb, gb = util.run_dps(inputs, alpha, causal, k_diff, flags=1)
+        assert torch.isfinite(a).all() and torch.isfinite(ma).all() and all(torch.isfinite(x).all() for x in ga)
+        tol = dict(rtol=5e-2 * qscale, atol=2e-2 * qscale)
+        util.assert_mostly_close("out", a, b, **tol)
+        util.assert_mostly_close("m", ma, mb, **tol)
+        for name, x, y in zip(util.NAMES, ga, gb):
+            util.assert_mostly_close(name, x, y, **tol)
+
+
 def test_tensors_of_more_than_2_31_elements():
     """Element offsets beyond 32 bits: B*H = 52500 heads of T=640, D=64 (4.3 GB per bf16 tensor)."""
     print("case beyond 2^31 elements (7, 7500, 640, 64)", flush=True)

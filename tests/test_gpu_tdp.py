@@ -269,6 +269,40 @@ def test_fp16_scores_beyond_the_half_precision_range(B, H, T, D, seed, windows):
         util.assert_mostly_close(name, a, b, **LOWP)
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_shapes_mfma_against_fp32_kernels(seed):
+    """Seeded random draws of (B, H, T, D, dtype, causal, windows): the MFMA kernels against the fp32 VALU
+    kernels of the same library on the same 16-bit inputs (both go through the C ABI; the fp32 kernels are
+    pinned to the oracle by the tests above).  Every third case scales Q by 3: finiteness and agreement there
+    too (fp16 scores beyond the half-precision range included)."""
+    import random
+
+    rng = random.Random(seed)
+    for it in range(12):
+        D = rng.choice([32, 64, 128])
+        T = rng.choice([1, 7, 31, 32, 33, 63, 64, 65, 95, 127, 129, 191, 200, 257, 320, 449])
+        B, H = rng.choice([(1, 1), (1, 3), (2, 5), (1, 9), (3, 3)])
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        causal = rng.random() < 0.85
+        windows = (None,) * 4
+        if rng.random() < 0.7:
+            windows = tuple(rng.choice([0, 1, 2, 5, 16, 31, 32, 33, 64, 100, 200, T, 2 * T]) for _ in range(4))
+        qscale = 3 if it % 3 == 2 else 1
+        print(f"case random {seed}.{it}: {B, H, T, D} {dtype} causal={causal} {windows} q*{qscale}", flush=True)
+        inputs = list(orc.make_inputs(B, H, T, D, dtype, seed=100 * seed + it))
+        inputs[0] = (inputs[0].float() * qscale).to(dtype)
+        alpha = 1 / math.sqrt(D)
+        a, ga = util.run_tdp(inputs, alpha, causal, windows, flags=FORCE_MFMA)
+        b, gb = util.run_tdp(inputs, alpha, causal, windows, flags=FORCE_GENERIC)
+        assert torch.isfinite(a).all() and all(torch.isfinite(x).all() for x in ga)
+        # scores three times larger sharpen the softmax: the 16-bit rounding of P and dS then shows in the
+        # gradients' cancellations, so those cases get three times the tolerance
+        tol = dict(rtol=LOWP["rtol"] * qscale, atol=LOWP["atol"] * qscale)
+        util.assert_mostly_close("out", a, b, **tol)
+        for name, x, y in zip(util.NAMES, ga, gb):
+            util.assert_mostly_close(name, x, y, **tol)
+
+
 def test_mfma_and_generic_agree_bf16():
     inputs = orc.make_inputs(1, 2, 192, 64, torch.bfloat16, seed=23)
     a, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
