@@ -605,12 +605,12 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                         for (int ks = 0; ks < KS; ++ks)
                             ka[ks] = *reinterpret_cast<const v8*>(k1p + half * 32 * LDK + ks * 16);
                     };
-                    auto load_u = [&](int half) {
+                    // U^T operands of key half `half`, k-step h: fetched as soon as the registers they take over
+                    // (K1 operands, or the other half's U^T operands) have been issued to their last MFMA
+                    auto load_u = [&](int half, int h) {
 #pragma unroll
                         for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                            for (int h = 0; h < 2; ++h)
-                                ua[dt][h] = *reinterpret_cast<const v8*>(utp + half * 32 + dt * 32 * LDU + h * 16);
+                            ua[dt][h] = *reinterpret_cast<const v8*>(utp + half * 32 + dt * 32 * LDU + h * 16);
                     };
                     auto pair = [&](int half, int r) {  // register pair r (0..7): 2 exp2, 1 pack, 1 row-sum step
                         const int h = r >> 2, e = 2 * (r & 3);
@@ -629,25 +629,28 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     for (int ks = 0; ks < KS; ++ks) sc[0] = M::mma(ka[ks], bq[0][ks], sc[0]);
                     __builtin_amdgcn_sched_barrier(0);
                     load_k(1);
-                    load_u(0);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks) {
                         sc[1] = M::mma(ka[ks], bq[0][ks], sc[1]);
                         __builtin_amdgcn_sched_barrier(0);
+                        if (ks == KS / 2 - 1) load_u(0, 0);
 #pragma unroll
                         for (int r = ks * 8 / KS; r < (ks + 1) * 8 / KS; ++r) pair(0, r);
                         __builtin_amdgcn_sched_barrier(0);
                     }
+                    load_u(0, 1);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int r = 0; r < 2 * DT; ++r) {
                         value_mma(0, r);
                         __builtin_amdgcn_sched_barrier(0);
+                        if (r == DT - 1) load_u(1, 0);
 #pragma unroll
                         for (int q2 = r * 8 / (2 * DT); q2 < (r + 1) * 8 / (2 * DT); ++q2) pair(1, q2);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    load_u(1);
+                    load_u(1, 1);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int r = 0; r < 2 * DT; ++r) value_mma(1, r);
