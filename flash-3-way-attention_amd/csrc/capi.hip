@@ -1,6 +1,7 @@
 // C ABI of libtrittention_hip.so: argument checks, scratch layout, dispatch.
 // Declarations and the contract of each entry point: include/trittention_hip.h.
 #include <cstdint>
+#include <mutex>
 #include "../../include/trittention_hip.h"
 
 #include "common.hpp"
@@ -288,6 +289,32 @@ bool any_misaligned(std::initializer_list<const void*> ps) {
     return false;
 }
 
+// Library-owned scratch of tritt_tdp_fwd_static_scratch: one copy per GPU the code object is loaded on, held
+// until the process ends.  The name is a host-side stand-in; the device address comes from hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char scratch[TRITT_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up once per device).
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return TRITT_ERR_INVALID;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p || (reinterpret_cast<uintptr_t>(p) & 255)) return TRITT_ERR_INVALID;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return TRITT_OK;
+}
+
 }  // namespace
 }  // namespace tritt
 
@@ -304,6 +331,7 @@ const char* tritt_status_string(int status) {
         case TRITT_ERR_HEAD_DIM: return "head dimension must be 16, 32, 64 or 128";
         case TRITT_ERR_WORKSPACE: return "workspace missing or too small";
         case TRITT_ERR_UNSUPPORTED: return "requested implementation does not support this configuration";
+        case TRITT_ERR_SCRATCH_LIMIT: return "problem needs more scratch than the library's static buffer holds";
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
     return "unknown status";
@@ -356,6 +384,27 @@ int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1,
     Arena ar(workspace);
     return tdp_fwd_generic(ar, true, q, k1, k2, v1, v2, o, lse, B, H, T, D, dtype, alpha, causal, w1, w2, kl, kr,
                            (hipStream_t)stream);
+}
+
+size_t tritt_static_scratch_bytes(void) { return TRITT_STATIC_SCRATCH_BYTES; }
+
+int tritt_tdp_fwd_static_scratch(const void* q, const void* k1, const void* k2, const void* v1, const void* v2, void* o,
+                                 float* lse, int B, int H, int T, int D, int dtype, float alpha, int causal,
+                                 int k1_window, int k2_window, int kk_left, int kk_right, unsigned flags,
+                                 void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    const size_t need = tritt_tdp_fwd_workspace_bytes(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left,
+                                                      kk_right, flags);
+    if (need > TRITT_STATIC_SCRATCH_BYTES) return TRITT_ERR_SCRATCH_LIMIT;
+    void* ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc != TRITT_OK) return rc;
+    // every kernel of the forward writes the part of the scratch it later reads (the transposed SiLU(V1) copy
+    // including its zero padding, the parts of a split forward): nothing has to be cleared between calls
+    return tritt_tdp_fwd(q, k1, k2, v1, v2, o, lse, B, H, T, D, dtype, alpha, causal, k1_window, k2_window, kk_left,
+                         kk_right, ws, TRITT_STATIC_SCRATCH_BYTES, flags, stream);
 }
 
 size_t tritt_tdp_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,

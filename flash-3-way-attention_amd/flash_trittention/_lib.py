@@ -26,6 +26,8 @@ _PROTOS = {
     "tritt_status_string": (ctypes.c_char_p, [_i]),
     "tritt_tdp_fwd_workspace_bytes": (_sz, [_i] * 10 + [_u]),
     "tritt_tdp_fwd": (_i, [_vp] * 7 + [_i] * 5 + [_f] + [_i] * 5 + [_vp, _sz, _u, _vp]),
+    "tritt_static_scratch_bytes": (_sz, []),
+    "tritt_tdp_fwd_static_scratch": (_i, [_vp] * 7 + [_i] * 5 + [_f] + [_i] * 5 + [_u, _vp]),
     "tritt_tdp_bwd_workspace_bytes": (_sz, [_i] * 10 + [_u]),
     "tritt_tdp_bwd": (_i, [_vp] * 13 + [_i] * 5 + [_f] + [_i] * 5 + [_vp, _sz, _u, _vp]),
     "tritt_dps_fwd_workspace_bytes": (_sz, [_i] * 5 + [_u]),

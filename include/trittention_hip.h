@@ -38,7 +38,9 @@ enum {
                                    B*H above 65535 or B*H*T above 2^31-1                    */
     TRITT_ERR_HEAD_DIM = -2,    /* D not one of 16, 32, 64, 128                            */
     TRITT_ERR_WORKSPACE = -3,   /* workspace missing or smaller than *_workspace_bytes     */
-    TRITT_ERR_UNSUPPORTED = -4  /* requested implementation cannot run this configuration */
+    TRITT_ERR_UNSUPPORTED = -4, /* requested implementation cannot run this configuration */
+    TRITT_ERR_SCRATCH_LIMIT = -5 /* tritt_tdp_fwd_static_scratch: the problem needs more scratch
+                                    than TRITT_STATIC_SCRATCH_BYTES                         */
 };
 
 /* `flags` bits */
@@ -76,6 +78,25 @@ int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1,
                   int B, int H, int T, int D, int dtype, float alpha, int causal,
                   int k1_window, int k2_window, int kk_left, int kk_right,
                   void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
+/* tritt_tdp_fwd_static_scratch has no counterpart in the reference.  It is tritt_tdp_fwd for
+ * callers that cannot allocate device memory at all (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the scratch that tritt_tdp_fwd takes as
+ * `workspace` lives in a static device array inside the library instead, of
+ * TRITT_STATIC_SCRATCH_BYTES bytes per GPU, held until the process ends.  The call allocates
+ * and frees nothing.  Problems whose tritt_tdp_fwd_workspace_bytes() exceeds that size are
+ * rejected with TRITT_ERR_SCRATCH_LIMIT before anything is launched (32 MiB covers the
+ * forward up to B*H*T*D = 16 Mi 16-bit elements, e.g. B=1 H=16 T=4096 D=128).  All calls on
+ * one GPU share the one array: calls that overlap in time on the same GPU (different
+ * streams or threads) race; serialise them.  Results are identical to tritt_tdp_fwd's.
+ * tritt_static_scratch_bytes() returns the limit the library was built with. */
+#define TRITT_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+size_t tritt_static_scratch_bytes(void);
+int tritt_tdp_fwd_static_scratch(const void* q, const void* k1, const void* k2, const void* v1,
+                                 const void* v2, void* o, float* lse,
+                                 int B, int H, int T, int D, int dtype, float alpha, int causal,
+                                 int k1_window, int k2_window, int kk_left, int kk_right,
+                                 unsigned flags, void* stream);
 
 size_t tritt_tdp_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
                                      int k1_window, int k2_window, int kk_left, int kk_right,
