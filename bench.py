@@ -25,13 +25,13 @@ for _p in (ROOT, os.path.join(ROOT, "flash-3-way-attention_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch at the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# scaled by a plain 256 MiB copy (see the summaries under profiles/); not measured live
-TRAFFIC_FWD = 27.0e6        # 21.6 MiB fetched + 4.1 MiB written
-# average of the two launches: 264-268 MiB of fp32 atomics written and 34-90 MiB fetched; in some dispatches (most of
-# them on some boxes) the first launch fetches ~500 MiB instead: its atomically accumulated row gradients then fall
-# out of their XCD's L2 (same duration either way)
-TRAFFIC_BWD_ROWS = 350e6
+NOMINAL_CLOCK_MHZ = 2400.0  # the clock behind the published peak
+# HBM bytes per launch, NOT measured live: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script at the
+# default workload only, scaled by a plain 256 MiB copy (summary and commands:
+# profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt).  Reported only when the workload is the default one.
+TRAFFIC_SOURCE = "profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt (rocprofv3 --pmc, default workload only)"
+TRAFFIC_FWD = 27.0e6        # 22.7 MiB fetched + 4.1 MiB written
+TRAFFIC_BWD_ROWS = 600e6    # average of the two launches: ~530 MiB of 64-bit atomics written, 40-95 MiB fetched
 
 
 def triples(B, H, T, causal=True):
@@ -93,6 +93,45 @@ def time_events(fn, iters, warmup, torch):
     return start.elapsed_time(stop) / iters
 
 
+def cpu_info():
+    """Model string of the host CPU and how many of its cores this process may use."""
+    model = None
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    quota = None
+    try:
+        with open("/sys/fs/cgroup/cpu.max") as f:
+            lim, period = f.read().split()
+            if lim != "max":
+                quota = float(lim) / float(period)
+    except (OSError, ValueError):
+        pass
+    return {"model": model, "os_cpu_count": os.cpu_count(), "affinity": len(os.sched_getaffinity(0)),
+            "cgroup_cpu_quota": quota, "OMP_NUM_THREADS": os.environ.get("OMP_NUM_THREADS")}
+
+
+def mfma_probe(torch, _lib, blocks=2048, iters=4096):
+    """Rate of a kernel that does nothing but bf16 MFMAs (tritt_probe_mfma), and the clock it implies."""
+    out = torch.empty(blocks * 512, dtype=torch.float32, device="cuda")
+    lib = _lib.lib()
+
+    def run():
+        _lib.check(lib.tritt_probe_mfma(_lib.ptr(out), blocks, iters, _lib.stream_ptr(out.device)), "tritt_probe_mfma")
+
+    ms = time_events(run, 5, 2, torch)
+    tflops = blocks * 8 * iters * 4 * 32768 / ms / 1e9
+    return {"tflops": tflops, "ms": ms,
+            "implied_clock_mhz": tflops / PEAK_BF16_TFLOPS * NOMINAL_CLOCK_MHZ,
+            "what": "a kernel of independent 32x32x16 bf16 MFMAs only, 16 waves per CU: the matrix rate this chip "
+                    "sustains; implied clock = rate / 2500 TFLOP/s x 2400 MHz"}
+
+
 def cpu_baseline(T, D, alpha, seconds_budget=30.0):
     """The oracle's naive dense path (einsum -> mask -> softmax over the flattened (j,k)
     plane -> einsum, gradients by autograd), fp32, on this host's cores: a few heads of the
@@ -102,8 +141,14 @@ def cpu_baseline(T, D, alpha, seconds_budget=30.0):
 
     from oracle import trittention_oracle as orc
 
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
+    # every core this process may use: the smaller of its affinity mask, its cgroup quota and an OMP_NUM_THREADS the
+    # box sets for its share of the host (oversubscribing a share only slows the ATen kernels down)
+    info = cpu_info()
+    cores = info["affinity"]
+    if info["cgroup_cpu_quota"]:
+        cores = min(cores, max(1, int(info["cgroup_cpu_quota"])))
+    if info["OMP_NUM_THREADS"] and info["OMP_NUM_THREADS"].isdigit():
+        cores = min(cores, int(info["OMP_NUM_THREADS"]))
     torch.set_num_threads(cores)
     max_heads = 8
     full = orc.make_inputs(1, max_heads, T, D, torch.bfloat16, seed=0)
@@ -121,11 +166,93 @@ def cpu_baseline(T, D, alpha, seconds_budget=30.0):
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
+        "cpu": info,
         "seconds": dt,
         "sample": f"{heads} of the 32 heads of the workload (T={T}, D={D}), all query rows, fwd+bwd, "
                   "dense fp32 in 64-row query chunks, heads one after another until 12 s have passed; "
                   "throughput = algorithmic flops of those heads / time",
     }
+
+
+def sweep_rows(torch, flash_trittention, dev, steps):
+    """BASELINE config 5: triple-dot forward, B=1 H=16 D=128 bf16 causal, T = 512 .. 4096."""
+    rows = []
+    for Ts in (512, 1024, 2048, 4096):
+        ins = [t.to(dev) for t in make_inputs(1, 16, Ts, 128, torch.bfloat16, seed=0, n=5)]
+        torch.cuda.reset_peak_memory_stats()
+        base_mem = torch.cuda.memory_allocated()
+
+        def f():
+            with torch.no_grad():
+                return flash_trittention(*ins, softmax_scale=1 / math.sqrt(128), k1_window=None, k2_window=None,
+                                         kk_left=None, kk_right=None, causal=True)
+
+        ms = time_events(f, max(3, min(4 * steps, 65536 // Ts)), 3 if Ts <= 2048 else 1, torch)
+        fl = 4 * 128 * triples(1, 16, Ts)
+        rows.append({"T": Ts, "ms": ms, "tflops": fl / ms / 1e9, "frac_of_bf16_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS,
+                     "extra_device_bytes": torch.cuda.max_memory_allocated() - base_mem,
+                     "one_tensor_bytes": 16 * Ts * 128 * 2})
+    return rows
+
+
+def dps_times(torch, dev, B, H, T, D, steps, warmup):
+    """BASELINE config 4: dot-product-sum forward and backward (events around the Python calls)."""
+    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
+
+    alpha = 1 / math.sqrt(D)
+    ins = [t.to(dev) for t in make_inputs(B, H, T, D, torch.bfloat16, seed=0)]
+    lv = [t.clone().requires_grad_(True) for t in ins[:5]]
+    mod = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=T)
+    hold = {}
+
+    def f():
+        hold["o"] = mod(*lv)[0]
+
+    def b():
+        hold["o"].backward(ins[5], retain_graph=True)
+
+    ms_f = time_events(f, steps, max(warmup, 3), torch)
+    ms_b = time_events(b, steps, max(warmup, 3), torch)  # the first backward pays one-time set-up
+    n3 = B * H * T * (T + 1) * (T + 2) // 6   # valid (q,s,t) triples of the reference's formulation
+    n2 = B * H * T * (T + 1) // 2              # (row, column) pairs of the factorised one
+    bytes_f, bytes_b = 6 * B * H * T * D * 2 + 4 * B * H * T, 12 * B * H * T * D * 2 + 8 * B * H * T
+    return {"fwd_ms": ms_f, "bwd_ms": ms_b,
+            "executed_fwd_tflops": 8 * D * n2 / ms_f / 1e9, "executed_bwd_tflops": 20 * D * n2 / ms_b / 1e9,
+            "reference_formulation_fwd_tflops_equiv": 4 * D * n3 / ms_f / 1e9,
+            "algorithmic_bytes_fwd": bytes_f, "algorithmic_bytes_bwd": bytes_b,
+            "io_gbs_fwd": bytes_f / ms_f / 1e6, "io_gbs_bwd": bytes_b / ms_b / 1e6,
+            # the factorised path is bound by HBM (8.6 / 21.5 GFLOP on 25 / 50 MB): fraction of the 8 TB/s floor
+            "roofline_fwd": {"bound": "hbm", "achieved": bytes_f / ms_f / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": bytes_f / ms_f / 1e6 / PEAK_HBM_GBS},
+            "roofline_bwd": {"bound": "hbm", "achieved": bytes_b / ms_b / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": bytes_b / ms_b / 1e6 / PEAK_HBM_GBS},
+            "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} bf16 causal"}}
+
+
+def tdp_times(torch, flash_trittention, dev, B, H, T, D, dtype, steps, warmup, backward=True):
+    """Triple-dot forward (and backward) milliseconds at one shape, full windows."""
+    alpha = 1 / math.sqrt(D)
+    q, k1, k2, v1, v2, do = (t.to(dev) for t in make_inputs(B, H, T, D, dtype, seed=0))
+    leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+    kw = dict(softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True)
+    hold = {}
+
+    def fwd():
+        with torch.no_grad():
+            return flash_trittention(q, k1, k2, v1, v2, **kw)
+
+    def bwd():
+        hold["o"].backward(do, retain_graph=True)
+
+    n = triples(B, H, T)
+    row = {"workload": f"triple-dot B={B} H={H} T={T} D={D} {str(dtype).split('.')[-1]} causal",
+           "fwd_ms": time_events(fwd, steps, warmup, torch)}
+    row["fwd_tflops"] = 4 * D * n / row["fwd_ms"] / 1e9
+    if backward:
+        hold["o"] = flash_trittention(*leaves, **kw)
+        row["bwd_ms"] = time_events(bwd, steps, warmup, torch)
+        row["bwd_tflops"] = 12 * D * n / row["bwd_ms"] / 1e9
+    return row
 
 
 def main():
@@ -134,6 +261,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--brief", action="store_true", help="default mode: skip the other BASELINE configurations")
     ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "dps", "tdp", "published"], default="both",
                     help="fwd: time only the forward (for profiling runs); copy: a plain 256 MiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against; "
@@ -172,22 +300,7 @@ def main():
     B, H, T, D = args.B, args.H, args.T, args.D
     alpha = 1 / math.sqrt(D)
     if args.mode == "sweep":
-        rows = []
-        for Ts in (512, 1024, 2048, 4096):
-            ins = [t.to(dev) for t in make_inputs(1, 16, Ts, 128, torch.bfloat16, seed=0, n=5)]
-            torch.cuda.reset_peak_memory_stats()
-            base_mem = torch.cuda.memory_allocated()
-
-            def f():
-                with torch.no_grad():
-                    return flash_trittention(*ins, softmax_scale=1 / math.sqrt(128), k1_window=None, k2_window=None,
-                                             kk_left=None, kk_right=None, causal=True)
-
-            ms = time_events(f, max(3, min(4 * args.steps, 65536 // Ts)), 3 if Ts <= 2048 else 1, torch)
-            fl = 4 * 128 * triples(1, 16, Ts)
-            rows.append({"T": Ts, "ms": ms, "tflops": fl / ms / 1e9, "frac_of_bf16_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS,
-                         "extra_device_bytes": torch.cuda.max_memory_allocated() - base_mem,
-                         "one_tensor_bytes": 16 * Ts * 128 * 2})
+        rows = sweep_rows(torch, flash_trittention, dev, args.steps)
         print(json.dumps({"metric": "triple-dot trittention fwd TFLOP/s vs T", "unit": "TFLOP/s",
                           "config": {"workload": "triple-dot fwd B=1 H=16 D=128 bf16 causal"}, "rows": rows}), flush=True)
         return
@@ -215,28 +328,8 @@ def main():
                           "config": {"workload": "triple-dot fwd B=2 H=8 D=64 fp16 causal"}, "rows": rows}), flush=True)
         return
     if args.mode == "dps":
-        from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
-
-        ins = [t.to(dev) for t in make_inputs(B, H, T, D, torch.bfloat16, seed=0)]
-        lv = [t.clone().requires_grad_(True) for t in ins[:5]]
-        mod = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=T)
-        hold = {}
-
-        def f():
-            hold["o"] = mod(*lv)[0]
-
-        def b():
-            hold["o"].backward(ins[5], retain_graph=True)
-
-        ms_f = time_events(f, args.steps, max(args.warmup, 3), torch)
-        ms_b = time_events(b, args.steps, max(args.warmup, 3), torch)  # the first backward pays one-time set-up
-        n3 = B * H * T * (T + 1) * (T + 2) // 6   # valid (q,s,t) triples of the reference's formulation
-        n2 = B * H * T * (T + 1) // 2              # (row, column) pairs of the factorised one
-        print(json.dumps({"metric": "dot-product-sum trittention fwd / bwd ms", "unit": "ms", "fwd_ms": ms_f, "bwd_ms": ms_b,
-                          "executed_fwd_tflops": 8 * D * n2 / ms_f / 1e9, "executed_bwd_tflops": 20 * D * n2 / ms_b / 1e9,
-                          "reference_formulation_fwd_tflops_equiv": 4 * D * n3 / ms_f / 1e9,
-                          "io_gbs_fwd": (6 * B * H * T * D * 2) / ms_f / 1e6,
-                          "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} bf16 causal"}}), flush=True)
+        r = dps_times(torch, dev, B, H, T, D, args.steps, args.warmup)
+        print(json.dumps({"metric": "dot-product-sum trittention fwd / bwd ms", "unit": "ms", **r}), flush=True)
         return
     tdtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype if args.mode == "tdp" else "bf16"]
     q, k1, k2, v1, v2, do = (t.to(dev) for t in make_inputs(B, H, T, D, tdtype, seed=0))
@@ -300,6 +393,8 @@ def main():
     ms_bwd = time_events(bwd_only, max(args.steps // 2, 3), 1, torch)
 
     fwd_tf, bwd_tf = f_fwd / ms_fwd / 1e9, f_bwd / ms_bwd / 1e9
+    default_workload = (B, H, T, D) == (4, 8, 1024, 64)
+    probe = mfma_probe(torch, _lib)
     elem = 2
     bytes_fwd = 6 * B * H * T * D * elem + 4 * B * H * T
     bytes_bwd = 12 * B * H * T * D * elem + 8 * B * H * T
@@ -323,19 +418,38 @@ def main():
         "fwd_hbm_gbs": bytes_fwd / ms_fwd / 1e6, "bwd_hbm_gbs": bytes_bwd / ms_bwd / 1e6,
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "nominal_clock_mhz": nominal_clock_mhz(),
-                   "peak_used": "2.5 PFLOP/s bf16 dense (256 CUs x 4096 flop/clk x 2.4 GHz nominal)"},
+                   "peak_used": "2.5 PFLOP/s bf16 dense (256 CUs x 4096 flop/clk x 2.4 GHz nominal)",
+                   # measured in this run: what a pure-MFMA kernel reaches, and the clock that implies
+                   "mfma_probe": probe},
         # dominant kernel by time: tdp_bwd_rows_kernel, launched twice per backward (dQ,dK2,dV2 then
         # dK1,dU).  Each launch is credited half of the backward's algorithmic flops (6*D*N) and
         # half of the event-timed backward (the prep/finish kernels in that time are < 1 %).
         "roofline": {"bound": "mfma", "kernel": "tdp_bwd_rows_kernel<bf16,64> (avg of its 2 launches)",
                      "achieved": bwd_tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": bwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BWD_ROWS,
+                     "frac": bwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BWD_ROWS if default_workload else None,
+                     "traffic_source": TRAFFIC_SOURCE if default_workload else None,
+                     "frac_of_sustained_mfma_rate": bwd_tf / probe["tflops"],
                      "flops_per_launch": f_bwd // 2, "ms_per_launch": ms_bwd / 2},
         "roofline_fwd": {"bound": "mfma", "kernel": "tdp_fwd_mfma_kernel<bf16,64,NT=2,8 waves>",
                          "achieved": fwd_tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": fwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_FWD,
+                         "frac": fwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_FWD if default_workload else None,
+                         "traffic_source": TRAFFIC_SOURCE if default_workload else None,
+                         "frac_of_sustained_mfma_rate": fwd_tf / probe["tflops"],
                          "flops_per_launch": f_fwd, "ms_per_launch": ms_fwd},
     }
+    if not args.brief:
+        # the other BASELINE configurations, timed in the same run (parity for each: tests/test_gpu_*.py)
+        short = max(5, min(args.steps, 20))
+        result["other_configs"] = {
+            "config1_tdp_fwd_fp32": tdp_times(torch, flash_trittention, dev, 1, 2, 64, 32, torch.float32, 20, 5,
+                                              backward=False),
+            "config2_tdp_fwd_bwd": tdp_times(torch, flash_trittention, dev, 2, 4, 256, 64, torch.bfloat16, 20, 5),
+            "config4_dps_fwd_bwd": dps_times(torch, dev, 4, 8, 1024, 64, 20, 5),
+            "config5_tdp_fwd_sweep": {"workload": "triple-dot fwd B=1 H=16 D=128 bf16 causal",
+                                      "rows": sweep_rows(torch, flash_trittention, dev, short)},
+            "tdp_fwd_bwd_d128": tdp_times(torch, flash_trittention, dev, 4, 8, 1024, 128, torch.bfloat16, 3, 1),
+            "tdp_fwd_bwd_fp32_d32": tdp_times(torch, flash_trittention, dev, 4, 8, 1024, 32, torch.float32, 2, 1),
+        }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(T, D, alpha)
     print(json.dumps(result), flush=True)

@@ -1,13 +1,62 @@
 // C ABI of libtrittention_hip.so: argument checks, scratch layout, dispatch.
 // Declarations and the contract of each entry point: include/trittention_hip.h.
+#include <atomic>
 #include <cstdint>
+#include <cstdlib>
+#include <cstring>
 #include <mutex>
+#include <vector>
 #include "../../include/trittention_hip.h"
 
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace tritt {
+
+namespace {
+std::atomic<int> g_knobs[TRITT_TUNE_COUNT_];
+std::once_flag g_knobs_once;
+void init_knobs() {
+    std::call_once(g_knobs_once, [] {
+        if (const char* e = getenv("TRITT_FWD_SPLITS")) g_knobs[TRITT_TUNE_FWD_SPLITS] = atoi(e);
+        if (const char* e = getenv("TRITT_FWD_BAND")) g_knobs[TRITT_TUNE_FWD_BAND] = atoi(e) == 0 ? -1 : 0;
+        if (const char* e = getenv("TRITT_BWD_SPLITS")) g_knobs[TRITT_TUNE_BWD_SPLITS] = atoi(e);
+        if (const char* e = getenv("TRITT_BWD128_VARIANT"))
+            g_knobs[TRITT_TUNE_BWD128_WAVES] = strcmp(e, "w4") == 0 ? 4 : strcmp(e, "w8") == 0 ? 8 : 0;
+    });
+}
+}  // namespace
+
+Knobs knobs() {
+    init_knobs();
+    return Knobs{g_knobs[TRITT_TUNE_FWD_SPLITS].load(), g_knobs[TRITT_TUNE_FWD_BAND].load(),
+                 g_knobs[TRITT_TUNE_BWD_SPLITS].load(), g_knobs[TRITT_TUNE_BWD128_WAVES].load()};
+}
+
+hipError_t ensure_dynamic_smem(const void* kernel, size_t bytes) {
+    struct Entry {
+        int device;
+        const void* kernel;
+        size_t bytes;
+    };
+    static std::mutex mutex;
+    static std::vector<Entry> done;
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(mutex);
+    for (Entry& en : done)
+        if (en.device == device && en.kernel == kernel) {
+            if (en.bytes >= bytes) return hipSuccess;
+            e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+            if (e == hipSuccess) en.bytes = bytes;
+            return e;
+        }
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) done.push_back({device, kernel, bytes});
+    return e;
+}
+
 namespace {
 
 // Bump allocator over the caller's workspace; with base == nullptr it only measures.
@@ -63,12 +112,14 @@ __global__ __launch_bounds__(256) void from_f32_kernel(const float* __restrict__
 template <typename T>
 __global__ __launch_bounds__(256) void rowdot_kernel(const T* __restrict__ a, const T* __restrict__ b,
                                                      float* __restrict__ out, int rows, int D) {
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (row >= rows) return;
-    float part = 0.f;
-    for (int d = lane; d < D; d += 64) part += to_float(a[(size_t)row * D + d]) * to_float(b[(size_t)row * D + d]);
-    part = wave_sum(part);
-    if (lane == 0) out[row] = part;
+    const int lane = threadIdx.x & 63;
+    // grid-stride over rows: the grid is capped, and rows may be close to 2^31
+    for (long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += (long long)gridDim.x * 4) {
+        float part = 0.f;
+        for (int d = lane; d < D; d += 64) part += to_float(a[(size_t)row * D + d]) * to_float(b[(size_t)row * D + d]);
+        part = wave_sum(part);
+        if (lane == 0) out[row] = part;
+    }
 }
 
 unsigned ew_grid(size_t n) {
@@ -96,7 +147,8 @@ void from_f32(const float* src, const void* v1, void* dst, size_t n, int dtype, 
 }
 
 void rowdot(const void* a, const void* b, float* out, int rows, int D, int dtype, hipStream_t st) {
-    dim3 grid((rows + 3) / 4);
+    const long long blocks = ((long long)rows + 3) / 4;
+    dim3 grid((unsigned)(blocks > 65536 ? 65536 : blocks));
     if (dtype == TRITT_F32)
         hipLaunchKernelGGL(rowdot_kernel<float>, grid, dim3(256), 0, st, (const float*)a, (const float*)b, out, rows, D);
     else if (dtype == TRITT_BF16)
@@ -322,7 +374,13 @@ using namespace tritt;
 
 extern "C" {
 
-int tritt_version(void) { return 100; }
+int tritt_version(void) { return 200; }
+
+int tritt_set_tuning(int knob, int value) {
+    if (knob < 0 || knob >= TRITT_TUNE_COUNT_) return TRITT_ERR_INVALID;
+    init_knobs();
+    return g_knobs[knob].exchange(value);
+}
 
 const char* tritt_status_string(int status) {
     switch (status) {
@@ -411,7 +469,7 @@ size_t tritt_tdp_bwd_workspace_bytes(int B, int H, int T, int D, int dtype, int 
                                      int kk_left, int kk_right, unsigned flags) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
     if (use_mfma_bwd(T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags))
-        return mfma_tdp_bwd_workspace(B * H, T, D);
+        return mfma_tdp_bwd_workspace(B * H, T, D, (flags & TRITT_FLAG_FLOAT_ATOMICS) == 0);
     Arena ar(nullptr);
     tdp_bwd_generic(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                     nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f, causal, k1_window, k2_window, kk_left, kk_right,
@@ -443,6 +501,7 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
         a.is_bf16 = dtype == TRITT_BF16;
         a.windowed = full_windows(T, causal, w1, w2, kl, kr) ? 0 : 1;
         a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+        a.deterministic = (flags & TRITT_FLAG_FLOAT_ATOMICS) ? 0 : 1;
         return (int)mfma_tdp_bwd(a, (hipStream_t)stream);
     }
     Arena ar(workspace);

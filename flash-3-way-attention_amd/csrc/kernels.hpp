@@ -5,6 +5,20 @@
 
 namespace tritt {
 
+// Tuning overrides (tritt_set_tuning; initial values from the environment, read once per process, so that a
+// workspace query and the launch that follows it agree).  0 = automatic.
+struct Knobs {
+    int fwd_splits;      // TRITT_TUNE_FWD_SPLITS / env TRITT_FWD_SPLITS: workgroups per query tile, forward (1..8)
+    int fwd_band;        // TRITT_TUNE_FWD_BAND / env TRITT_FWD_BAND: -1 switches the band-resident forward off
+    int bwd_splits;      // TRITT_TUNE_BWD_SPLITS / env TRITT_BWD_SPLITS: workgroups per query tile, backward (1..16)
+    int bwd128_variant;  // TRITT_TUNE_BWD128_WAVES / env TRITT_BWD128_VARIANT=w8|w4: 8 or 4 waves per workgroup
+};
+Knobs knobs();
+
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per (device, kernel): the attribute belongs to the
+// device's copy of the kernel, and a process may drive several devices.
+hipError_t ensure_dynamic_smem(const void* kernel, size_t bytes);
+
 // fp32 [BH, T, D] operands of the VALU triple-dot kernels (u = SiLU(V1)).
 struct GenericTdpArgs {
     const float *q, *k1, *k2, *u, *v2;
@@ -68,8 +82,9 @@ struct MfmaBwdArgs {
     int is_bf16;
     int windowed;  // some window can exclude a pair with j, k <= q: the banded kernels
     int k1_window, k2_window, kk_left, kk_right;
+    int deterministic;  // 64-bit fixed-point accumulators: bitwise reproducible gradients
 };
-size_t mfma_tdp_bwd_workspace(int BH, int T, int D);
+size_t mfma_tdp_bwd_workspace(int BH, int T, int D, bool deterministic);
 bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st);
 

@@ -38,6 +38,10 @@ struct BwdParams {
     // one, dQ / alpha is accumulated into acc_q (fp32, zero on entry) instead of being written to dq
     float* acc_q;
     int splits;
+    // accumulate the row gradients (and a split dQ) as 64-bit fixed point with integer atomics: integer addition is
+    // associative, so the sums are bitwise the same whatever order the workgroups arrive in.  The accumulators
+    // then hold long long where they otherwise hold float (twice the bytes, same element index).
+    int fixed_point;
     int T, Tp, BH, nqt;
     float alpha;
     int causal;
@@ -45,6 +49,18 @@ struct BwdParams {
     // iff a, b <= q, q - a <= wa, q - b <= wb, b - a <= lab, a - b <= rab
     int wa, wb, lab, rab;
 };
+
+// 2^30: the accumulators cover |sum| < 8.6e9 in steps of 9.3e-10
+constexpr float kFixedScale = 1073741824.0f;
+
+// One contribution to a gradient accumulator that several workgroups add to.
+template <typename E>
+__device__ __forceinline__ void accumulate(const BwdParams<E>& p, float* acc, size_t idx, float v) {
+    if (p.fixed_point)
+        atomicAdd(reinterpret_cast<unsigned long long*>(acc) + idx, (unsigned long long)__float2ll_rn(v * kFixedScale));
+    else
+        unsafeAtomicAdd(acc + idx, v);
+}
 
 }  // namespace tritt
 
@@ -407,8 +423,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 sk += __shfl_xor(sk, 32, 64);
                 sv += __shfl_xor(sv, 32, 64);
                 if (g == 0) {
-                    unsafeAtomicAdd(p.acc_k + base + (size_t)k * D + d, sk * p.alpha);
-                    unsafeAtomicAdd(p.acc_v + base + (size_t)k * D + d, sv);
+                    accumulate(p, p.acc_k, base + (size_t)k * D + d, sk * p.alpha);
+                    accumulate(p, p.acc_v, base + (size_t)k * D + d, sv);
                 }
             }
         }
@@ -440,7 +456,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         for (int e = 0; e < 4; ++e)
             if (q0 + r0 + e < T) {
                 const size_t off = base + (size_t)(q0 + r0 + e) * D + d;
-                if (p.splits > 1) unsafeAtomicAdd(p.acc_q + off, out[e]);  // scaled by alpha when converted
+                if (p.splits > 1) accumulate(p, p.acc_q, off, out[e]);  // scaled by alpha when converted
                 else p.dq[off] = (E)(out[e] * p.alpha);
             }
     }
@@ -459,7 +475,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
                                                        float* __restrict__ delta, float* __restrict__ zero_a,
                                                        float* __restrict__ zero_b, float* __restrict__ zero_c,
                                                        float* __restrict__ zero_d, float* __restrict__ zero_e, int T,
-                                                       int Tp, int D) {
+                                                       int Tp, int D, int zero_width) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * Tp;
     // two tiles at a time (static LDS stays under 64 KB at D = 128): their loads are in flight together
@@ -476,11 +492,12 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
     __syncthreads();
     transpose_store<E>(k2t + tbase, tiles, j0, Tp, D);
     transpose_store<E>(v2t + tbase, tiles + kTile, j0, Tp, D);
+    // the accumulators: zero_width 4-byte words per row (D floats, or D 64-bit fixed-point sums)
     const float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int idx = threadIdx.x; idx < 64 * (D / 4); idx += 256) {
-        const int j = j0 + idx / (D / 4);
+    for (int idx = threadIdx.x; idx < 64 * (zero_width / 4); idx += 256) {
+        const int j = j0 + idx / (zero_width / 4);
         if (j < T) {
-            const size_t off = base + (size_t)j * D + (idx % (D / 4)) * 4;
+            const size_t off = ((size_t)bh * T + j) * zero_width + (idx % (zero_width / 4)) * 4;
             *reinterpret_cast<float4*>(zero_a + off) = z4;
             *reinterpret_cast<float4*>(zero_b + off) = z4;
             *reinterpret_cast<float4*>(zero_c + off) = z4;
@@ -514,20 +531,24 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
                                                          const float* __restrict__ dqacc, float alpha,
                                                          E* __restrict__ dq, const E* __restrict__ v1,
                                                          E* __restrict__ dk1, E* __restrict__ dv1, E* __restrict__ dk2,
-                                                         E* __restrict__ dv2, size_t n) {
+                                                         E* __restrict__ dv2, size_t n, int fixed_point) {
+    auto value = [&](const float* acc, size_t i) {
+        if (!fixed_point) return acc[i];
+        return (float)((double)reinterpret_cast<const long long*>(acc)[i] * (1.0 / (double)kFixedScale));
+    };
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        dk1[i] = (E)dk1acc[i];
-        dv1[i] = (E)(duacc[i] * silu_grad_f((float)v1[i]));
-        dk2[i] = (E)dk2acc[i];
-        dv2[i] = (E)dv2acc[i];
-        if (dqacc) dq[i] = (E)(dqacc[i] * alpha);
+        dk1[i] = (E)value(dk1acc, i);
+        dv1[i] = (E)(value(duacc, i) * silu_grad_f((float)v1[i]));
+        dk2[i] = (E)value(dk2acc, i);
+        dv2[i] = (E)value(dv2acc, i);
+        if (dqacc) dq[i] = (E)(value(dqacc, i) * alpha);
     }
 }
 
 struct BwdLayout {
     size_t u, ut, k1t, k2t, v2t, delta, dk1acc, duacc, dk2acc, dv2acc, dqacc, total;
 };
-static BwdLayout bwd_layout(int BH, int T, int D) {
+static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     const size_t Tp = (size_t)(T + 63) / 64 * 64, n = (size_t)BH * T * D;
     BwdLayout l{};
     size_t off = 0;
@@ -543,11 +564,12 @@ static BwdLayout bwd_layout(int BH, int T, int D) {
     l.k2t = take((size_t)BH * D * Tp * 2);
     l.v2t = take((size_t)BH * D * Tp * 2);
     l.delta = take((size_t)BH * T * 4);
-    l.dk1acc = take(n * 4);
-    l.duacc = take(n * 4);
-    l.dk2acc = take(n * 4);
-    l.dv2acc = take(n * 4);
-    l.dqacc = take(n * 4);  // used when the rows of a query tile are split over workgroups (small grids)
+    const size_t acc = fixed_point ? 8 : 4;
+    l.dk1acc = take(n * acc);
+    l.duacc = take(n * acc);
+    l.dk2acc = take(n * acc);
+    l.dv2acc = take(n * acc);
+    l.dqacc = take(n * acc);  // used when the rows of a query tile are split over workgroups (small grids)
     l.total = (off + 255) & ~size_t(255);
     return l;
 }
@@ -555,7 +577,7 @@ static BwdLayout bwd_layout(int BH, int T, int D) {
 template <typename E, int D>
 static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + 63) / 64 * 64;
-    const BwdLayout l = bwd_layout(a.BH, a.T, D);
+    const BwdLayout l = bwd_layout(a.BH, a.T, D, a.deterministic);
     char* ws = static_cast<char*>(a.workspace);
     const E *u = (const E*)(ws + l.u), *ut = (const E*)(ws + l.ut), *k1t = (const E*)(ws + l.k1t);
     const E *k2t = (const E*)(ws + l.k2t), *v2t = (const E*)(ws + l.v2t);
@@ -568,13 +590,14 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     const int tiles = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32);
     int splits = 1;
     if (tiles < 1024) splits = std::min(16, (1024 + tiles - 1) / tiles);
-    if (const char* v = getenv("TRITT_BWD_SPLITS")) splits = std::max(1, std::min(16, atoi(v)));  // tuning sweeps
+    if (knobs().bwd_splits > 0) splits = std::min(16, knobs().bwd_splits);  // tuning sweeps
     float* dqacc = splits > 1 ? (float*)(ws + l.dqacc) : nullptr;
 
     hipLaunchKernelGGL(bwd_prep_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (const E*)a.k1,
                        (const E*)a.k2, (const E*)a.v2, (const E*)a.o, (const E*)a.d_o, (E*)(ws + l.u),
                        (E*)(ws + l.ut), (E*)(ws + l.k1t), (E*)(ws + l.k2t), (E*)(ws + l.v2t),
-                       (float*)(ws + l.delta), dk1acc, duacc, dk2acc, dv2acc, dqacc, a.T, Tp, D);
+                       (float*)(ws + l.delta), dk1acc, duacc, dk2acc, dv2acc, dqacc, a.T, Tp, D,
+                       a.deterministic ? 2 * D : D);
 
     BwdParams<E> p;
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o;
@@ -582,7 +605,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.dq = (E*)a.dq;
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
-    p.acc_q = dqacc; p.splits = splits;
+    p.acc_q = dqacc; p.splits = splits; p.fixed_point = a.deterministic ? 1 : 0;
 
     // D = 64, full windows: three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO
     // tiles (twice: operand and epilogue layout), four dQ slices.  Otherwise: tdp_bwd_rows_general.hpp
@@ -604,12 +627,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         // Two waves per SIMD, 64 gradient columns per workgroup (S and dP computed by both column halves) is the
         // faster shape at every grid size measured, now that it fits the register file without scratch memory;
         // the one-wave-per-SIMD shape with all 128 columns stays selectable.
-        // TRITT_BWD128_VARIANT=w8 / w4 overrides the choice (read at every call).
-        bool w8 = true;
-        if (const char* v = getenv("TRITT_BWD128_VARIANT")) {
-            if (strcmp(v, "w8") == 0) w8 = true;
-            if (strcmp(v, "w4") == 0) w8 = false;
-        }
+        // TRITT_BWD128_VARIANT=w8 / w4 overrides the choice.
+        const bool w8 = knobs().bwd128_variant != 4;
         if (w8) {
             smem = bwdg_smem(128, 8, 64, true);
             kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 8, 64, false>;
@@ -627,14 +646,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         kern_dq = tdp_bwd_rows_kernel<E, 64, true>;
         kern_nodq = tdp_bwd_rows_kernel<E, 64, false>;
     }
-    {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_nodq),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return e;
-    }
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
     const int groups = (a.BH + 7) / 8;
     const dim3 grid(8 * groups * p.nqt * col_parts * p.splits);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
@@ -655,11 +668,14 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     if (gridf > 4096) gridf = 4096;
     hipLaunchKernelGGL(bwd_finish_kernel<E>, dim3((unsigned)gridf), dim3(256), 0, st, (const float*)dk1acc,
                        (const float*)duacc, (const float*)dk2acc, (const float*)dv2acc, (const float*)dqacc, a.alpha,
-                       (E*)a.dq, (const E*)a.v1, (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n);
+                       (E*)a.dq, (const E*)a.v1, (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n,
+                       a.deterministic ? 1 : 0);
     return hipGetLastError();
 }
 
-size_t mfma_tdp_bwd_workspace(int BH, int T, int D) { return bwd_layout(BH, T, D).total; }
+size_t mfma_tdp_bwd_workspace(int BH, int T, int D, bool deterministic) {
+    return bwd_layout(BH, T, D, deterministic).total;
+}
 bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
 
 hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st) {

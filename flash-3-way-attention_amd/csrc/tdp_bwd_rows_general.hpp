@@ -469,8 +469,8 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                 sk += __shfl_xor(sk, 32, 64);
                 sv += __shfl_xor(sv, 32, 64);
                 if (g == 0) {
-                    unsafeAtomicAdd(p.acc_k + base + (size_t)k * D + d, sk * p.alpha);
-                    unsafeAtomicAdd(p.acc_v + base + (size_t)k * D + d, sv);
+                    accumulate(p, p.acc_k, base + (size_t)k * D + d, sk * p.alpha);
+                    accumulate(p, p.acc_v, base + (size_t)k * D + d, sv);
                 }
             }
         }
@@ -506,7 +506,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             for (int e = 0; e < 4; ++e)
                 if (q0 + r0 + e < T) {
                     const size_t off = base + (size_t)(q0 + r0 + e) * D + d;
-                    if (p.splits > 1) unsafeAtomicAdd(p.acc_q + off, out[e]);  // scaled by alpha when converted
+                    if (p.splits > 1) accumulate(p, p.acc_q, off, out[e]);  // scaled by alpha when converted
                     else p.dq[off] = (E)(out[e] * p.alpha);
                 }
         }

@@ -776,10 +776,12 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 template <typename E>
 __global__ __launch_bounds__(256) void fwd_merge_kernel(const float* __restrict__ part, E* __restrict__ o,
                                                         float* __restrict__ lse, int rows, int D, int splits) {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    const int row = idx / D, d = idx % D;
-    if (row >= rows) return;
-    const float* src = part + (size_t)row * splits * (D + 2);
+    // 64-bit element index: rows * D can pass 2^31 (the forced-split override applies at any size)
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t row = idx / D;
+    const int d = (int)(idx % D);
+    if (row >= (size_t)rows) return;
+    const float* src = part + row * splits * (D + 2);
     float m = -INFINITY;
     for (int s = 0; s < splits; ++s) m = fmaxf(m, src[s * (D + 2) + D]);
     float l = 0.f, acc = 0.f;
@@ -790,7 +792,7 @@ __global__ __launch_bounds__(256) void fwd_merge_kernel(const float* __restrict_
         l += w * src[s * (D + 2) + D + 1];
         acc += w * src[s * (D + 2) + d];
     }
-    o[(size_t)row * D + d] = (E)(acc / l);
+    o[row * D + d] = (E)(acc / l);
     if (d == 0) lse[row] = (m + fast_log2(l)) * kLn2;
 }
 
@@ -831,15 +833,13 @@ static size_t ut_bytes(int BH, int T, int D) {
     return ((size_t)BH * D * Tp * 2 + 255) / 256 * 256;
 }
 
-// TRITT_FWD_SPLITS overrides the count (tests, tuning sweeps); read per call, so the workspace query and
-// the launch that follows it must see the same value
+// TRITT_FWD_SPLITS overrides the count (tests, tuning sweeps); read once per process (knobs())
 // The band-resident kernel takes windowed causal masks whose band fits in LDS (with room to spare for the
 // compiler's own use).  TRITT_FWD_BAND=0 switches it off (A/B runs).
 constexpr size_t kBandSmemLimit = 156 * 1024;
 static bool use_band_kernel(const MfmaFwdArgs& a) {
     if (!(a.windowed && a.causal)) return false;
-    if (const char* e = getenv("TRITT_FWD_BAND"))
-        if (atoi(e) == 0) return false;
+    if (knobs().fwd_band < 0) return false;
     const int nr = band_rows(a.k1_window, a.k2_window);
     const size_t smem = a.D == 32 ? band_smem_bytes<32>(nr) : a.D == 64 ? band_smem_bytes<64>(nr) : band_smem_bytes<128>(nr);
     return smem <= kBandSmemLimit;
@@ -862,8 +862,7 @@ static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
     const int nr = band_rows(p.wa, p.wb);
     const size_t smem = band_smem_bytes<D>(nr);
     auto kern = tdp_fwd_band_kernel<E, D>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)smem);
+    hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem);
     if (e != hipSuccess) return e;
     const int groups = (a.BH + 7) / 8;
     hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p, nr);
@@ -872,7 +871,7 @@ static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
 
 static int fwd_splits(const MfmaFwdArgs& a, int bq) {
     if (use_band_kernel(a)) return 1;
-    if (const char* e = getenv("TRITT_FWD_SPLITS")) return max(1, min(atoi(e), kMaxFwdSplits));
+    if (knobs().fwd_splits > 0) return min(knobs().fwd_splits, kMaxFwdSplits);
     const int wgs = a.BH * ((a.T + bq - 1) / bq);
     const bool banded = a.windowed && a.causal;
     // keys k the heaviest query tile walks
@@ -899,18 +898,13 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     p.part = reinterpret_cast<float*>(static_cast<char*>(a.ut) + ut_bytes(a.BH, a.T, D));
     constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS>();
     auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG>;
-    {
-        // per call: the attribute belongs to the current device, and a process may drive several
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return e;
-    }
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
     const int groups = (a.BH + 7) / 8;
     hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt * p.splits), dim3(64 * WAVES), smem, st, p);
     if (p.splits > 1) {
         const int rows = a.BH * a.T;
-        hipLaunchKernelGGL(fwd_merge_kernel<E>, dim3((rows * D + 255) / 256), dim3(256), 0, st, p.part, (E*)a.o, a.lse,
-                           rows, D, p.splits);
+        hipLaunchKernelGGL(fwd_merge_kernel<E>, dim3((unsigned)(((size_t)rows * D + 255) / 256)), dim3(256), 0, st,
+                           p.part, (E*)a.o, a.lse, rows, D, p.splits);
     }
     return hipGetLastError();
 }

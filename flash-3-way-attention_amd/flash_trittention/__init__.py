@@ -3,16 +3,17 @@
 Same public names as the reference package (src/flash_trittention/__init__.py:11-14):
 ``flash_trittention`` (triple-dot-product) and ``TrittentionTriton``
 (dot-product-sum; the name is kept so imports drop in — there is no Triton
-inside).  Imports are lazy so ``import flash_trittention`` works without a GPU.
+inside), plus ``FlashTrittentionModule``, an ``nn.Module`` front of the former.  Imports are lazy so ``import flash_trittention`` works without a GPU.
 """
 
 __version__ = "0.1.0"
 
-__all__ = ["flash_trittention", "TrittentionTriton"]
+__all__ = ["flash_trittention", "TrittentionTriton", "FlashTrittentionModule"]
 
 _LAZY = {
     "flash_trittention": (".triple_dot_product.flash_trittention", "flash_trittention"),
     "TrittentionTriton": (".dot_product_sum.trittention_triton", "TrittentionTriton"),
+    "FlashTrittentionModule": (".triple_dot_product.flash_trittention", "FlashTrittentionModule"),
 }
 
 

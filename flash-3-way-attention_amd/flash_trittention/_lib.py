@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libtrittention_hip.so")
 CSRC_DIR = os.path.join(os.path.dirname(_HERE), "csrc")
 
 TRITT_F32, TRITT_BF16, TRITT_F16 = 0, 1, 2
-FLAG_AUTO, FLAG_FORCE_GENERIC, FLAG_FORCE_MFMA = 0, 1, 2
+FLAG_AUTO, FLAG_FORCE_GENERIC, FLAG_FORCE_MFMA, FLAG_FLOAT_ATOMICS = 0, 1, 2, 4
 
 _DTYPES = {torch.float32: TRITT_F32, torch.bfloat16: TRITT_BF16, torch.float16: TRITT_F16}
 
@@ -24,6 +24,8 @@ _vp, _i, _f, _sz, _u = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_s
 _PROTOS = {
     "tritt_version": (_i, []),
     "tritt_status_string": (ctypes.c_char_p, [_i]),
+    "tritt_set_tuning": (_i, [_i, _i]),
+    "tritt_probe_mfma": (_i, [_vp, _i, _i, _vp]),
     "tritt_tdp_fwd_workspace_bytes": (_sz, [_i] * 10 + [_u]),
     "tritt_tdp_fwd": (_i, [_vp] * 7 + [_i] * 5 + [_f] + [_i] * 5 + [_vp, _sz, _u, _vp]),
     "tritt_static_scratch_bytes": (_sz, []),
@@ -63,6 +65,39 @@ def lib():
 
 def exported_symbols():
     return list(_PROTOS)
+
+
+TUNE_FWD_SPLITS, TUNE_FWD_BAND, TUNE_BWD_SPLITS, TUNE_BWD128_WAVES = 0, 1, 2, 3
+
+
+class tuning:
+    """``with _lib.tuning(_lib.TUNE_BWD_SPLITS, 4): ...`` (tests and sweeps): sets a knob of the library and
+    puts the previous value back on exit."""
+
+    def __init__(self, knob: int, value: int):
+        self.knob, self.value = knob, value
+
+    def __enter__(self):
+        self.previous = lib().tritt_set_tuning(self.knob, self.value)
+        return self
+
+    def __exit__(self, *exc):
+        lib().tritt_set_tuning(self.knob, self.previous)
+        return False
+
+
+_flagged = {}
+
+
+def flagged_subclass(cls, flags: int):
+    """A subclass of an autograd Function whose IMPL_FLAGS is `flags` (one per (class, flags), cached)."""
+    flags = int(flags)
+    if flags == cls.IMPL_FLAGS:
+        return cls
+    key = (cls, flags)
+    if key not in _flagged:
+        _flagged[key] = type(f"{cls.__name__}Flags{flags}", (cls,), {"IMPL_FLAGS": flags})
+    return _flagged[key]
 
 
 def dtype_code(dtype) -> int:

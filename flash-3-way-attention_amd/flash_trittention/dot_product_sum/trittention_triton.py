@@ -13,10 +13,16 @@ import torch
 import torch.nn as nn
 
 from .. import _lib
+from ..triple_dot_product.utils import clamp_window
 
 
 class TrittentionTritonFunction(torch.autograd.Function):
-    impl_flags = _lib.FLAG_AUTO
+    # `flags` of the C ABI; a class constant (see FlashTrittention.IMPL_FLAGS)
+    IMPL_FLAGS = _lib.FLAG_AUTO
+
+    @classmethod
+    def with_flags(cls, flags: int):
+        return _lib.flagged_subclass(cls, flags)
 
     @staticmethod
     def forward(ctx, q, k1, k2, v1, v2, causal, softmax_scale, k_diff, convert_to_float32=False,
@@ -36,8 +42,8 @@ class TrittentionTritonFunction(torch.autograd.Function):
         code = _lib.dtype_code(q.dtype)
         _lib.require_gpu(q, "TrittentionTriton")
         q, k1, k2, v1, v2 = (_lib.dense(t) for t in (q, k1, k2, v1, v2))
-        k_diff = T if k_diff is None else int(k_diff)
-        flags = TrittentionTritonFunction.impl_flags
+        k_diff = clamp_window(k_diff, T, "k_diff")
+        flags = getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
         lib = _lib.lib()
         o = torch.empty_like(q)
         m = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
@@ -86,7 +92,9 @@ class TrittentionTriton(nn.Module):
         self.convert_to_float32 = convert_to_float32
         self.input_precision = input_precision
 
+    _function = TrittentionTritonFunction
+
     def forward(self, q, k1, k2, v1, v2):
         """q, k1, k2, v1, v2: [B, N, S, D] -> (o [B, N, S, D], m [B, N, S] fp32 logsumexp)."""
-        return TrittentionTritonFunction.apply(q, k1, k2, v1, v2, self.causal, self.softmax_scale, self.k_diff,
+        return self._function.apply(q, k1, k2, v1, v2, self.causal, self.softmax_scale, self.k_diff,
                                                self.convert_to_float32, self.input_precision)

@@ -7,8 +7,10 @@ return values and ValueErrors.  The work itself is one call into the HIP
 library per direction (SiLU, Delta and SiLU' are done inside it).
 """
 import warnings
+from typing import Optional
 
 import torch
+import torch.nn as nn
 
 from .. import _lib
 from .utils import process_masking_variables
@@ -33,8 +35,14 @@ def _validate(Q, others):
 
 
 class FlashTrittention(torch.autograd.Function):
-    # set by tests/bench to pin an implementation: _lib.FLAG_AUTO / FORCE_GENERIC / FORCE_MFMA
-    impl_flags = _lib.FLAG_AUTO
+    # `flags` of the C ABI (_lib.FLAG_*).  A constant of the class, never assigned to: a caller that wants
+    # another implementation uses the subclass `with_flags(flags)` returns.
+    IMPL_FLAGS = _lib.FLAG_AUTO
+
+    @classmethod
+    def with_flags(cls, flags: int):
+        """The Function whose calls pass `flags` to the library (tests pin the fp32 or the MFMA kernels)."""
+        return _lib.flagged_subclass(cls, flags)
 
     @staticmethod
     def forward(ctx, Q, K1, K2, V1, V2, softmax_scale, kk_left, kk_right, k1_window, k2_window, causal,
@@ -45,7 +53,9 @@ class FlashTrittention(torch.autograd.Function):
         Q, K1, K2, V1, V2 = (_lib.dense(t) for t in (Q, K1, K2, V1, V2))
         k1_window, k2_window, kk_left, kk_right = process_masking_variables(T, k1_window, k2_window, kk_left, kk_right)
         causal = bool(causal)
-        flags = FlashTrittention.impl_flags
+        flags = getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
+        if torch.are_deterministic_algorithms_enabled():
+            flags &= ~_lib.FLAG_FLOAT_ATOMICS  # the default (fixed-point accumulation) is bitwise reproducible
         lib = _lib.lib()
         code = _lib.dtype_code(Q.dtype)
         O = torch.empty_like(Q)
@@ -105,3 +115,34 @@ def flash_trittention(q, k1, k2, v1, v2, softmax_scale=1 / 8, kk_left=1, kk_righ
             f"(got {input_precision!r}).", stacklevel=2)
     return FlashTrittention.apply(q, k1, k2, v1, v2, softmax_scale, kk_left, kk_right, k1_window, k2_window, causal,
                                   convert_to_float32)
+
+
+class FlashTrittentionModule(nn.Module):
+    """``nn.Module`` front of ``flash_trittention`` (the triple-dot counterpart of ``TrittentionTriton``).
+
+    The constructor takes what the reference's naive module takes
+    (triple_dot_product/trittention_pytorch.py:12-21: causal, softmax_scale, n_ctx and the four windows, ``None`` =
+    no window), so a model built on ``Trittention_pytorch`` can swap the class; ``n_ctx`` is accepted and only
+    checked (no mask is precomputed).  ``forward`` returns O [B, H, T, D] alone: the dense score and gated-value
+    tensors the naive module also returns are never formed here."""
+
+    def __init__(self, causal: bool = True, softmax_scale: float = 1 / 8, n_ctx: Optional[int] = None,
+                 k1_window: Optional[int] = None, k2_window: Optional[int] = None, kk_left: Optional[int] = None,
+                 kk_right: Optional[int] = None, convert_to_float32: bool = False):
+        super().__init__()
+        self.causal = causal
+        self.softmax_scale = softmax_scale
+        self.n_ctx = n_ctx
+        self.k1_window, self.k2_window, self.kk_left, self.kk_right = k1_window, k2_window, kk_left, kk_right
+        self.convert_to_float32 = convert_to_float32
+
+    def forward(self, q, k1, k2, v1, v2):
+        if self.n_ctx is not None and q.shape[-2] > self.n_ctx:
+            raise ValueError(f"sequence length {q.shape[-2]} exceeds n_ctx={self.n_ctx}")
+        return flash_trittention(q, k1, k2, v1, v2, softmax_scale=self.softmax_scale, kk_left=self.kk_left,
+                                 kk_right=self.kk_right, k1_window=self.k1_window, k2_window=self.k2_window,
+                                 causal=self.causal, convert_to_float32=self.convert_to_float32)
+
+    def extra_repr(self):
+        return (f"causal={self.causal}, softmax_scale={self.softmax_scale}, windows="
+                f"({self.k1_window}, {self.k2_window}, {self.kk_left}, {self.kk_right})")

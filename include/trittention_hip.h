@@ -47,13 +47,30 @@ enum {
 enum {
     TRITT_FLAG_AUTO = 0,
     TRITT_FLAG_FORCE_GENERIC = 1, /* use the fp32 VALU kernels even where an MFMA kernel exists */
-    TRITT_FLAG_FORCE_MFMA = 2     /* fail with TRITT_ERR_UNSUPPORTED instead of falling back    */
+    TRITT_FLAG_FORCE_MFMA = 2,    /* fail with TRITT_ERR_UNSUPPORTED instead of falling back    */
+    TRITT_FLAG_FLOAT_ATOMICS = 4  /* tritt_tdp_bwd, MFMA path: accumulate the shared gradients with fp32
+                                     atomics instead of 64-bit fixed point (see tritt_tdp_bwd)     */
 };
 
 /* Library version (major*10000 + minor*100 + patch) and a static, human
  * readable description of a return code. */
 int tritt_version(void);
 const char* tritt_status_string(int status);
+
+/* Tuning overrides for sweeps and tests; production callers never need them.  Each knob
+ * starts from an environment variable that is read once per process (the first time any
+ * entry point needs it), so a *_workspace_bytes query and the launch that follows always see
+ * the same value; tritt_set_tuning changes a knob afterwards and returns its previous value
+ * (TRITT_ERR_INVALID for an unknown knob).  0 = automatic.  Process-wide: do not change a knob
+ * while another thread is inside the library.
+ *   TRITT_TUNE_FWD_SPLITS   (env TRITT_FWD_SPLITS)     workgroups per query tile in the triple-dot forward, 1..8
+ *   TRITT_TUNE_FWD_BAND     (env TRITT_FWD_BAND=0)     -1: narrow windowed masks take the streaming forward
+ *                                                      instead of the band-resident one
+ *   TRITT_TUNE_BWD_SPLITS   (env TRITT_BWD_SPLITS)     workgroups per query tile in the triple-dot backward, 1..16
+ *   TRITT_TUNE_BWD128_WAVES (env TRITT_BWD128_VARIANT=w8|w4)  workgroup shape of the D = 128 backward: 8 or 4 */
+enum { TRITT_TUNE_FWD_SPLITS = 0, TRITT_TUNE_FWD_BAND = 1, TRITT_TUNE_BWD_SPLITS = 2, TRITT_TUNE_BWD128_WAVES = 3,
+       TRITT_TUNE_COUNT_ = 4 };
+int tritt_set_tuning(int knob, int value);
 
 /* ---- triple-dot-product:  s[q,j,k] = alpha * sum_d Q[q,d] K1[j,d] K2[k,d] ----------------
  * O[q] = sum_{j,k} softmax_{(j,k)}(s[q]) * SiLU(V1[j]) * V2[k].
@@ -67,8 +84,16 @@ const char* tritt_status_string(int status);
  * tritt_tdp_bwd replaces FlashTrittention.backward and its five launches
  *   (triple_dot_product/flash_trittention.py:141-393, kernels/bwd_{dq,dk1,dk2,dv1,dv2}.py),
  *   including Delta = rowsum(dO*O) and the SiLU' factor on dV1.  On the 16-bit MFMA path
- *   (16-bit tensors, D = 64 or 128, any mask) dK1/dV1/dK2/dV2 are accumulated with fp32 atomics: equal to rounding
- *   from run to run, not bitwise; dQ and every fp32-tensor result are bitwise reproducible.
+ *   (16-bit tensors, D = 32, 64 or 128, any mask) the workgroups of different query tiles add their
+ *   shares of dK1/dV1/dK2/dV2 (and of dQ, when a small grid splits a tile's rows) to common
+ *   accumulators.  The shares are added as 64-bit fixed point (steps of 2^-30, |sum| below 8.6e9)
+ *   with integer atomics, whose result does not depend on the order of arrival: like the
+ *   reference's owner-computes kernels, and like every other entry point here, the call is
+ *   bitwise reproducible from run to run (measured cost against fp32 atomics: none).
+ *   TRITT_FLAG_FLOAT_ATOMICS selects fp32 atomics instead (reproducible to rounding only; no
+ *   bound on the magnitude of the sums; accumulators half the size: pass the same flags to
+ *   tritt_tdp_bwd_workspace_bytes).  Workspace of the MFMA path: about 15 (fixed point: 25) times
+ *   one 16-bit [B,H,T,D] tensor (five accumulators, four transposed copies, SiLU(V1)).
  */
 size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
                                      int k1_window, int k2_window, int kk_left, int kk_right,
@@ -134,6 +159,13 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
                   void* dq, void* dk1, void* dk2, void* dv1, void* dv2,
                   int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
                   void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
+/* Calibration for benchmarks (no counterpart in the reference).  Launches `blocks` workgroups of
+ * eight waves that each issue iters * 4 independent 32x32x16 bf16 MFMAs and nothing else:
+ * blocks * 8 * iters * 4 * 32768 flop.  Timed by the caller, it gives the rate the matrix pipes
+ * sustain on this chip under a pure matrix load, hence the clock it holds there (rate / published
+ * peak * nominal clock).  `out` receives blocks * 512 floats (so the work cannot be optimised away). */
+int tritt_probe_mfma(float* out, int blocks, int iters, void* stream);
 
 #ifdef __cplusplus
 }

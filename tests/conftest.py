@@ -12,3 +12,20 @@ for p in (ROOT, PKG_DIR):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture
+def tune():
+    """tune(knob, value): sets a tuning knob of the library (tritt_set_tuning) for the rest of the test; every
+    knob the test touched goes back to its previous value afterwards."""
+    from flash_trittention import _lib
+
+    first = {}
+
+    def set_knob(knob, value):
+        previous = _lib.lib().tritt_set_tuning(knob, value)
+        first.setdefault(knob, previous)
+
+    yield set_knob
+    for knob, previous in first.items():
+        _lib.lib().tritt_set_tuning(knob, previous)

@@ -46,7 +46,12 @@ def main():
 
     def run(module, tag):
         leaves = [t.clone().requires_grad_(True) for t in base[:5]]
-        z = module(*leaves)[0]
+        res = module(*leaves)
+        z = res[0]
+        # the modules' auxiliary returns (pre-softmax scores, gated values, M and, for triple-dot, L): they pin
+        # the return tuples of the oracle's drop-in Trittention_pytorch classes
+        for name, t in zip(("pre", "vgated", "M", "L"), res[1:]):
+            out[f"{tag}_{name}"] = t.detach().numpy().copy()
         z.backward(base[5])
         out[tag + "_o"] = z.detach().numpy()
         for n, t in zip(("dq", "dk1", "dk2", "dv1", "dv2"), leaves):

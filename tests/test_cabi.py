@@ -100,11 +100,49 @@ def test_python_host_validation_matches_reference_errors():
         TrittentionTriton()(q, k1, k2, v1, v2)
 
 
+def test_window_arguments_are_clamped_before_they_reach_32_bit_ints():
+    """ctypes would silently wrap 2**32 to 0 (a window of zero): the host clamps to seq_len first."""
+    from flash_trittention.triple_dot_product.utils import clamp_window, process_masking_variables
+
+    assert process_masking_variables(100, None, 2**31, 2**32, 10**12) == (100, 100, 100, 100)
+    assert process_masking_variables(100, 0, 5, 99, 100) == (0, 5, 99, 100)
+    assert clamp_window(2**32 + 5, 64) == 64
+    for bad in (-1, -2**31):
+        with pytest.raises(ValueError):
+            process_masking_variables(100, bad, None, None, None)
+        with pytest.raises(ValueError):
+            clamp_window(bad, 100, "k_diff")
+
+
+def test_implementation_flags_are_class_constants():
+    """Pinning an implementation makes a subclass; the public Functions are never mutated."""
+    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTritonFunction
+    from flash_trittention.triple_dot_product.flash_trittention import FlashTrittention
+
+    for cls in (FlashTrittention, TrittentionTritonFunction):
+        forced = cls.with_flags(_lib.FLAG_FORCE_GENERIC)
+        assert forced is not cls and issubclass(forced, cls) and forced.IMPL_FLAGS == _lib.FLAG_FORCE_GENERIC
+        assert cls.with_flags(_lib.FLAG_FORCE_GENERIC) is forced and cls.with_flags(0) is cls
+        assert cls.IMPL_FLAGS == _lib.FLAG_AUTO
+
+
+def test_module_front_of_triple_dot():
+    from flash_trittention import FlashTrittentionModule
+
+    m = FlashTrittentionModule(causal=True, softmax_scale=0.25, n_ctx=16, k1_window=4)
+    assert "k1_window" not in dict(m.named_parameters()) and "windows=(4, None, None, None)" in repr(m)
+    q = torch.randn(1, 1, 32, 32)
+    with pytest.raises(ValueError, match="n_ctx"):
+        m(q, q, q, q, q)
+    with pytest.raises(RuntimeError, match="GPU"):
+        FlashTrittentionModule()(q, q, q, q, q)
+
+
 def test_lazy_package_exports():
     import flash_trittention as ft
 
-    assert ft.__all__ == ["flash_trittention", "TrittentionTriton"]
-    assert callable(ft.flash_trittention) and callable(ft.TrittentionTriton)
+    assert ft.__all__ == ["flash_trittention", "TrittentionTriton", "FlashTrittentionModule"]
+    assert callable(ft.flash_trittention) and callable(ft.TrittentionTriton) and callable(ft.FlashTrittentionModule)
     with pytest.raises(AttributeError):
         ft.nope
 

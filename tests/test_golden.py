@@ -94,3 +94,44 @@ def test_hip_dps_matches_reference_vectors(gold, i):
     np.testing.assert_allclose(out.numpy(), gold[f"dps{i}_o"], rtol=1e-4, atol=2e-5)
     for n, g in zip(NAMES, grads):
         np.testing.assert_allclose(g.numpy(), gold[f"dps{i}_{n}"], rtol=1e-4, atol=2e-5, err_msg=n)
+
+
+def _module_grads(module, ins):
+    leaves = [t.clone().requires_grad_(True) for t in ins[:5]]
+    res = module(*leaves)
+    res[0].backward(ins[5])
+    return res, [t.grad for t in leaves]
+
+
+@pytest.mark.parametrize("i", _cases("tdp"))
+def test_naive_module_tdp_returns_match_reference_vectors(gold, i):
+    """The drop-in Trittention_pytorch class (triple-dot): all five returns and the autograd gradients."""
+    from oracle.triple_dot_product.trittention_pytorch import Trittention_pytorch
+
+    cfg = gold[f"tdp{i}_cfg"]
+    wins = [_win(v) for v in cfg[1:]]
+    m = Trittention_pytorch(causal=bool(cfg[0]), softmax_scale=float(gold["alpha"]), n_ctx=16, k1_window=wins[0],
+                            k2_window=wins[1], kk_left=wins[2], kk_right=wins[3])
+    (z, pre, vg, M, L), grads = _module_grads(m, _inputs(gold, torch.float64))
+    np.testing.assert_allclose(z.detach().numpy(), gold[f"tdp{i}_o"], rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(pre.detach().numpy(), gold[f"tdp{i}_pre"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(vg.detach().numpy(), gold[f"tdp{i}_vgated"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(M.detach().numpy(), gold[f"tdp{i}_M"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(L.detach().numpy(), gold[f"tdp{i}_L"], rtol=1e-11, atol=1e-12)
+    for n, g in zip(NAMES, grads):
+        np.testing.assert_allclose(g.numpy(), gold[f"tdp{i}_{n}"], rtol=1e-8, atol=1e-10, err_msg=n)
+
+
+@pytest.mark.parametrize("i", _cases("dps"))
+def test_naive_module_dps_returns_match_reference_vectors(gold, i):
+    from oracle.dot_product_sum.trittention_pytorch import Trittention_pytorch
+
+    m = Trittention_pytorch(causal=bool(gold[f"dps{i}_cfg"][0]), softmax_scale=float(gold["alpha"]), n_ctx=16,
+                            k_diff=int(gold[f"dps{i}_cfg"][1]))
+    (z, pre, vg, M), grads = _module_grads(m, _inputs(gold, torch.float64))
+    np.testing.assert_allclose(z.detach().numpy(), gold[f"dps{i}_o"], rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(pre.detach().numpy(), gold[f"dps{i}_pre"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(vg.detach().numpy(), gold[f"dps{i}_vgated"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(M.detach().numpy(), gold[f"dps{i}_M"], rtol=1e-11, atol=1e-12)
+    for n, g in zip(NAMES, grads):
+        np.testing.assert_allclose(g.numpy(), gold[f"dps{i}_{n}"], rtol=1e-8, atol=1e-10, err_msg=n)

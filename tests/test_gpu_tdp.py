@@ -10,6 +10,7 @@ import pytest
 import torch
 
 from oracle import trittention_oracle as orc
+from flash_trittention import _lib
 from tests import util
 
 pytestmark = pytest.mark.gpu
@@ -91,29 +92,64 @@ def test_lse_matches_oracle():
     util.assert_close("lse", ctx.saved[6].cpu(), lse, rtol=1e-5, atol=1e-5)
 
 
-def test_reproducible(monkeypatch):
-    """Forward and (one workgroup per query tile) dQ have a single owner per element and a fixed summation
-    order: bitwise equal from run to run.  dK1/dV1/dK2/dV2 of the MFMA path are summed over query tiles with
-    fp32 atomics, and so is dQ when a small grid deals the rows of a tile out to several workgroups: those are
-    reproducible to rounding only.  The fp32 VALU path is bitwise reproducible throughout."""
+def test_reproducible(tune):
+    """Every result is bitwise equal from run to run: the forward and (one workgroup per query tile) dQ have a
+    single owner per element and a fixed summation order; dK1/dV1/dK2/dV2 of the MFMA path are summed over
+    query tiles, and so is dQ when a small grid deals the rows of a tile out to several workgroups, in 64-bit
+    fixed point with integer atomics, whose sum does not depend on the order of arrival.  The fp32 VALU path
+    has one owner per element throughout."""
     inputs = orc.make_inputs(1, 2, 96, 64, torch.bfloat16, seed=5)
-    monkeypatch.setenv("TRITT_BWD_SPLITS", "1")
+    tune(_lib.TUNE_BWD_SPLITS, 1)
     a = util.run_tdp(inputs, 1 / 8, True)
     b = util.run_tdp(inputs, 1 / 8, True)
     assert torch.equal(a[0], b[0])
-    assert torch.equal(a[1][0], b[1][0]), "dq"
-    for i in (1, 2, 3, 4):
-        util.assert_close(util.NAMES[i], a[1][i], b[1][i], rtol=1e-2, atol=1e-2)
-    monkeypatch.delenv("TRITT_BWD_SPLITS")
-    e = util.run_tdp(inputs, 1 / 8, True)  # this grid is small: rows split, dQ accumulated atomically
+    for i in range(5):
+        assert torch.equal(a[1][i], b[1][i]), util.NAMES[i]
+    tune(_lib.TUNE_BWD_SPLITS, 0)
+    e = util.run_tdp(inputs, 1 / 8, True)  # this grid is small: rows split, dQ accumulated too
+    f = util.run_tdp(inputs, 1 / 8, True)
     assert torch.equal(a[0], e[0])
     for i in range(5):
+        assert torch.equal(e[1][i], f[1][i]), util.NAMES[i]
         util.assert_close(util.NAMES[i], a[1][i], e[1][i], rtol=1e-2, atol=1e-2)
     c = util.run_tdp(inputs, 1 / 8, True, flags=1)
     d = util.run_tdp(inputs, 1 / 8, True, flags=1)
     assert torch.equal(c[0], d[0])
     for x, y in zip(c[1], d[1]):
         assert torch.equal(x, y)
+
+
+FLOAT_ATOMICS = _lib.FLAG_FLOAT_ATOMICS
+
+
+@pytest.mark.parametrize("shape", [(2, 4, 256, 64), (4, 8, 1024, 64), (1, 3, 203, 128), (1, 3, 203, 32)])
+def test_backward_is_bitwise_reproducible(shape):
+    """The shares of the row gradients (and of a split dQ) are added as 64-bit fixed point with integer atomics,
+    so two runs agree bit for bit in all five gradients whatever order the workgroups arrive in: BASELINE
+    configs 2 (a small grid: rows split, dQ accumulated too) and 3, and the general kernel (D = 128, D = 32,
+    ragged length).  With TRITT_FLAG_FLOAT_ATOMICS (fp32 atomics) the results differ from these by rounding."""
+    print(f"case reproducible {shape}", flush=True)
+    B, H, T, D = shape
+    inputs = orc.make_inputs(B, H, T, D, torch.bfloat16, seed=T + D)
+    alpha = 1 / math.sqrt(D)
+    out_a, a = util.run_tdp(inputs, alpha, True)
+    out_b, b = util.run_tdp(inputs, alpha, True)
+    assert torch.equal(out_a, out_b)
+    for name, x, y in zip(util.NAMES, a, b):
+        assert torch.equal(x, y), name
+    _, c = util.run_tdp(inputs, alpha, True, flags=FLOAT_ATOMICS)
+    for name, x, y in zip(util.NAMES, a, c):
+        util.assert_close(name, x, y, rtol=1e-2, atol=1e-2)
+
+
+def test_float_atomics_flag_config2_against_oracle():
+    inputs = orc.make_inputs(2, 4, 256, 64, torch.bfloat16, seed=2)
+    z, lse, grads = util.oracle_tdp(inputs, 1 / 8, True)
+    out, g = util.run_tdp(inputs, 1 / 8, True, flags=FLOAT_ATOMICS)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_close(name, a, b, **LOWP)
+        assert util.rel_err(a, b) <= 2e-2, (name, util.rel_err(a, b))
 
 
 def test_non_contiguous_inputs():
@@ -378,11 +414,11 @@ def test_mfma_backward_bf16(seq_len, causal):
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("seq_len", [1, 33, 100, 256, 300])
 @pytest.mark.parametrize("shape", ["w4", "w8"])
-def test_mfma_backward_d128_bf16(seq_len, causal, shape, monkeypatch):
+def test_mfma_backward_d128_bf16(seq_len, causal, shape, tune):
     """Head dimension 128, both workgroup shapes of the backward kernel (one wave per SIMD with all
     128 gradient columns / two waves per SIMD with one half of them)."""
     print(f"case mfma bwd D=128 T={seq_len} causal={causal} shape={shape}", flush=True)
-    monkeypatch.setenv("TRITT_BWD128_VARIANT", shape)
+    tune(_lib.TUNE_BWD128_WAVES, int(shape[1]))
     inputs = orc.make_inputs(1, 3, seq_len, 128, torch.bfloat16, seed=seq_len + 7)
     alpha = 1 / math.sqrt(128)
     z, _, grads = util.oracle_tdp(inputs, alpha, causal)
@@ -427,10 +463,10 @@ def test_mfma_windows_fp16_batched(D):
 
 @pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("splits", [2, 5, 16])
-def test_mfma_backward_row_splits(splits, D, monkeypatch):
+def test_mfma_backward_row_splits(splits, D, tune):
     """The rows of a query tile dealt out to several workgroups (what small grids get): dQ then goes
     through an fp32 accumulator like the row gradients.  Windowed and full masks, ragged length."""
-    monkeypatch.setenv("TRITT_BWD_SPLITS", str(splits))
+    tune(_lib.TUNE_BWD_SPLITS, splits)
     alpha = 1 / math.sqrt(D)
     for windows in ((None,) * 4, (40, 100, 20, 7)):
         inputs = orc.make_inputs(1, 3, 203, D, torch.bfloat16, seed=splits + D)
@@ -444,11 +480,11 @@ def test_mfma_backward_row_splits(splits, D, monkeypatch):
 
 @pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("splits", [2, 3, 8])
-def test_mfma_forward_k_splits(splits, D, monkeypatch):
+def test_mfma_forward_k_splits(splits, D, tune):
     """The k-tiles of a query tile dealt out to several workgroups and joined by the merge kernel (what
     small grids get): full, non-causal and windowed masks at a ragged length.  Parts with no k-tile at all
     (early query tiles) must drop out of the merge.  The backward reads the merged log-sum-exp."""
-    monkeypatch.setenv("TRITT_FWD_SPLITS", str(splits))
+    tune(_lib.TUNE_FWD_SPLITS, splits)
     alpha = 1 / math.sqrt(D)
     inputs = orc.make_inputs(1, 3, 203, D, torch.bfloat16, seed=splits + D)
     for causal, windows in ((True, (None,) * 4), (False, (None,) * 4), (True, (40, 100, 20, 7))):
@@ -460,7 +496,7 @@ def test_mfma_forward_k_splits(splits, D, monkeypatch):
 
 
 @pytest.mark.parametrize("splits", [1, 4])
-def test_mfma_forward_k_splits_large_logits(splits, monkeypatch):
+def test_mfma_forward_k_splits_large_logits(splits, tune):
     """Scores spanning hundreds with the k-tiles split: every part goes through the repeat sweep with its own
     reference maximum, and the merge must bring them to a common one.  Same statistical bound as the
     unsplit large-logit case; split and unsplit runs must agree far more closely than either does with the
@@ -469,9 +505,9 @@ def test_mfma_forward_k_splits_large_logits(splits, monkeypatch):
     inputs[1] = (inputs[1].float() * 6).bfloat16()
     inputs[2] = (inputs[2].float() * 6).bfloat16()
     z, _, _ = util.oracle_tdp(inputs, 1 / 8, True)
-    monkeypatch.setenv("TRITT_FWD_SPLITS", "1")
+    tune(_lib.TUNE_FWD_SPLITS, 1)
     whole, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
-    monkeypatch.setenv("TRITT_FWD_SPLITS", str(splits))
+    tune(_lib.TUNE_FWD_SPLITS, splits)
     out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False, flags=FORCE_MFMA)
     assert torch.isfinite(out).all()
     err = (out - z).abs()
@@ -499,7 +535,7 @@ def test_small_grid_forward_splits_by_itself():
 @pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("windows", [(128, 128, 32, 32), (64, 64, 16, 16), (32, 90, 8, 60), (90, 32, 33, 0), (17, 5, 40, 40),
                                      (3, 100, 1, 2)])
-def test_band_resident_forward_matches_streaming_and_oracle(windows, D, monkeypatch):
+def test_band_resident_forward_matches_streaming_and_oracle(windows, D, tune):
     """Narrow windows take the band-resident forward (the whole band of a 32-query tile in LDS); switched off,
     the streaming windowed kernel takes the same problem.  Both against the oracle, and against each other
     far more tightly (they round the same products).  T = 333: eleven query tiles, the last one ragged;
@@ -508,7 +544,7 @@ def test_band_resident_forward_matches_streaming_and_oracle(windows, D, monkeypa
     inputs = orc.make_inputs(1, 2, 333, D, torch.bfloat16, seed=D + windows[0])
     z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
     out, g = util.run_tdp(inputs, alpha, True, windows, flags=FORCE_MFMA)
-    monkeypatch.setenv("TRITT_FWD_BAND", "0")
+    tune(_lib.TUNE_FWD_BAND, -1)
     ref, _ = util.run_tdp(inputs, alpha, True, windows, backward=False, flags=FORCE_MFMA)
     util.assert_close("out", out, z, **LOWP)
     util.assert_close("out vs streaming", out, ref, rtol=1e-2, atol=4e-3)
@@ -572,8 +608,7 @@ def test_forward_and_backward_replay_from_a_hip_graph(shape):
     """The library only launches kernels on the stream it is given (no allocation, copy, memset or
     synchronisation inside), so a forward + backward can be captured into a HIP graph once and replayed for
     launch-bound small problems.  Three replays on fresh inputs, with eager work and synchronisations in between,
-    each against the eager result of the same inputs: bitwise for O, to rounding for the gradients
-    (atomically accumulated)."""
+    each against the eager result of the same inputs, bit for bit (O and all five gradients)."""
     from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
 
     B, H, T, D, windows = shape
@@ -611,7 +646,7 @@ def test_forward_and_backward_replay_from_a_hip_graph(shape):
         torch.cuda.synchronize()
         assert torch.equal(got_out, e_out), rep
         for name, a, b in zip(util.NAMES, got_grads, e_grads):
-            util.assert_close(f"{name} replay {rep}", a.float().cpu(), b.float().cpu(), rtol=2e-2, atol=2e-2)
+            assert torch.equal(a, b), f"{name} replay {rep}"
         z, _, ref = util.oracle_tdp(fresh, alpha, True, windows)
         util.assert_close("out vs oracle", got_out.float().cpu(), z, **LOWP)
 
@@ -700,8 +735,8 @@ def _headline_inputs(seed=5):
 
 
 def test_config3_heads_are_independent_and_order_free():
-    """Permuting the (batch, head) slices permutes outputs and gradients bit for bit in the forward and
-    in dQ (owner-computes), and to rounding in the atomically accumulated gradients."""
+    """Permuting the (batch, head) slices permutes outputs and all five gradients bit for bit (one owner per
+    element, or order-independent fixed-point accumulation)."""
     inputs = _headline_inputs()
     out, g = util.run_tdp(inputs, 1 / 8, True)
     perm = torch.randperm(32, generator=torch.Generator().manual_seed(1))
@@ -709,9 +744,8 @@ def test_config3_heads_are_independent_and_order_free():
     out2, g2 = util.run_tdp(shuffled, 1 / 8, True)
     unperm = lambda t: t.reshape(32, 1024, 64)[torch.argsort(perm)].reshape(4, 8, 1024, 64)
     assert torch.equal(unperm(out2), out)
-    assert torch.equal(unperm(g2[0]), g[0])
-    for name, a, b in zip(util.NAMES[1:], g[1:], g2[1:]):
-        util.assert_close(name, unperm(b), a, rtol=2e-2, atol=2e-3)
+    for name, a, b in zip(util.NAMES, g, g2):
+        assert torch.equal(unperm(b), a), name
 
 
 def test_config3_linear_in_v2_and_do():

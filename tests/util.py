@@ -44,11 +44,11 @@ def oracle_dps(inputs, alpha, causal, k_diff, factorised=False):
 def run_tdp(inputs, alpha, causal, windows=(None,) * 4, backward=True, device="cuda", flags=0):
     from flash_trittention.triple_dot_product.flash_trittention import FlashTrittention, flash_trittention
 
-    FlashTrittention.impl_flags = flags
-    try:
-        return _run_tdp(flash_trittention, inputs, alpha, causal, windows, backward, device)
-    finally:
-        FlashTrittention.impl_flags = 0
+    if flags:
+        fn = FlashTrittention.with_flags(flags)
+        flash_trittention = lambda q, k1, k2, v1, v2, softmax_scale, k1_window, k2_window, kk_left, kk_right, causal: \
+            fn.apply(q, k1, k2, v1, v2, softmax_scale, kk_left, kk_right, k1_window, k2_window, causal, False)
+    return _run_tdp(flash_trittention, inputs, alpha, causal, windows, backward, device)
 
 
 def _run_tdp(flash_trittention, inputs, alpha, causal, windows, backward, device):
@@ -68,19 +68,13 @@ def _run_tdp(flash_trittention, inputs, alpha, causal, windows, backward, device
 def run_dps(inputs, alpha, causal, k_diff, backward=True, device="cuda", flags=0):
     from flash_trittention.dot_product_sum.trittention_triton import TrittentionTritonFunction
 
-    TrittentionTritonFunction.impl_flags = flags
-    try:
-        return _run_dps(inputs, alpha, causal, k_diff, backward, device)
-    finally:
-        TrittentionTritonFunction.impl_flags = 0
+    return _run_dps(inputs, alpha, causal, k_diff, backward, device, TrittentionTritonFunction.with_flags(flags))
 
 
-def _run_dps(inputs, alpha, causal, k_diff, backward, device):
-    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
-
+def _run_dps(inputs, alpha, causal, k_diff, backward, device, function):
     q, k1, k2, v1, v2, do = (t.to(device) for t in inputs)
     leaves = [t.detach().clone().requires_grad_(backward) for t in (q, k1, k2, v1, v2)]
-    out, m = TrittentionTriton(causal=causal, softmax_scale=alpha, k_diff=k_diff)(*leaves)
+    out, m = function.apply(*leaves, causal, alpha, k_diff)
     grads = None
     if backward:
         out.backward(do)
