@@ -219,28 +219,41 @@ int tdp_bwd_generic(Arena& ar, bool run, const void* q, const void* k1, const vo
     float* do32 = dtype == TRITT_F32 ? (float*)d_o : ar.take<float>(n);
     float* delta = ar.take<float>((size_t)B * H * T);
     float* du = ar.take<float>(n);
+    // fp32 results: the caller's tensors when they are fp32, scratch otherwise; `spare` stands in for the
+    // unwanted (null) half of a gradient pair whose other half is wanted (one kernel writes both halves)
     float *dq32 = (float*)dq, *dk132 = (float*)dk1, *dk232 = (float*)dk2, *dv232 = (float*)dv2;
+    float* spare = nullptr;
     if (dtype != TRITT_F32) {
         dq32 = ar.take<float>(n); dk132 = ar.take<float>(n); dk232 = ar.take<float>(n); dv232 = ar.take<float>(n);
+    } else {
+        spare = ar.take<float>(n);
     }
     if (!run) return TRITT_OK;
+    const bool want_k2 = dk2 || dv2, want_k1 = dk1 || dv1;
+    if (dtype == TRITT_F32) {
+        if (want_k2 && !dk2) dk232 = spare;
+        if (want_k2 && !dv2) dv232 = spare;
+        if (want_k1 && !dk1) dk132 = spare;
+    }
     fill_inputs(q, k1, k2, v1, v2, n, dtype, copies, u, st);
     if (dtype != TRITT_F32) to_f32<false>(d_o, do32, n, dtype, st);
     rowdot(d_o, o, delta, B * H * T, D, dtype, st);
     GenericTdpArgs a{};
     a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
     a.lse_in = lse; a.d_o = do32; a.delta = delta;
-    a.dq = dq32; a.dk1 = dk132; a.dk2 = dk232; a.du = du; a.dv2 = dv232;
+    a.dq = dq ? dq32 : nullptr;
+    a.dk2 = want_k2 ? dk232 : nullptr; a.dv2 = want_k2 ? dv232 : nullptr;
+    a.dk1 = want_k1 ? dk132 : nullptr; a.du = want_k1 ? du : nullptr;
     a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha;
     a.causal = causal; a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
     hipError_t e = generic_tdp_bwd(a, st);
     if (e != hipSuccess) return (int)e;
-    from_f32(du, v1, dv1, n, dtype, st);
+    if (dv1) from_f32(du, v1, dv1, n, dtype, st);
     if (dtype != TRITT_F32) {
-        from_f32(dq32, nullptr, dq, n, dtype, st);
-        from_f32(dk132, nullptr, dk1, n, dtype, st);
-        from_f32(dk232, nullptr, dk2, n, dtype, st);
-        from_f32(dv232, nullptr, dv2, n, dtype, st);
+        if (dq) from_f32(dq32, nullptr, dq, n, dtype, st);
+        if (dk1) from_f32(dk132, nullptr, dk1, n, dtype, st);
+        if (dk2) from_f32(dk232, nullptr, dk2, n, dtype, st);
+        if (dv2) from_f32(dv232, nullptr, dv2, n, dtype, st);
     }
     return (int)hipGetLastError();
 }
@@ -485,8 +498,9 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
     if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
     int rc = check_common(B, H, T, D, dtype);
     if (rc != TRITT_OK) return rc;
-    if (any_null({q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
-    if (any_misaligned({q, k1, k2, v1, v2, o, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
+    if (any_null({q, k1, k2, v1, v2, o, lse, d_o})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o, d_o, dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;  // null is aligned
+    if (!dq && !dk1 && !dk2 && !dv1 && !dv2) return TRITT_OK;  // no gradient wanted
     if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
     const bool mfma = use_mfma_bwd(T, D, dtype, causal, w1, w2, kl, kr, flags);

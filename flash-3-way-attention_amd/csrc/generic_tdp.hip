@@ -343,12 +343,16 @@ static hipError_t launch_bwd(const GenericTdpArgs& a, hipStream_t st) {
     TdpMask m{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
     // transposed roles: staged = k (K2/V2), owner = j (K1/U)
     TdpMask mt{a.causal, a.k2_window, a.k1_window, a.kk_right, a.kk_left};
-    hipLaunchKernelGGL(tdp_bwd_q_generic_kernel<D>, grid, dim3(256), 0, st, a.q, a.k1, a.k2, a.u, a.v2,
-                       a.d_o, a.lse_in, a.delta, a.dq, a.T, a.alpha, m);
-    hipLaunchKernelGGL(tdp_bwd_b_generic_kernel<D>, grid, dim3(256), 0, st, a.q, a.k1, a.k2, a.u, a.v2,
-                       a.d_o, a.lse_in, a.delta, a.dk2, a.dv2, a.T, a.alpha, m);
-    hipLaunchKernelGGL(tdp_bwd_b_generic_kernel<D>, grid, dim3(256), 0, st, a.q, a.k2, a.k1, a.v2, a.u,
-                       a.d_o, a.lse_in, a.delta, a.dk1, a.du, a.T, a.alpha, mt);
+    // a null output pair is a launch the caller does not want
+    if (a.dq)
+        hipLaunchKernelGGL(tdp_bwd_q_generic_kernel<D>, grid, dim3(256), 0, st, a.q, a.k1, a.k2, a.u, a.v2,
+                           a.d_o, a.lse_in, a.delta, a.dq, a.T, a.alpha, m);
+    if (a.dk2 && a.dv2)
+        hipLaunchKernelGGL(tdp_bwd_b_generic_kernel<D>, grid, dim3(256), 0, st, a.q, a.k1, a.k2, a.u, a.v2,
+                           a.d_o, a.lse_in, a.delta, a.dk2, a.dv2, a.T, a.alpha, m);
+    if (a.dk1 && a.du)
+        hipLaunchKernelGGL(tdp_bwd_b_generic_kernel<D>, grid, dim3(256), 0, st, a.q, a.k2, a.k1, a.v2, a.u,
+                           a.d_o, a.lse_in, a.delta, a.dk1, a.du, a.T, a.alpha, mt);
     return hipGetLastError();
 }
 

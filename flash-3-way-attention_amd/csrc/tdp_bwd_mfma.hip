@@ -536,12 +536,13 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
         if (!fixed_point) return acc[i];
         return (float)((double)reinterpret_cast<const long long*>(acc)[i] * (1.0 / (double)kFixedScale));
     };
+    // a null output is a gradient the caller does not want
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        dk1[i] = (E)value(dk1acc, i);
-        dv1[i] = (E)(value(duacc, i) * silu_grad_f((float)v1[i]));
-        dk2[i] = (E)value(dk2acc, i);
-        dv2[i] = (E)value(dv2acc, i);
-        if (dqacc) dq[i] = (E)(value(dqacc, i) * alpha);
+        if (dk1) dk1[i] = (E)value(dk1acc, i);
+        if (dv1) dv1[i] = (E)(value(duacc, i) * silu_grad_f((float)v1[i]));
+        if (dk2) dk2[i] = (E)value(dk2acc, i);
+        if (dv2) dv2[i] = (E)value(dv2acc, i);
+        if (dqacc && dq) dq[i] = (E)(value(dqacc, i) * alpha);
     }
 }
 
@@ -655,13 +656,16 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
     p.acc_k = dk2acc; p.acc_v = dv2acc;
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
-    hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
+    // a launch whose gradients the caller does not want (null outputs) is skipped
+    const bool want_q = a.dq != nullptr, want_k2 = a.dk2 || a.dv2, want_k1 = a.dk1 || a.dv1;
+    if (want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
+    else if (want_k2) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU
     p.row_k = (const E*)a.k1; p.row_v = u;
     p.st_k = (const E*)a.k2; p.st_v = (const E*)a.v2; p.st_kt = k2t; p.st_vt = v2t;
     p.acc_k = dk1acc; p.acc_v = duacc;
     p.wa = a.k2_window; p.wb = a.k1_window; p.lab = a.kk_right; p.rab = a.kk_left;  // the mask with j and k exchanged
-    hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
+    if (want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
 
     const size_t n = (size_t)a.BH * a.T * D;
     size_t gridf = (n + 255) / 256;

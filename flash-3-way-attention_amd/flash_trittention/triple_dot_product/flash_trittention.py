@@ -86,14 +86,19 @@ class FlashTrittention(torch.autograd.Function):
         k1_window, k2_window, kk_left, kk_right = ctx.windows
         lib = _lib.lib()
         code = _lib.dtype_code(Q.dtype)
-        dq, dk1, dk2, dv1, dv2 = (torch.empty_like(Q) for _ in range(5))
+        # only the gradients autograd asks for: a null pointer tells the library to skip one (and the kernel launch
+        # that serves nothing else)
+        wanted = list(getattr(ctx, "needs_input_grad", (True,) * 5)[:5])
+        grads = [torch.empty_like(Q) if w else None for w in wanted]
+        dq, dk1, dk2, dv1, dv2 = grads
+        gptr = lambda t: _lib.ptr(t) if t is not None else None
         with torch.cuda.device(Q.device):
             need = lib.tritt_tdp_bwd_workspace_bytes(B, H, T, D, code, int(ctx.causal), k1_window, k2_window, kk_left,
                                                      kk_right, ctx.flags)
             ws = _lib.workspace(need, Q.device)
             st = lib.tritt_tdp_bwd(_lib.ptr(Q), _lib.ptr(K1), _lib.ptr(K2), _lib.ptr(V1), _lib.ptr(V2), _lib.ptr(O),
-                                   _lib.ptr(LSE), _lib.ptr(dO), _lib.ptr(dq), _lib.ptr(dk1), _lib.ptr(dk2),
-                                   _lib.ptr(dv1), _lib.ptr(dv2), B, H, T, D, code, ctx.softmax_scale, int(ctx.causal),
+                                   _lib.ptr(LSE), _lib.ptr(dO), gptr(dq), gptr(dk1), gptr(dk2),
+                                   gptr(dv1), gptr(dv2), B, H, T, D, code, ctx.softmax_scale, int(ctx.causal),
                                    k1_window, k2_window, kk_left, kk_right, _lib.ptr(ws), ws.numel(), ctx.flags,
                                    _lib.stream_ptr(Q.device))
         _lib.check(st, "tritt_tdp_bwd")

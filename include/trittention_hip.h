@@ -83,7 +83,10 @@ int tritt_set_tuning(int knob, int value);
  *   applies SiLU to V1 itself and writes the final lse (the reference's M + log L).
  * tritt_tdp_bwd replaces FlashTrittention.backward and its five launches
  *   (triple_dot_product/flash_trittention.py:141-393, kernels/bwd_{dq,dk1,dk2,dv1,dv2}.py),
- *   including Delta = rowsum(dO*O) and the SiLU' factor on dV1.  On the 16-bit MFMA path
+ *   including Delta = rowsum(dO*O) and the SiLU' factor on dV1.  Any of dq, dk1, dk2, dv1, dv2 may
+ *   be NULL: that gradient is not wanted, and a kernel launch that only serves unwanted gradients
+ *   is skipped (the launches produce {dq, dk2, dv2} and {dk1, dv1}; the fp32 kernels {dq},
+ *   {dk2, dv2} and {dk1, dv1}).  On the 16-bit MFMA path
  *   (16-bit tensors, D = 32, 64 or 128, any mask) the workgroups of different query tiles add their
  *   shares of dK1/dV1/dK2/dV2 (and of dQ, when a small grid splits a tile's rows) to common
  *   accumulators.  The shares are added as 64-bit fixed point (steps of 2^-30, |sum| below 8.6e9)

@@ -152,6 +152,26 @@ def test_float_atomics_flag_config2_against_oracle():
         assert util.rel_err(a, b) <= 2e-2, (name, util.rel_err(a, b))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_only_the_requested_gradients_are_computed(dtype):
+    """Inputs that do not require a gradient get none (a null pointer at the C ABI; launches that serve only
+    unwanted gradients are skipped); the requested ones equal those of a run that asks for all five, bit for bit."""
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    inputs = [t.cuda() for t in orc.make_inputs(1, 2, 150, 64, dtype, seed=12)]
+    kw = dict(softmax_scale=1 / 8, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True)
+    full = [t.clone().requires_grad_(True) for t in inputs[:5]]
+    flash_trittention(*full, **kw).backward(inputs[5])
+    for wanted in ((0,), (1, 3), (2,), (4,), (0, 1), (3, 4)):
+        leaves = [t.clone().requires_grad_(i in wanted) for i, t in enumerate(inputs[:5])]
+        flash_trittention(*leaves, **kw).backward(inputs[5])
+        for i, (a, b) in enumerate(zip(leaves, full)):
+            if i in wanted:
+                assert torch.equal(a.grad, b.grad), (wanted, util.NAMES[i])
+            else:
+                assert a.grad is None, (wanted, util.NAMES[i])
+
+
 def test_non_contiguous_inputs():
     g = torch.Generator().manual_seed(11)
     q, v1, v2, do = (torch.randn(2, 4, 64, 32, generator=g) for _ in range(4))
