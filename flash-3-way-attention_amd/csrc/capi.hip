@@ -30,7 +30,8 @@ void init_knobs() {
 Knobs knobs() {
     init_knobs();
     return Knobs{g_knobs[TRITT_TUNE_FWD_SPLITS].load(), g_knobs[TRITT_TUNE_FWD_BAND].load(),
-                 g_knobs[TRITT_TUNE_BWD_SPLITS].load(), g_knobs[TRITT_TUNE_BWD128_WAVES].load()};
+                 g_knobs[TRITT_TUNE_BWD_SPLITS].load(), g_knobs[TRITT_TUNE_BWD128_WAVES].load(),
+                 g_knobs[TRITT_TUNE_F32_VALU].load()};
 }
 
 hipError_t ensure_dynamic_smem(const void* kernel, size_t bytes) {
@@ -188,6 +189,13 @@ void fill_inputs(const void* q, const void* k1, const void* k2, const void* v1, 
 
 int clampw(int w, int T) { return w > T ? T : w; }
 
+// The fp32 path has two sets of kernels: on the matrix cores (v_mfma_f32_32x32x2_f32; a workgroup per 32 queries)
+// and on the vector ALUs (a wave per query: far more workgroups, the better shape for problems of a few tiles).
+bool use_f32_mfma(int BH, int T) {
+    if (knobs().f32_valu) return false;
+    return (long long)BH * ((T + 31) / 32) >= 64;
+}
+
 // ---------------------------------------------------------------- triple-dot, fp32 VALU path
 int tdp_fwd_generic(Arena& ar, bool run, const void* q, const void* k1, const void* k2, const void* v1,
                     const void* v2, void* o, float* lse, int B, int H, int T, int D, int dtype, float alpha,
@@ -203,7 +211,8 @@ int tdp_fwd_generic(Arena& ar, bool run, const void* q, const void* k1, const vo
     a.o = o32; a.lse = lse;
     a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha;
     a.causal = causal; a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
-    hipError_t e = generic_tdp_fwd(a, st);
+    // fp32 on the matrix cores where a kernel exists (D = 32, 64), fp32 VALU kernels otherwise
+    hipError_t e = (f32_mfma_tdp_supported(D) && use_f32_mfma(B * H, T)) ? f32_mfma_tdp_fwd(a, st) : generic_tdp_fwd(a, st);
     if (e != hipSuccess) return (int)e;
     if (dtype != TRITT_F32) from_f32(o32, nullptr, o, n, dtype, st);
     return (int)hipGetLastError();
@@ -228,6 +237,12 @@ int tdp_bwd_generic(Arena& ar, bool run, const void* q, const void* k1, const vo
     } else {
         spare = ar.take<float>(n);
     }
+    long long* fixed = f32_mfma_tdp_supported(D) ? ar.take<long long>(f32_mfma_tdp_bwd_scratch_elems(B * H, T, D)) : nullptr;
+    // 16-bit tensors on the fp32 path: the output and the log-sum-exp are formed once more in fp32, because Delta =
+    // rowsum(dO * O) from the stored 16-bit output carries that output's rounding, which nearly one-hot softmax
+    // rows (large scores, first causal rows) turn into gradient errors far above it
+    float* o32 = dtype != TRITT_F32 ? ar.take<float>(n) : nullptr;
+    float* lse32 = dtype != TRITT_F32 ? ar.take<float>((size_t)B * H * T) : nullptr;
     if (!run) return TRITT_OK;
     const bool want_k2 = dk2 || dv2, want_k1 = dk1 || dv1;
     if (dtype == TRITT_F32) {
@@ -237,16 +252,25 @@ int tdp_bwd_generic(Arena& ar, bool run, const void* q, const void* k1, const vo
     }
     fill_inputs(q, k1, k2, v1, v2, n, dtype, copies, u, st);
     if (dtype != TRITT_F32) to_f32<false>(d_o, do32, n, dtype, st);
-    rowdot(d_o, o, delta, B * H * T, D, dtype, st);
     GenericTdpArgs a{};
     a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
+    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha;
+    a.causal = causal; a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+    const bool mfma32 = fixed && use_f32_mfma(B * H, T);
+    if (o32) {
+        a.o = o32; a.lse = lse32;
+        hipError_t ef = mfma32 ? f32_mfma_tdp_fwd(a, st) : generic_tdp_fwd(a, st);
+        if (ef != hipSuccess) return (int)ef;
+        rowdot(do32, o32, delta, B * H * T, D, TRITT_F32, st);
+        lse = lse32;
+    } else {
+        rowdot(d_o, o, delta, B * H * T, D, dtype, st);
+    }
     a.lse_in = lse; a.d_o = do32; a.delta = delta;
     a.dq = dq ? dq32 : nullptr;
     a.dk2 = want_k2 ? dk232 : nullptr; a.dv2 = want_k2 ? dv232 : nullptr;
     a.dk1 = want_k1 ? dk132 : nullptr; a.du = want_k1 ? du : nullptr;
-    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha;
-    a.causal = causal; a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
-    hipError_t e = generic_tdp_bwd(a, st);
+    hipError_t e = mfma32 ? f32_mfma_tdp_bwd(a, fixed, st) : generic_tdp_bwd(a, st);
     if (e != hipSuccess) return (int)e;
     if (dv1) from_f32(du, v1, dv1, n, dtype, st);
     if (dtype != TRITT_F32) {

@@ -12,6 +12,7 @@ struct Knobs {
     int fwd_band;        // TRITT_TUNE_FWD_BAND / env TRITT_FWD_BAND: -1 switches the band-resident forward off
     int bwd_splits;      // TRITT_TUNE_BWD_SPLITS / env TRITT_BWD_SPLITS: workgroups per query tile, backward (1..16)
     int bwd128_variant;  // TRITT_TUNE_BWD128_WAVES / env TRITT_BWD128_VARIANT=w8|w4: 8 or 4 waves per workgroup
+    int f32_valu;        // TRITT_TUNE_F32_VALU: 1 = fp32 tensors take the VALU kernels at every head dimension
 };
 Knobs knobs();
 
@@ -34,6 +35,32 @@ struct GenericTdpArgs {
 };
 hipError_t generic_tdp_fwd(const GenericTdpArgs& a, hipStream_t st);
 hipError_t generic_tdp_bwd(const GenericTdpArgs& a, hipStream_t st);
+
+// fp32 MFMA triple-dot kernels (D = 32 or 64, any mask): same operands as the VALU kernels
+bool f32_mfma_tdp_supported(int D);
+hipError_t f32_mfma_tdp_fwd(const GenericTdpArgs& a, hipStream_t st);
+// backward: `scratch` = f32_mfma_tdp_bwd_scratch_elems() 64-bit words (fixed-point accumulators of the four
+// key / value gradients; zeroed by the call)
+size_t f32_mfma_tdp_bwd_scratch_elems(int BH, int T, int D);
+hipError_t f32_mfma_tdp_bwd(const GenericTdpArgs& a, long long* scratch, hipStream_t st);
+
+// The first `tiles` query tiles (32 queries each) of a 16-bit triple-dot backward, computed in fp32 from the
+// 16-bit tensors (D = 32, 64 or 128) and added to the accumulators of the 16-bit MFMA backward, which then starts
+// at the tile after them.
+struct FirstTileArgs {
+    const void *q, *d_o, *k1, *u, *k2, *v2;  // 16-bit [BH][T][D]; u = SiLU(V1)
+    float *lse_f32, *delta_f32;               // scratch [BH][T]: the covered rows' LSE and Delta, recomputed in fp32
+    void* dq;                                 // written when acc_q is null
+    void *acc_k2, *acc_v2, *acc_k1, *acc_u;   // fixed point (long long) or float
+    void* acc_q;                              // dQ / alpha accumulator of a split backward, or null
+    float fixed_scale;                        // 0: float accumulators
+    int BH, T, D, is_bf16;
+    float alpha;
+    int causal, k1_window, k2_window, kk_left, kk_right;
+    bool want_q, want_k2, want_k1;
+    int tiles;
+};
+hipError_t f32_mfma_tdp_bwd_first_tile(const FirstTileArgs& a, hipStream_t st);
 
 // fp32 operands of the dot-product-sum kernels (two chained attention passes).
 struct DpsArgs {

@@ -547,7 +547,7 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
 }
 
 struct BwdLayout {
-    size_t u, ut, k1t, k2t, v2t, delta, dk1acc, duacc, dk2acc, dv2acc, dqacc, total;
+    size_t u, ut, k1t, k2t, v2t, delta, lse_f32, delta_f32, dk1acc, duacc, dk2acc, dv2acc, dqacc, total;
 };
 static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     const size_t Tp = (size_t)(T + 63) / 64 * 64, n = (size_t)BH * T * D;
@@ -565,6 +565,8 @@ static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     l.k2t = take((size_t)BH * D * Tp * 2);
     l.v2t = take((size_t)BH * D * Tp * 2);
     l.delta = take((size_t)BH * T * 4);
+    l.lse_f32 = take((size_t)BH * T * 4);    // fp32 tiles of the backward: their rows' LSE and Delta in fp32
+    l.delta_f32 = take((size_t)BH * T * 4);
     const size_t acc = fixed_point ? 8 : 4;
     l.dk1acc = take(n * acc);
     l.duacc = take(n * acc);
@@ -649,23 +651,46 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     }
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
+    const bool want_q = a.dq != nullptr, want_k2 = a.dk2 || a.dv2, want_k1 = a.dk1 || a.dv1;
+    // Under a causal mask the first query tile goes through the fp32 kernel (tdp_f32_mfma.hip): its softmax rows
+    // are nearly one-hot, and dS = P (dP - Delta) then cancels two numbers whose 16-bit operand rounding the
+    // kernels here cannot resolve (query 0 has a gradient of exactly zero in dQ).  The kernels below start at
+    // tile 1: the grid simply has one tile less, and the heaviest-first numbering never reaches tile 0.
+    // A windowed mask that leaves a query no more than about a thousand (j, k) pairs makes every row like that:
+    // then all query tiles take the fp32 kernel (the work of such masks is small: T times the pair count).
+    const bool first_in_f32 = a.causal != 0;
+    const long long pairs = (long long)(a.k2_window + 1) * std::min(a.k1_window + 1, a.kk_left + a.kk_right + 1);
+    const bool all_in_f32 = first_in_f32 && a.windowed && pairs <= 1024;
+    if (first_in_f32) {
+        FirstTileArgs f{};
+        f.q = a.q; f.d_o = a.d_o; f.k1 = a.k1; f.u = u; f.k2 = a.k2; f.v2 = a.v2;
+        f.lse_f32 = (float*)(ws + l.lse_f32); f.delta_f32 = (float*)(ws + l.delta_f32);
+        f.dq = a.dq; f.acc_k2 = dk2acc; f.acc_v2 = dv2acc; f.acc_k1 = dk1acc; f.acc_u = duacc; f.acc_q = dqacc;
+        f.fixed_scale = a.deterministic ? kFixedScale : 0.f;
+        f.BH = a.BH; f.T = a.T; f.D = D; f.is_bf16 = a.is_bf16;
+        f.alpha = a.alpha; f.causal = a.causal;
+        f.k1_window = a.k1_window; f.k2_window = a.k2_window; f.kk_left = a.kk_left; f.kk_right = a.kk_right;
+        f.want_q = want_q; f.want_k2 = want_k2; f.want_k1 = want_k1;
+        f.tiles = all_in_f32 ? p.nqt : 1;
+        if (hipError_t e = f32_mfma_tdp_bwd_first_tile(f, st); e != hipSuccess) return e;
+    }
+    const int tiles_here = all_in_f32 ? 0 : p.nqt - (first_in_f32 ? 1 : 0);
     const int groups = (a.BH + 7) / 8;
-    const dim3 grid(8 * groups * p.nqt * col_parts * p.splits);
+    const dim3 grid(8 * groups * std::max(tiles_here, 1) * col_parts * p.splits);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
     p.acc_k = dk2acc; p.acc_v = dv2acc;
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
     // a launch whose gradients the caller does not want (null outputs) is skipped
-    const bool want_q = a.dq != nullptr, want_k2 = a.dk2 || a.dv2, want_k1 = a.dk1 || a.dv1;
-    if (want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
-    else if (want_k2) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
+    if (tiles_here > 0 && want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
+    else if (tiles_here > 0 && want_k2) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU
     p.row_k = (const E*)a.k1; p.row_v = u;
     p.st_k = (const E*)a.k2; p.st_v = (const E*)a.v2; p.st_kt = k2t; p.st_vt = v2t;
     p.acc_k = dk1acc; p.acc_v = duacc;
     p.wa = a.k2_window; p.wb = a.k1_window; p.lab = a.kk_right; p.rab = a.kk_left;  // the mask with j and k exchanged
-    if (want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
+    if (tiles_here > 0 && want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
 
     const size_t n = (size_t)a.BH * a.T * D;
     size_t gridf = (n + 255) / 256;

@@ -1,0 +1,679 @@
+// Triple-dot-product trittention in true fp32 on the matrix cores (v_mfma_f32_32x32x2_f32), D = 32 or 64,
+// every mask.  This is the path of fp32 tensors: fp32 operands, fp32 products, fp32 accumulation (the 1e-4
+// relative bar), at the fp32 matrix rate (157 TFLOP/s peak) instead of the fp32 vector rate of the VALU kernels.
+//
+// All tensors here are fp32 [BH, T, D]; U = SiLU(V1) (see capi.hip).
+//
+// Formulation (the same virtual-query one as the 16-bit kernels).  A workgroup owns 32 consecutive queries;
+// its eight waves take eight consecutive rows b per round (one per wave; b = k, the K2 / V2 row, in the
+// natural orientation) and sweep the streamed index a (= j, K1 / U rows) in 32-row stages shared through LDS.
+// For a fixed row b the scores of the 32 queries against 32 streamed rows are one 32x32 tile
+//   S^T[a, q] = sum_d KA[a, d] * (scale * Q[q, d] * KB[b, d])
+// i.e. D / 2 MFMAs (K = 2 each).  The tile leaves the MFMA with lane <-> query and registers <-> streamed rows,
+// which is exactly the B-operand layout of the next product
+//   Tv^T[d, q] += sum_a VA^T[d, a] * P^T[a, q]
+// so P is never moved between lanes, and every per-query quantity (running maximum, row sum, the merge of a
+// finished row b into the output, O^T[d, q] += Tv^T[d, q] * VB[b, d]) is lane-local.
+// With 64-cycle MFMAs the kernels are bound by the matrix pipe; the element-wise work (mask predicate on every
+// element, online softmax) hides under it, so there is one loop body for every mask.
+#include "common.hpp"
+#include "kernels.hpp"
+#include "mfma.hpp"
+
+namespace tritt {
+namespace {
+
+constexpr int kF32Waves = 8;
+constexpr float kNegBig = -1.0e30f;  // finite stand-in for "no maximum yet"
+
+__device__ __forceinline__ f32x16 mma_f32(float a, float b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+template <typename E>
+struct F32Params {
+    const E *q, *ka, *kb, *va, *vb;  // streamed = (ka, va), rows = (kb, vb)
+    E* o;
+    float* lse;
+    // STATS mode (the 16-bit backward's fp32 tiles): O is not written; lse receives the fp32 log-sum-exp of the
+    // covered rows and delta their rowsum(dO * O) with O in fp32
+    const E* d_o;
+    float* delta;
+    int T, BH, nqt;  // nqt: query tiles this launch covers (tiles 0 .. nqt - 1)
+    float scale_log2;
+    TdpMask mask;  // in terms of the streamed index a and the row index b
+};
+
+// Ranges of streamed rows / owner rows a tile of queries [q0, q1] can touch.
+struct Range {
+    int lo, hi;
+};
+__device__ __forceinline__ Range row_range(const TdpMask& m, int q0, int q1, int T) {
+    if (!m.causal) return {0, T - 1};
+    return {max(0, q0 - m.wb), q1};
+}
+__device__ __forceinline__ Range streamed_range(const TdpMask& m, int q0, int q1, int b, int T) {
+    if (!m.causal) return {0, T - 1};
+    // a <= q, q - a <= wa, b - a <= lab, a - b <= rab
+    return {max(0, max(q0 - m.wa, b - m.lab)), min(q1, b + m.rab)};
+}
+
+// Staging of 32 x D tiles of E through registers (16-byte pieces), converted to fp32 on the way into LDS.
+template <typename E, int D>
+struct StageE {
+    static constexpr int VE = 16 / (int)sizeof(E);           // elements per piece
+    static constexpr int kPieces = 32 * D / VE;               // per tensor
+    static constexpr int kPer = (kPieces + 255) / 256;        // per thread
+    uint4 x[kPer];
+};
+template <typename E, int D>
+__device__ __forceinline__ void stage_fetch_e(StageE<E, D>& r, const E* __restrict__ ka, const E* __restrict__ va, int a0,
+                                              int T) {
+    using S = StageE<E, D>;
+    constexpr int kVec = D / S::VE;
+    const int t = threadIdx.x & 255;
+    const E* src = threadIdx.x < 256 ? ka : va;
+#pragma unroll
+    for (int i = 0; i < S::kPer; ++i) {
+        const int idx = t + i * 256;
+        if (idx < S::kPieces) {
+            const int row = idx / kVec, c = idx % kVec;
+            r.x[i] = *reinterpret_cast<const uint4*>(src + (size_t)min(a0 + row, T - 1) * D + c * S::VE);
+        }
+    }
+}
+template <typename E, int D>
+__device__ __forceinline__ void stage_store_e(const StageE<E, D>& r, float* sk, float* sv) {
+    using S = StageE<E, D>;
+    constexpr int kVec = D / S::VE, LD = D + 1;
+    const int t = threadIdx.x & 255;
+    float* dst = threadIdx.x < 256 ? sk : sv;
+#pragma unroll
+    for (int i = 0; i < S::kPer; ++i) {
+        const int idx = t + i * 256;
+        if (idx < S::kPieces) {
+            const int row = idx / kVec, c = idx % kVec;
+            float* p = dst + row * LD + c * S::VE;
+            const E* e = reinterpret_cast<const E*>(&r.x[i]);
+#pragma unroll
+            for (int k = 0; k < S::VE; ++k) p[k] = (float)e[k];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ forward
+template <typename E, int D, bool STATS>
+__global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
+    constexpr int DT = D / 32, KS = D / 2, LD = D + 1, NW = kF32Waves;
+    constexpr bool FLY = D > 64;  // form the B operand of the score product as it is used
+    extern __shared__ __align__(16) float smem_f[];
+    float* sK = smem_f;                 // [2][32][LD] streamed key rows
+    float* sV = sK + 2 * 32 * LD;       // [2][32][LD] streamed value rows
+    float* sQ = sV + 2 * 32 * LD;       // [32][LD]    the tile's queries * scale
+    float* sKb = sQ + 32 * LD;          // [NW][D]     row operands of the round
+    float* sVb = sKb + NW * D;          // [NW][D]
+    float* sM = sVb + NW * D;           // [NW][32]    end of kernel: per-wave maxima and sums
+    float* sL = sM + NW * 32;           // [NW][32]
+    float* sO = sK;                     // [D][33]     end of kernel: merged output (aliases the stages)
+
+    const int groups = (p.BH + 7) / 8;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int bh = (slot % groups) * 8 + xcd;
+    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
+    if (bh >= p.BH) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int T = p.T;
+    const size_t base = (size_t)bh * T * D;
+    const E* __restrict__ KA = p.ka + base;
+    const E* __restrict__ VA = p.va + base;
+    const E* __restrict__ KB = p.kb + base;
+    const E* __restrict__ VB = p.vb + base;
+    const TdpMask mask = p.mask;
+
+    const int q0 = qt * 32, q1 = min(T - 1, q0 + 31);
+    const int q = q0 + n;  // this lane's query (column of every tile)
+    for (int idx = tid; idx < 32 * D; idx += 512) {
+        const int r = idx / D, d = idx % D;
+        sQ[r * LD + d] = (float)p.q[base + (size_t)min(q0 + r, T - 1) * D + d] * p.scale_log2;
+    }
+
+    const Range rows = row_range(mask, q0, q1, T);
+    const int m_lo = rows.lo / NW, m_hi = rows.hi / NW;  // rounds of NW rows
+
+    f32x16 accO[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) accO[dt][i] = 0.f;
+    float m_run = kNegBig, l_run = 0.f;  // per query, over every (a, b) this wave has seen (l: this lane's half)
+
+    StageE<E, D> regs;
+    for (int m = m_lo; m <= m_hi; ++m) {
+        const int b = m * NW + wave;
+        // the streamed stages this round needs: the union over its rows
+        const Range ra = streamed_range(mask, q0, q1, min(m * NW, T - 1), T);
+        const Range rb = streamed_range(mask, q0, q1, min(m * NW + NW - 1, T - 1), T);
+        const int st_lo = min(ra.lo, rb.lo) / 32, st_hi = max(ra.hi, rb.hi) / 32;
+        const bool row_ok = b <= rows.hi && b >= rows.lo;
+        const Range mine = streamed_range(mask, q0, q1, min(b, T - 1), T);
+
+        __syncthreads();  // previous round: everyone is done with sKb / sVb and the stage buffers
+        for (int idx = tid; idx < NW * D; idx += 512) {
+            const int r = idx / D, d = idx % D;
+            const size_t off = (size_t)min(m * NW + r, T - 1) * D + d;
+            sKb[idx] = (float)KB[off];
+            sVb[idx] = (float)VB[off];
+        }
+        if (st_lo <= st_hi) {
+            stage_fetch_e<E, D>(regs, KA, VA, st_lo * 32, T);
+            stage_store_e<E, D>(regs, sK, sV);
+        }
+        __syncthreads();
+
+        // B operand of the score product: lane (q, g), step s holds scale * Q[q, g*D/2 + s] * KB[b, g*D/2 + s]
+        float bq[FLY ? 1 : KS];
+        if constexpr (!FLY) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) bq[s] = sQ[n * LD + g * KS + s] * sKb[wave * D + g * KS + s];
+        }
+
+        f32x16 accT[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) accT[dt][i] = 0.f;
+
+        for (int st = st_lo; st <= st_hi; ++st) {
+            const int buf = (st - st_lo) & 1;
+            const float* cK = sK + buf * 32 * LD;
+            const float* cV = sV + buf * 32 * LD;
+            const bool more = st < st_hi;
+            if (more) stage_fetch_e<E, D>(regs, KA, VA, (st + 1) * 32, T);
+            const int a0 = st * 32;
+            if (row_ok && a0 + 31 >= mine.lo && a0 <= mine.hi) {
+                f32x16 s;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int col = g * KS + ks;
+                    const float oq = FLY ? sQ[n * LD + col] * sKb[wave * D + col] : bq[FLY ? 0 : ks];
+                    s = mma_f32(cK[n * LD + col], oq, s);
+                }
+                // mask, tile maximum of this lane's 16 rows
+                float tmax = kNegBig;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int a = a0 + c_row(g, i);
+                    const bool ok = a < T && tdp_valid(mask, q, a, b);
+                    s[i] = ok ? s[i] : -INFINITY;
+                    tmax = fmaxf(tmax, s[i]);
+                }
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+                const float m_new = fmaxf(m_run, tmax);
+                if (__any(m_new > m_run)) {
+                    const float sc = fast_exp2(m_run - m_new);
+                    l_run *= sc;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            accT[dt][i] *= sc;
+                            accO[dt][i] *= sc;
+                        }
+                    m_run = m_new;
+                }
+                float psum = 0.f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = fast_exp2(s[i] - m_run);
+                    psum += s[i];
+                }
+                l_run += psum;
+                // Tv^T[d, q] += VA^T[d, a] P^T[a, q]: step i contracts the two streamed rows c_row(0, i), c_row(1, i)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) accT[dt] = mma_f32(cV[c_row(g, i) * LD + dt * 32 + n], s[i], accT[dt]);
+            }
+            if (more) {
+                stage_store_e<E, D>(regs, sK + (buf ^ 1) * 32 * LD, sV + (buf ^ 1) * 32 * LD);
+                __syncthreads();
+            }
+        }
+        // the finished row: O^T[d, q] += Tv^T[d, q] * VB[b, d]   (register i of half g is d = 32 dt + c_row(g, i))
+        if (row_ok) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) accO[dt][i] += accT[dt][i] * sVb[wave * D + dt * 32 + c_row(g, i)];
+        }
+    }
+
+    // ---- merge the eight waves' partial results (each relative to its own maximum), one wave after another
+    l_run += __shfl_xor(l_run, 32, 64);
+    __syncthreads();
+    if (g == 0) {
+        sM[wave * 32 + n] = m_run;
+        sL[wave * 32 + n] = l_run;
+    }
+    for (int idx = tid; idx < D * 33; idx += 512) sO[idx] = 0.f;
+    __syncthreads();
+    float M = kNegBig;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sM[w * 32 + n]);
+    const float mine_scale = fast_exp2(m_run - M);
+    for (int w = 0; w < NW; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) sO[(dt * 32 + c_row(g, i)) * 33 + n] += accO[dt][i] * mine_scale;
+        }
+        __syncthreads();
+    }
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) L += sL[w * 32 + n] * fast_exp2(sM[w * 32 + n] - M);
+    if constexpr (STATS) {
+        // Delta[q] = sum_d dO[q, d] O[q, d] with O in fp32 (lane n of wave 0 walks its query's row)
+        if (wave == 0 && g == 0 && q < T) {
+            float dsum = 0.f;
+            for (int d = 0; d < D; ++d) dsum += (float)p.d_o[base + (size_t)q * D + d] * sO[d * 33 + n];
+            p.delta[(size_t)bh * T + q] = dsum / L;
+        }
+    } else {
+        for (int idx = tid; idx < 32 * D; idx += 512) {
+            const int r = idx / D, d = idx % D;
+            if (q0 + r < T) {
+                float Lr = 0.f, Mr = kNegBig;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) Mr = fmaxf(Mr, sM[w * 32 + r]);
+#pragma unroll
+                for (int w = 0; w < NW; ++w) Lr += sL[w * 32 + r] * fast_exp2(sM[w * 32 + r] - Mr);
+                p.o[base + (size_t)(q0 + r) * D + d] = (E)(sO[d * 33 + r] / Lr);
+            }
+        }
+    }
+    if (wave == 0 && g == 0 && q < T) p.lse[(size_t)bh * T + q] = (M + fast_log2(L)) * kLn2;
+}
+
+// ------------------------------------------------------------------------------------------ backward
+// Launched twice, like the 16-bit backward: rows = (K2, V2), streamed = (K1, U) gives dQ, dK2, dV2; with the roles
+// exchanged, dK1 and dU.  Per (query tile, row b, 32 streamed rows):
+//   S^T, dP^T (D / 2 MFMAs each),  P = exp2(S - LSE2[q]),  dS = P (dP - Delta[q])   (both lane-local)
+//   Yq^T[d, q] += KA^T[d, a] dS^T[a, q]      Tv^T[d, q] += VA^T[d, a] P^T[a, q]      (DOUT / 2 MFMAs each)
+// and when the row is finished
+//   dQ^T[d, q] += Yq^T[d, q] KB[b, d]                                  (registers, all rounds)
+//   dKB[b, d]  += alpha sum_q Yq^T[d, q] Q[q, d],   dVB[b, d] += sum_q Tv^T[d, q] dO[q, d]
+// The sums over the tile's 32 queries are lane reductions; the sums over query tiles (workgroups) go to shared
+// accumulators: 64-bit fixed point with integer atomics (the result does not depend on the order of arrival), or
+// fp32 atomics when the caller's accumulators are fp32.
+//
+// The tensors may be 16-bit (E = bf16 / f16): they are converted as they are staged, everything after that is
+// fp32.  That is how the 16-bit backward runs its first query tile: for the first few causal queries the softmax
+// is nearly one-hot and dS = P (dP - Delta) cancels two O(10) numbers, which the 16-bit operands of the MFMA
+// kernels (dO * V2 rounded to 16 bit) cannot resolve.
+// D = 128: a workgroup produces DOUT = 64 of the gradient columns (blockIdx.y picks the half), and the B operands
+// of the score products are formed as they are used instead of being held in registers.
+constexpr float kF32FixedScale = 68719476736.0f;  // 2^36: |sum| < 1.3e8 in steps of 1.5e-11
+
+template <typename E>
+struct F32BwdParams {
+    const E *q, *d_o, *ka, *kb, *va, *vb;
+    const float *lse, *delta;
+    E* dq;                 // WITH_DQ, when acc_q is null
+    void *acc_k, *acc_v;   // [BH][T][D] gradients of the rows: fixed point (long long) or float
+    void* acc_q;           // WITH_DQ: when non-null, dQ / alpha is added here instead of being written to dq
+    float fixed_scale;     // scale of the fixed-point accumulators; 0: the accumulators are float
+    int T, BH, nqt;        // nqt: query tiles this launch covers (tiles 0 .. nqt - 1)
+    float alpha;
+    TdpMask mask;
+};
+
+__device__ __forceinline__ float half_sum(float v) {  // over the 32 lanes of a wave half
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ void shared_add(void* acc, size_t idx, float v, float fixed_scale) {
+    if (fixed_scale != 0.f)
+        atomicAdd(reinterpret_cast<unsigned long long*>(acc) + idx, (unsigned long long)__float2ll_rn(v * fixed_scale));
+    else
+        unsafeAtomicAdd(reinterpret_cast<float*>(acc) + idx, v);
+}
+
+template <typename E, int D, int DOUT, bool WITH_DQ>
+__global__ __launch_bounds__(512) void tdp_f32_bwd_kernel(F32BwdParams<E> p) {
+    constexpr int DTO = DOUT / 32, KS = D / 2, LD = D + 1, NW = kF32Waves;
+    constexpr bool FLY = D > 64;  // form the B operands of the score products as they are used
+    extern __shared__ __align__(16) float smem_f[];
+    float* sK = smem_f;                 // [2][32][LD]
+    float* sV = sK + 2 * 32 * LD;       // [2][32][LD]
+    float* sQ = sV + 2 * 32 * LD;       // [32][LD]  Q * alpha * log2(e)
+    float* sDO = sQ + 32 * LD;          // [32][LD]
+    float* sKb = sDO + 32 * LD;         // [NW][D]
+    float* sVb = sKb + NW * D;          // [NW][D]
+    float* sO = sK;                     // [DOUT][33]   end of kernel: dQ of the tile (aliases the stages)
+
+    const int groups = (p.BH + 7) / 8;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int bh = (slot % groups) * 8 + xcd;
+    const int qt = p.nqt - 1 - slot / groups;
+    const int c0 = blockIdx.y * DOUT;  // first gradient column of this workgroup
+    if (bh >= p.BH) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int T = p.T;
+    const size_t base = (size_t)bh * T * D;
+    const E* __restrict__ KA = p.ka + base;
+    const E* __restrict__ VA = p.va + base;
+    const E* __restrict__ KB = p.kb + base;
+    const E* __restrict__ VB = p.vb + base;
+    const TdpMask mask = p.mask;
+    const float scale_log2 = p.alpha * kLog2e;
+
+    const int q0 = qt * 32, q1 = min(T - 1, q0 + 31);
+    const int q = q0 + n;
+    for (int idx = tid; idx < 32 * D; idx += 512) {
+        const int r = idx / D, d = idx % D;
+        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
+        sQ[r * LD + d] = (float)p.q[off] * scale_log2;
+        sDO[r * LD + d] = (float)p.d_o[off];
+    }
+    // a query past the end of the sequence gets a huge LSE: its P is exactly 0
+    const float lse2 = q < T ? p.lse[(size_t)bh * T + q] * kLog2e : 1.0e30f;
+    const float delta = q < T ? p.delta[(size_t)bh * T + q] : 0.f;
+
+    const Range rows = row_range(mask, q0, q1, T);
+    const int m_lo = rows.lo / NW, m_hi = rows.hi / NW;
+
+    f32x16 accDQ[DTO];
+#pragma unroll
+    for (int dt = 0; dt < DTO; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) accDQ[dt][i] = 0.f;
+
+    StageE<E, D> regs;
+    for (int m = m_lo; m <= m_hi; ++m) {
+        const int b = m * NW + wave;
+        const Range ra = streamed_range(mask, q0, q1, min(m * NW, T - 1), T);
+        const Range rb = streamed_range(mask, q0, q1, min(m * NW + NW - 1, T - 1), T);
+        const int st_lo = min(ra.lo, rb.lo) / 32, st_hi = max(ra.hi, rb.hi) / 32;
+        const bool row_ok = b <= rows.hi && b >= rows.lo;
+        const Range mine = streamed_range(mask, q0, q1, min(b, T - 1), T);
+
+        __syncthreads();
+        for (int idx = tid; idx < NW * D; idx += 512) {
+            const int r = idx / D, d = idx % D;
+            const size_t off = (size_t)min(m * NW + r, T - 1) * D + d;
+            sKb[idx] = (float)KB[off];
+            sVb[idx] = (float)VB[off];
+        }
+        if (st_lo <= st_hi) {
+            stage_fetch_e<E, D>(regs, KA, VA, st_lo * 32, T);
+            stage_store_e<E, D>(regs, sK, sV);
+        }
+        __syncthreads();
+
+        float bq[FLY ? 1 : KS], bg[FLY ? 1 : KS];
+        if constexpr (!FLY) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                bq[s] = sQ[n * LD + g * KS + s] * sKb[wave * D + g * KS + s];
+                bg[s] = sDO[n * LD + g * KS + s] * sVb[wave * D + g * KS + s];
+            }
+        }
+        f32x16 accQ[DTO], accT[DTO];
+#pragma unroll
+        for (int dt = 0; dt < DTO; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                accQ[dt][i] = 0.f;
+                accT[dt][i] = 0.f;
+            }
+
+        for (int st = st_lo; st <= st_hi; ++st) {
+            const int buf = (st - st_lo) & 1;
+            const float* cK = sK + buf * 32 * LD;
+            const float* cV = sV + buf * 32 * LD;
+            const bool more = st < st_hi;
+            if (more) stage_fetch_e<E, D>(regs, KA, VA, (st + 1) * 32, T);
+            const int a0 = st * 32;
+            if (row_ok && a0 + 31 >= mine.lo && a0 <= mine.hi) {
+                f32x16 s, dp;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = 0.f;
+                    dp[i] = 0.f;
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int col = g * KS + ks;
+                    const float oq = FLY ? sQ[n * LD + col] * sKb[wave * D + col] : bq[FLY ? 0 : ks];
+                    const float og = FLY ? sDO[n * LD + col] * sVb[wave * D + col] : bg[FLY ? 0 : ks];
+                    s = mma_f32(cK[n * LD + col], oq, s);
+                    dp = mma_f32(cV[n * LD + col], og, dp);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int a = a0 + c_row(g, i);
+                    const bool ok = a < T && tdp_valid(mask, q, a, b);
+                    const float pv = ok ? fast_exp2(s[i] - lse2) : 0.f;
+                    s[i] = pv;
+                    dp[i] = pv * (dp[i] - delta);
+                }
+#pragma unroll
+                for (int dt = 0; dt < DTO; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        accT[dt] = mma_f32(cV[c_row(g, i) * LD + c0 + dt * 32 + n], s[i], accT[dt]);
+                        accQ[dt] = mma_f32(cK[c_row(g, i) * LD + c0 + dt * 32 + n], dp[i], accQ[dt]);
+                    }
+            }
+            if (more) {
+                stage_store_e<E, D>(regs, sK + (buf ^ 1) * 32 * LD, sV + (buf ^ 1) * 32 * LD);
+                __syncthreads();
+            }
+        }
+        if (row_ok) {
+#pragma unroll
+            for (int dt = 0; dt < DTO; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int d = c0 + dt * 32 + c_row(g, i);
+                    if constexpr (WITH_DQ) accDQ[dt][i] += accQ[dt][i] * sKb[wave * D + d];
+                    // sQ holds Q * alpha * log2(e): alpha is wanted, log2(e) is not
+                    const float rk = half_sum(accQ[dt][i] * sQ[n * LD + d]) * kLn2;
+                    const float rv = half_sum(accT[dt][i] * sDO[n * LD + d]);
+                    if (n == 0) {
+                        const size_t idx = base + (size_t)b * D + d;
+                        shared_add(p.acc_k, idx, rk, p.fixed_scale);
+                        shared_add(p.acc_v, idx, rv, p.fixed_scale);
+                    }
+                }
+        }
+    }
+
+    if constexpr (WITH_DQ) {
+        __syncthreads();
+        for (int idx = tid; idx < DOUT * 33; idx += 512) sO[idx] = 0.f;
+        __syncthreads();
+        for (int w = 0; w < NW; ++w) {  // one wave after another: a fixed summation order
+            if (wave == w) {
+#pragma unroll
+                for (int dt = 0; dt < DTO; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) sO[(dt * 32 + c_row(g, i)) * 33 + n] += accDQ[dt][i];
+            }
+            __syncthreads();
+        }
+        for (int idx = tid; idx < 32 * DOUT; idx += 512) {
+            const int r = idx / DOUT, d = idx % DOUT;
+            if (q0 + r < T) {
+                const size_t off = base + (size_t)(q0 + r) * D + c0 + d;
+                if (p.acc_q) shared_add(p.acc_q, off, sO[d * 33 + r], p.fixed_scale);
+                else p.dq[off] = (E)(sO[d * 33 + r] * p.alpha);
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void f32_zero_kernel(long long* __restrict__ a, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) a[i] = 0;
+}
+// fixed point -> fp32
+__global__ __launch_bounds__(256) void f32_finish_kernel(const long long* __restrict__ acc, float* __restrict__ dk_rows,
+                                                         float* __restrict__ dv_rows, size_t n) {
+    const double inv = 1.0 / (double)kF32FixedScale;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        dk_rows[i] = (float)((double)acc[i] * inv);
+        dv_rows[i] = (float)((double)acc[n + i] * inv);
+    }
+}
+
+template <int D>
+constexpr size_t f32_bwd_smem() {
+    return sizeof(float) * (size_t)(4 * 32 * (D + 1) + 2 * 32 * (D + 1) + 2 * kF32Waves * D);
+}
+
+// both launches of the backward over query tiles 0 .. nqt - 1
+template <typename E, int D>
+hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, const E* k2, const E* v2, void* acc_k2,
+                                void* acc_v2, void* acc_k1, void* acc_u, const TdpMask& natural, bool want_q,
+                                bool want_k2, bool want_k1, hipStream_t st) {
+    constexpr int DOUT = D > 64 ? 64 : D;
+    auto kern_dq = tdp_f32_bwd_kernel<E, D, DOUT, true>;
+    auto kern_nodq = tdp_f32_bwd_kernel<E, D, DOUT, false>;
+    constexpr size_t smem = f32_bwd_smem<D>();
+    static_assert(DOUT * 33 <= 4 * 32 * (D + 1), "dQ of the tile aliases the stage buffers");
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
+    const int groups = (p.BH + 7) / 8;
+    const dim3 grid(8 * groups * p.nqt, D / DOUT);
+    // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
+    p.ka = k1; p.va = u; p.kb = k2; p.vb = v2;
+    p.acc_k = acc_k2; p.acc_v = acc_v2;
+    p.mask = natural;
+    if (want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(512), smem, st, p);
+    else if (want_k2) hipLaunchKernelGGL(kern_nodq, grid, dim3(512), smem, st, p);
+    // rows = (K1, U), streamed = (K2, V2): dK1, dU (the mask with the two key indices exchanged)
+    p.ka = k2; p.va = v2; p.kb = k1; p.vb = u;
+    p.acc_k = acc_k1; p.acc_v = acc_u;
+    p.mask = TdpMask{natural.causal, natural.wb, natural.wa, natural.rab, natural.lab};
+    if (want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(512), smem, st, p);
+    return hipGetLastError();
+}
+
+template <int D>
+hipError_t launch_f32_bwd(const GenericTdpArgs& a, long long* acc, hipStream_t st) {
+    const size_t n = (size_t)a.BH * a.T * D;
+    const bool want_q = a.dq != nullptr, want_k2 = a.dk2 && a.dv2, want_k1 = a.dk1 && a.du;
+    F32BwdParams<float> p{};
+    p.q = a.q; p.d_o = a.d_o; p.lse = a.lse_in; p.delta = a.delta;
+    p.dq = a.dq; p.acc_q = nullptr; p.fixed_scale = kF32FixedScale;
+    p.T = a.T; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
+    p.alpha = a.alpha;
+    size_t gz = (4 * n + 255) / 256;
+    if (gz > 8192) gz = 8192;
+    hipLaunchKernelGGL(f32_zero_kernel, dim3((unsigned)gz), dim3(256), 0, st, acc, 4 * n);
+    const TdpMask natural{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
+    if (hipError_t e = launch_f32_bwd_tiles<float, D>(p, a.k1, a.u, a.k2, a.v2, acc, acc + n, acc + 2 * n, acc + 3 * n,
+                                                      natural, want_q, want_k2, want_k1, st);
+        e != hipSuccess)
+        return e;
+    size_t gf = (n + 255) / 256;
+    if (gf > 4096) gf = 4096;
+    if (want_k2) hipLaunchKernelGGL(f32_finish_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc, a.dk2, a.dv2, n);
+    if (want_k1) hipLaunchKernelGGL(f32_finish_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc + 2 * n, a.dk1, a.du, n);
+    return hipGetLastError();
+}
+
+template <int D>
+constexpr size_t f32_fwd_smem() {
+    return sizeof(float) * (size_t)(4 * 32 * (D + 1) + 32 * (D + 1) + 2 * kF32Waves * D + 2 * kF32Waves * 32);
+}
+
+template <int D>
+hipError_t launch_f32_fwd(const GenericTdpArgs& a, hipStream_t st) {
+    F32Params<float> p{};
+    p.q = a.q; p.ka = a.k1; p.kb = a.k2; p.va = a.u; p.vb = a.v2;
+    p.o = a.o; p.lse = a.lse;
+    p.T = a.T; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
+    p.scale_log2 = a.alpha * kLog2e;
+    p.mask = TdpMask{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
+    auto kern = tdp_f32_fwd_kernel<float, D, false>;
+    constexpr size_t smem = f32_fwd_smem<D>();
+    static_assert(D * 33 <= 4 * 32 * (D + 1), "the merged output aliases the stage buffers");
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
+    const int groups = (a.BH + 7) / 8;
+    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool f32_mfma_tdp_supported(int D) { return D == 32 || D == 64; }
+
+// The first query tiles of a 16-bit backward, in fp32 (see the comment above tdp_f32_bwd_kernel).
+template <typename E, int D>
+static hipError_t launch_stats(const FirstTileArgs& a, hipStream_t st) {
+    F32Params<E> p{};
+    p.q = (const E*)a.q; p.ka = (const E*)a.k1; p.kb = (const E*)a.k2; p.va = (const E*)a.u; p.vb = (const E*)a.v2;
+    p.o = nullptr; p.lse = a.lse_f32; p.d_o = (const E*)a.d_o; p.delta = a.delta_f32;
+    p.T = a.T; p.BH = a.BH; p.nqt = a.tiles;
+    p.scale_log2 = a.alpha * kLog2e;
+    p.mask = TdpMask{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
+    auto kern = tdp_f32_fwd_kernel<E, D, true>;
+    constexpr size_t smem = f32_fwd_smem<D>();
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(8 * ((a.BH + 7) / 8) * p.nqt), dim3(512), smem, st, p);
+    return hipGetLastError();
+}
+
+template <typename E>
+static hipError_t first_tile_typed(const FirstTileArgs& a, hipStream_t st) {
+    // the rows' log-sum-exp and Delta once more, in fp32 from the same tensors: the saved LSE carries the 16-bit
+    // rounding of the forward's scores and Delta that of the stored output, and nearly one-hot rows show both
+    hipError_t es = a.D == 32 ? launch_stats<E, 32>(a, st) : a.D == 64 ? launch_stats<E, 64>(a, st)
+                  : a.D == 128 ? launch_stats<E, 128>(a, st) : hipErrorInvalidValue;
+    if (es != hipSuccess) return es;
+    F32BwdParams<E> p{};
+    p.q = (const E*)a.q; p.d_o = (const E*)a.d_o; p.lse = a.lse_f32; p.delta = a.delta_f32;
+    p.dq = (E*)a.dq; p.acc_q = a.acc_q; p.fixed_scale = a.fixed_scale;
+    p.T = a.T; p.BH = a.BH; p.nqt = a.tiles;
+    p.alpha = a.alpha;
+    const TdpMask natural{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
+    const E *k1 = (const E*)a.k1, *u = (const E*)a.u, *k2 = (const E*)a.k2, *v2 = (const E*)a.v2;
+    const bool wq = a.want_q, wk2 = a.want_k2, wk1 = a.want_k1;
+    if (a.D == 32)
+        return launch_f32_bwd_tiles<E, 32>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st);
+    if (a.D == 64)
+        return launch_f32_bwd_tiles<E, 64>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st);
+    if (a.D == 128)
+        return launch_f32_bwd_tiles<E, 128>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st);
+    return hipErrorInvalidValue;
+}
+hipError_t f32_mfma_tdp_bwd_first_tile(const FirstTileArgs& a, hipStream_t st) {
+    return a.is_bf16 ? first_tile_typed<__bf16>(a, st) : first_tile_typed<_Float16>(a, st);
+}
+
+hipError_t f32_mfma_tdp_fwd(const GenericTdpArgs& a, hipStream_t st) {
+    if (a.D == 32) return launch_f32_fwd<32>(a, st);
+    if (a.D == 64) return launch_f32_fwd<64>(a, st);
+    return hipErrorInvalidValue;
+}
+
+size_t f32_mfma_tdp_bwd_scratch_elems(int BH, int T, int D) { return 4 * (size_t)BH * T * D; }
+
+hipError_t f32_mfma_tdp_bwd(const GenericTdpArgs& a, long long* scratch, hipStream_t st) {
+    if (a.D == 32) return launch_f32_bwd<32>(a, scratch, st);
+    if (a.D == 64) return launch_f32_bwd<64>(a, scratch, st);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace tritt

@@ -44,6 +44,8 @@ class TrittentionTritonFunction(torch.autograd.Function):
         q, k1, k2, v1, v2 = (_lib.dense(t) for t in (q, k1, k2, v1, v2))
         k_diff = clamp_window(k_diff, T, "k_diff")
         flags = getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
+        if convert_to_float32 and not flags & _lib.FLAG_FORCE_MFMA:
+            flags |= _lib.FLAG_FORCE_GENERIC  # fp32 operands throughout (trittention_triton.py:92-98 of the reference)
         lib = _lib.lib()
         o = torch.empty_like(q)
         m = torch.empty((B, H, T), dtype=torch.float32, device=q.device)

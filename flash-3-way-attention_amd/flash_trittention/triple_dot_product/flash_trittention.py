@@ -56,6 +56,10 @@ class FlashTrittention(torch.autograd.Function):
         flags = getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
         if torch.are_deterministic_algorithms_enabled():
             flags &= ~_lib.FLAG_FLOAT_ATOMICS  # the default (fixed-point accumulation) is bitwise reproducible
+        if convert_to_float32 and not flags & _lib.FLAG_FORCE_MFMA:
+            # the reference forms its scores in fp32 under this flag (flash_trittention.py:408, bwd_dq.py:197); here
+            # 16-bit tensors then take the fp32 kernels: fp32 operands and products throughout, 16-bit results
+            flags |= _lib.FLAG_FORCE_GENERIC
         lib = _lib.lib()
         code = _lib.dtype_code(Q.dtype)
         O = torch.empty_like(Q)
@@ -110,8 +114,10 @@ def flash_trittention(q, k1, k2, v1, v2, softmax_scale=1 / 8, kk_left=1, kk_righ
     """Triple-dot-product 3-way attention; returns O [B, H, T, D].
 
     Window arguments: ``None`` (or any value >= seq_len) disables a window; note that the
-    literal defaults are 1, a narrow band, exactly as in the reference.  ``convert_to_float32``
-    is accepted for compatibility: scores and softmax are always computed in fp32 here.
+    literal defaults are 1, a narrow band, exactly as in the reference.  Softmax and accumulation are
+    always fp32.  ``convert_to_float32=True`` also keeps the operands of the score products in fp32
+    (16-bit tensors then run the fp32 kernels: about ten times slower, but scores spanning hundreds
+    keep the full 16-bit tolerance, where the 16-bit operands of the default path do not).
     ``input_precision`` is accepted and ignored with a warning, as in the reference.
     """
     if input_precision is not None:

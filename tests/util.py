@@ -91,15 +91,17 @@ def rel_err(got, want):
     return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
 
 
-def assert_mostly_close(name, got, want, rtol, atol, outlier_frac=1e-3, outlier_scale=4.0):
-    """Like assert_close, but tolerates a tiny fraction of elements up to `outlier_scale` times the
-    tolerance.  Used only for 16-bit gradients of rows whose softmax is nearly one-hot (the first
-    few queries of a causal sequence): there dS = P (dP - Delta) is a difference of two O(10)
-    numbers that each carry 16-bit rounding error (dO*V2 is rounded to 16 bit before the MFMA),
-    so single elements can land a few 1e-2 away from an exactly-zero reference."""
+def assert_mostly_close(name, got, want, rtol, atol, outlier_frac=0.0, outlier_scale=1.0):
+    """assert_close that also prints the worst |err| / tol of the comparison.  By default every element must be
+    within tolerance.  `outlier_frac` / `outlier_scale` let a stated fraction of the elements reach a stated
+    multiple of the tolerance: used only where the comparison is not the parity bar itself (the library's MFMA
+    kernels against its own fp32 kernels under scores scaled by 3) or where a single element of a very large
+    tensor sits on the edge of the 16-bit bar; each such call says why."""
     err = (got - want).abs()
     tol = atol + rtol * want.abs()
     bad = err > tol
+    worst = (err / tol).max().item() if err.numel() else 0.0
+    print(f"    {name}: worst |err|/tol = {worst:.2f}, {int(bad.sum())} of {bad.numel()} beyond tol", flush=True)
     assert bad.float().mean().item() <= outlier_frac, f"{name}: {bad.sum().item()} of {bad.numel()} outside tolerance"
     assert (err <= outlier_scale * tol).all(), f"{name}: max error {err.max().item()}"
 
@@ -135,7 +137,10 @@ def check_offsets_beyond_32_bits(variant, B, H, T, D, windows=(None,) * 4, rtol=
                 z, _, grads = orc.dps_forward_backward(*ins, alpha, True, k_diff=T, factorised=True)
             assert_close(f"out[{hd}]", out.detach()[b, h].float().cpu(), z, rtol=rtol, atol=atol)
             for name, leaf, want in zip(NAMES, leaves, grads):
-                assert_mostly_close(f"{name}[{hd}]", leaf.grad[b, h].float().cpu(), want, rtol=rtol, atol=atol)
+                # 512 x 128 elements per head and gradient at the edge of the 16-bit bar: one element in 10^4 may
+                # reach 1.5 times the tolerance (seen: one of 65536 at 1.07)
+                assert_mostly_close(f"{name}[{hd}]", leaf.grad[b, h].float().cpu(), want, rtol=rtol, atol=atol,
+                                    outlier_frac=1e-4, outlier_scale=1.5)
     finally:
         del leaves, do, out
         torch.cuda.empty_cache()
