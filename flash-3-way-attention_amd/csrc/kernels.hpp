@@ -49,7 +49,10 @@ hipError_t f32_mfma_tdp_bwd(const GenericTdpArgs& a, long long* scratch, hipStre
 // at the tile after them.
 struct FirstTileArgs {
     const void *q, *d_o, *k1, *u, *k2, *v2;  // 16-bit [BH][T][D]; u = SiLU(V1)
-    float *lse_f32, *delta_f32;               // scratch [BH][T]: the covered rows' LSE and Delta, recomputed in fp32
+    // scratch, [BH][T] floats each: the covered rows' LSE and Delta, recomputed in fp32 (tiles == 1: delta_f32 holds
+    // the per-round partials of tile 0 instead, [BH][32][4][3])
+    float *lse_f32, *delta_f32;
+    void* dq0_acc;                            // tiles == 1 and acc_q null: [BH][32][D] accumulator of the tile's dQ / alpha
     void* dq;                                 // written when acc_q is null
     void *acc_k2, *acc_v2, *acc_k1, *acc_u;   // fixed point (long long) or float
     void* acc_q;                              // dQ / alpha accumulator of a split backward, or null

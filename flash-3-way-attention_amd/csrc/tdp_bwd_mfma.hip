@@ -531,7 +531,8 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
                                                          const float* __restrict__ dqacc, float alpha,
                                                          E* __restrict__ dq, const E* __restrict__ v1,
                                                          E* __restrict__ dk1, E* __restrict__ dv1, E* __restrict__ dk2,
-                                                         E* __restrict__ dv2, size_t n, int fixed_point) {
+                                                         E* __restrict__ dv2, size_t n, int fixed_point,
+                                                         const float* __restrict__ dq0acc, int T, int D) {
     auto value = [&](const float* acc, size_t i) {
         if (!fixed_point) return acc[i];
         return (float)((double)reinterpret_cast<const long long*>(acc)[i] * (1.0 / (double)kFixedScale));
@@ -543,11 +544,15 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
         if (dk2) dk2[i] = (E)value(dk2acc, i);
         if (dv2) dv2[i] = (E)value(dv2acc, i);
         if (dqacc && dq) dq[i] = (E)(value(dqacc, i) * alpha);
+        if (dq0acc && dq) {  // query tile 0 was summed over its rounds in a [BH][32][D] accumulator
+            const size_t row = i / D, t = row % T;
+            if (t < 32) dq[i] = (E)(value(dq0acc, (row / T * 32 + t) * D + i % D) * alpha);
+        }
     }
 }
 
 struct BwdLayout {
-    size_t u, ut, k1t, k2t, v2t, delta, lse_f32, delta_f32, dk1acc, duacc, dk2acc, dv2acc, dqacc, total;
+    size_t u, ut, k1t, k2t, v2t, delta, lse_f32, delta_f32, dq0acc, dk1acc, duacc, dk2acc, dv2acc, dqacc, total;
 };
 static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     const size_t Tp = (size_t)(T + 63) / 64 * 64, n = (size_t)BH * T * D;
@@ -566,7 +571,8 @@ static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     l.v2t = take((size_t)BH * D * Tp * 2);
     l.delta = take((size_t)BH * T * 4);
     l.lse_f32 = take((size_t)BH * T * 4);    // fp32 tiles of the backward: their rows' LSE and Delta in fp32
-    l.delta_f32 = take((size_t)BH * T * 4);
+    l.delta_f32 = take(std::max((size_t)BH * T, (size_t)BH * 32 * 4 * 3) * 4);
+    l.dq0acc = take((size_t)BH * 32 * D * 8);  // dQ / alpha of query tile 0, summed over its rounds
     const size_t acc = fixed_point ? 8 : 4;
     l.dk1acc = take(n * acc);
     l.duacc = take(n * acc);
@@ -665,6 +671,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         FirstTileArgs f{};
         f.q = a.q; f.d_o = a.d_o; f.k1 = a.k1; f.u = u; f.k2 = a.k2; f.v2 = a.v2;
         f.lse_f32 = (float*)(ws + l.lse_f32); f.delta_f32 = (float*)(ws + l.delta_f32);
+        f.dq0_acc = ws + l.dq0acc;
         f.dq = a.dq; f.acc_k2 = dk2acc; f.acc_v2 = dv2acc; f.acc_k1 = dk1acc; f.acc_u = duacc; f.acc_q = dqacc;
         f.fixed_scale = a.deterministic ? kFixedScale : 0.f;
         f.BH = a.BH; f.T = a.T; f.D = D; f.is_bf16 = a.is_bf16;
@@ -698,7 +705,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     hipLaunchKernelGGL(bwd_finish_kernel<E>, dim3((unsigned)gridf), dim3(256), 0, st, (const float*)dk1acc,
                        (const float*)duacc, (const float*)dk2acc, (const float*)dv2acc, (const float*)dqacc, a.alpha,
                        (E*)a.dq, (const E*)a.v1, (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n,
-                       a.deterministic ? 1 : 0);
+                       a.deterministic ? 1 : 0,
+                       (first_in_f32 && !all_in_f32 && !dqacc) ? (const float*)(ws + l.dq0acc) : nullptr, a.T, D);
     return hipGetLastError();
 }
 

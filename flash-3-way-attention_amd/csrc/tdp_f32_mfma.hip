@@ -16,6 +16,8 @@
 // finished row b into the output, O^T[d, q] += Tv^T[d, q] * VB[b, d]) is lane-local.
 // With 64-cycle MFMAs the kernels are bound by the matrix pipe; the element-wise work (mask predicate on every
 // element, online softmax) hides under it, so there is one loop body for every mask.
+#include <algorithm>
+
 #include "common.hpp"
 #include "kernels.hpp"
 #include "mfma.hpp"
@@ -39,6 +41,12 @@ struct F32Params {
     // covered rows and delta their rowsum(dO * O) with O in fp32
     const E* d_o;
     float* delta;
+    // STATS over query tile 0 with the rounds dealt out to `split_rounds` workgroups (blockIdx.y): each writes its
+    // partial (maximum, sum, sum_d dO * unnormalised O) to delta[((bh * 32 + q) * split_rounds + round) * 3 ..] and
+    // the first one clears `zero_words` 4-byte words at zero_ptr + bh * zero_words
+    int split_rounds;
+    unsigned* zero_ptr;
+    int zero_words;
     int T, BH, nqt;  // nqt: query tiles this launch covers (tiles 0 .. nqt - 1)
     float scale_log2;
     TdpMask mask;  // in terms of the streamed index a and the row index b
@@ -140,7 +148,13 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
     }
 
     const Range rows = row_range(mask, q0, q1, T);
-    const int m_lo = rows.lo / NW, m_hi = rows.hi / NW;  // rounds of NW rows
+    int m_lo = rows.lo / NW, m_hi = rows.hi / NW;  // rounds of NW rows
+    if (STATS && p.split_rounds) {
+        m_lo = max(m_lo, (int)blockIdx.y);  // this workgroup's round only (none at all if it is out of range)
+        m_hi = min(m_hi, (int)blockIdx.y);
+        if (blockIdx.y == 0)
+            for (int idx = tid; idx < p.zero_words; idx += 512) p.zero_ptr[(size_t)bh * p.zero_words + idx] = 0u;
+    }
 
     f32x16 accO[DT];
 #pragma unroll
@@ -282,8 +296,14 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
         if (wave == 0 && g == 0 && q < T) {
             float dsum = 0.f;
             for (int d = 0; d < D; ++d) dsum += (float)p.d_o[base + (size_t)q * D + d] * sO[d * 33 + n];
-            p.delta[(size_t)bh * T + q] = dsum / L;
+            if (p.split_rounds) {
+                float* part = p.delta + (((size_t)bh * 32 + n) * p.split_rounds + blockIdx.y) * 3;
+                part[0] = M; part[1] = L; part[2] = dsum;
+            } else {
+                p.delta[(size_t)bh * T + q] = dsum / L;
+            }
         }
+        if (p.split_rounds) return;
     } else {
         for (int idx = tid; idx < 32 * D; idx += 512) {
             const int r = idx / D, d = idx % D;
@@ -327,6 +347,10 @@ struct F32BwdParams {
     E* dq;                 // WITH_DQ, when acc_q is null
     void *acc_k, *acc_v;   // [BH][T][D] gradients of the rows: fixed point (long long) or float
     void* acc_q;           // WITH_DQ: when non-null, dQ / alpha is added here instead of being written to dq
+    int acc_q_rows;        // 0: acc_q is [BH][T][D]; else it holds the first acc_q_rows queries only, [BH][rows][D]
+    // when non-null, LSE and Delta of query tile 0 come from the partials the split STATS launch left here
+    const float* stats_part;
+    int split_rounds;      // tile 0 only: rounds dealt out to workgroups (see tdp_f32_tile0_kernel), else 0
     float fixed_scale;     // scale of the fixed-point accumulators; 0: the accumulators are float
     int T, BH, nqt;        // nqt: query tiles this launch covers (tiles 0 .. nqt - 1)
     float alpha;
@@ -346,8 +370,9 @@ __device__ __forceinline__ void shared_add(void* acc, size_t idx, float v, float
         unsafeAtomicAdd(reinterpret_cast<float*>(acc) + idx, v);
 }
 
+// `only_round` >= 0: this workgroup walks that round of rows only
 template <typename E, int D, int DOUT, bool WITH_DQ>
-__global__ __launch_bounds__(512) void tdp_f32_bwd_kernel(F32BwdParams<E> p) {
+__device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_round) {
     constexpr int DTO = DOUT / 32, KS = D / 2, LD = D + 1, NW = kF32Waves;
     constexpr bool FLY = D > 64;  // form the B operands of the score products as they are used
     extern __shared__ __align__(16) float smem_f[];
@@ -386,11 +411,31 @@ __global__ __launch_bounds__(512) void tdp_f32_bwd_kernel(F32BwdParams<E> p) {
         sDO[r * LD + d] = (float)p.d_o[off];
     }
     // a query past the end of the sequence gets a huge LSE: its P is exactly 0
-    const float lse2 = q < T ? p.lse[(size_t)bh * T + q] * kLog2e : 1.0e30f;
-    const float delta = q < T ? p.delta[(size_t)bh * T + q] : 0.f;
+    float lse2 = 1.0e30f, delta = 0.f;
+    if (q < T) {
+        if (p.stats_part) {  // tile 0: join the partials of the rounds
+            const float* part = p.stats_part + ((size_t)bh * 32 + n) * p.split_rounds * 3;
+            float M = kNegBig, L = 0.f, num = 0.f;
+            for (int z = 0; z < p.split_rounds; ++z) M = fmaxf(M, part[z * 3]);
+            for (int z = 0; z < p.split_rounds; ++z) {
+                const float w = fast_exp2(part[z * 3] - M);
+                L += part[z * 3 + 1] * w;
+                num += part[z * 3 + 2] * w;
+            }
+            lse2 = M + fast_log2(L);
+            delta = num / L;
+        } else {
+            lse2 = p.lse[(size_t)bh * T + q] * kLog2e;
+            delta = p.delta[(size_t)bh * T + q];
+        }
+    }
 
     const Range rows = row_range(mask, q0, q1, T);
-    const int m_lo = rows.lo / NW, m_hi = rows.hi / NW;
+    int m_lo = rows.lo / NW, m_hi = rows.hi / NW;
+    if (only_round >= 0) {
+        m_lo = max(m_lo, only_round);
+        m_hi = min(m_hi, only_round);
+    }
 
     f32x16 accDQ[DTO];
 #pragma unroll
@@ -516,10 +561,33 @@ __global__ __launch_bounds__(512) void tdp_f32_bwd_kernel(F32BwdParams<E> p) {
             const int r = idx / DOUT, d = idx % DOUT;
             if (q0 + r < T) {
                 const size_t off = base + (size_t)(q0 + r) * D + c0 + d;
-                if (p.acc_q) shared_add(p.acc_q, off, sO[d * 33 + r], p.fixed_scale);
-                else p.dq[off] = (E)(sO[d * 33 + r] * p.alpha);
+                if (p.acc_q)
+                    shared_add(p.acc_q, p.acc_q_rows ? ((size_t)bh * p.acc_q_rows + q0 + r) * D + c0 + d : off,
+                               sO[d * 33 + r], p.fixed_scale);
+                else
+                    p.dq[off] = (E)(sO[d * 33 + r] * p.alpha);
             }
         }
+    }
+}
+
+template <typename E, int D, int DOUT, bool WITH_DQ>
+__global__ __launch_bounds__(512) void tdp_f32_bwd_kernel(F32BwdParams<E> p) {
+    f32_bwd_body<E, D, DOUT, WITH_DQ>(p, -1);
+}
+
+// Query tile 0 of a 16-bit backward, both launches' roles and all rounds at once: blockIdx.z = role * rounds + round
+// (role 0: rows = (K2, V2), with dQ; role 1: rows = (K1, U)).  A tile of 32 queries has at most four rounds of
+// eight rows; one workgroup walking them one after another is 4 x ~25 us of pure latency.
+template <typename E, int D, int DOUT>
+__global__ __launch_bounds__(512) void tdp_f32_tile0_kernel(F32BwdParams<E> r0, F32BwdParams<E> r1, int roles_mask) {
+    const int role = blockIdx.z / r0.split_rounds, round = blockIdx.z % r0.split_rounds;
+    if (!((roles_mask >> role) & 1)) return;
+    if (role == 0) {
+        if (roles_mask & 4) f32_bwd_body<E, D, DOUT, true>(r0, round);
+        else f32_bwd_body<E, D, DOUT, false>(r0, round);
+    } else {
+        f32_bwd_body<E, D, DOUT, false>(r1, round);
     }
 }
 
@@ -575,7 +643,8 @@ hipError_t launch_f32_bwd(const GenericTdpArgs& a, long long* acc, hipStream_t s
     const bool want_q = a.dq != nullptr, want_k2 = a.dk2 && a.dv2, want_k1 = a.dk1 && a.du;
     F32BwdParams<float> p{};
     p.q = a.q; p.d_o = a.d_o; p.lse = a.lse_in; p.delta = a.delta;
-    p.dq = a.dq; p.acc_q = nullptr; p.fixed_scale = kF32FixedScale;
+    p.dq = a.dq; p.acc_q = nullptr; p.acc_q_rows = 0; p.stats_part = nullptr; p.split_rounds = 0;
+    p.fixed_scale = kF32FixedScale;
     p.T = a.T; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha;
     size_t gz = (4 * n + 255) / 256;
@@ -603,6 +672,7 @@ hipError_t launch_f32_fwd(const GenericTdpArgs& a, hipStream_t st) {
     F32Params<float> p{};
     p.q = a.q; p.ka = a.k1; p.kb = a.k2; p.va = a.u; p.vb = a.v2;
     p.o = a.o; p.lse = a.lse;
+    p.d_o = nullptr; p.delta = nullptr; p.split_rounds = 0; p.zero_ptr = nullptr; p.zero_words = 0;
     p.T = a.T; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.scale_log2 = a.alpha * kLog2e;
     p.mask = TdpMask{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
@@ -625,6 +695,7 @@ static hipError_t launch_stats(const FirstTileArgs& a, hipStream_t st) {
     F32Params<E> p{};
     p.q = (const E*)a.q; p.ka = (const E*)a.k1; p.kb = (const E*)a.k2; p.va = (const E*)a.u; p.vb = (const E*)a.v2;
     p.o = nullptr; p.lse = a.lse_f32; p.d_o = (const E*)a.d_o; p.delta = a.delta_f32;
+    p.split_rounds = 0; p.zero_ptr = nullptr; p.zero_words = 0;
     p.T = a.T; p.BH = a.BH; p.nqt = a.tiles;
     p.scale_log2 = a.alpha * kLog2e;
     p.mask = TdpMask{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
@@ -635,8 +706,55 @@ static hipError_t launch_stats(const FirstTileArgs& a, hipStream_t st) {
     return hipGetLastError();
 }
 
+// Query tile 0 alone: the STATS pass and the backward pass, each with its rounds dealt out to workgroups.
+template <typename E, int D>
+static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
+    constexpr int DOUT = D > 64 ? 64 : D;
+    const int rounds = (std::min(a.T, 32) + kF32Waves - 1) / kF32Waves;
+    const int groups = (a.BH + 7) / 8;
+    const TdpMask natural{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
+    const bool own_dq_acc = a.want_q && !a.acc_q;  // dQ of the tile is summed over its rounds in a.dq0_acc
+    {
+        F32Params<E> p{};
+        p.q = (const E*)a.q; p.ka = (const E*)a.k1; p.kb = (const E*)a.k2; p.va = (const E*)a.u; p.vb = (const E*)a.v2;
+        p.o = nullptr; p.lse = nullptr; p.d_o = (const E*)a.d_o; p.delta = a.delta_f32;
+        p.split_rounds = rounds;
+        p.zero_ptr = own_dq_acc ? (unsigned*)a.dq0_acc : nullptr;
+        p.zero_words = own_dq_acc ? 32 * D * (a.fixed_scale != 0.f ? 2 : 1) : 0;
+        p.T = a.T; p.BH = a.BH; p.nqt = 1;
+        p.scale_log2 = a.alpha * kLog2e;
+        p.mask = natural;
+        auto kern = tdp_f32_fwd_kernel<E, D, true>;
+        constexpr size_t smem = f32_fwd_smem<D>();
+        if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(8 * groups, rounds), dim3(512), smem, st, p);
+    }
+    F32BwdParams<E> r0{};
+    r0.q = (const E*)a.q; r0.d_o = (const E*)a.d_o; r0.lse = nullptr; r0.delta = nullptr;
+    r0.stats_part = a.delta_f32; r0.split_rounds = rounds;
+    r0.dq = (E*)a.dq; r0.acc_q = a.acc_q ? a.acc_q : a.dq0_acc; r0.acc_q_rows = a.acc_q ? 0 : 32;
+    r0.fixed_scale = a.fixed_scale;
+    r0.T = a.T; r0.BH = a.BH; r0.nqt = 1; r0.alpha = a.alpha;
+    F32BwdParams<E> r1 = r0;
+    r0.ka = (const E*)a.k1; r0.va = (const E*)a.u; r0.kb = (const E*)a.k2; r0.vb = (const E*)a.v2;
+    r0.acc_k = a.acc_k2; r0.acc_v = a.acc_v2; r0.mask = natural;
+    r1.ka = (const E*)a.k2; r1.va = (const E*)a.v2; r1.kb = (const E*)a.k1; r1.vb = (const E*)a.u;
+    r1.acc_k = a.acc_k1; r1.acc_v = a.acc_u;
+    r1.mask = TdpMask{natural.causal, natural.wb, natural.wa, natural.rab, natural.lab};
+    const int roles = ((a.want_q || a.want_k2) ? 1 : 0) | (a.want_k1 ? 2 : 0) | (a.want_q ? 4 : 0);
+    auto kern = tdp_f32_tile0_kernel<E, D, DOUT>;
+    constexpr size_t smem = f32_bwd_smem<D>();
+    if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(8 * groups, D / DOUT, 2 * rounds), dim3(512), smem, st, r0, r1, roles);
+    return hipGetLastError();
+}
+
 template <typename E>
 static hipError_t first_tile_typed(const FirstTileArgs& a, hipStream_t st) {
+    if (a.tiles == 1) {
+        return a.D == 32 ? launch_tile0_split<E, 32>(a, st) : a.D == 64 ? launch_tile0_split<E, 64>(a, st)
+             : a.D == 128 ? launch_tile0_split<E, 128>(a, st) : hipErrorInvalidValue;
+    }
     // the rows' log-sum-exp and Delta once more, in fp32 from the same tensors: the saved LSE carries the 16-bit
     // rounding of the forward's scores and Delta that of the stored output, and nearly one-hot rows show both
     hipError_t es = a.D == 32 ? launch_stats<E, 32>(a, st) : a.D == 64 ? launch_stats<E, 64>(a, st)
@@ -644,7 +762,8 @@ static hipError_t first_tile_typed(const FirstTileArgs& a, hipStream_t st) {
     if (es != hipSuccess) return es;
     F32BwdParams<E> p{};
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o; p.lse = a.lse_f32; p.delta = a.delta_f32;
-    p.dq = (E*)a.dq; p.acc_q = a.acc_q; p.fixed_scale = a.fixed_scale;
+    p.dq = (E*)a.dq; p.acc_q = a.acc_q; p.acc_q_rows = 0; p.stats_part = nullptr; p.split_rounds = 0;
+    p.fixed_scale = a.fixed_scale;
     p.T = a.T; p.BH = a.BH; p.nqt = a.tiles;
     p.alpha = a.alpha;
     const TdpMask natural{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
