@@ -1,4 +1,4 @@
-// Triple-dot-product trittention in true fp32 on the matrix cores (v_mfma_f32_32x32x2_f32), D = 32 or 64,
+// Triple-dot-product trittention in true fp32 on the matrix cores (v_mfma_f32_32x32x2_f32), D = 32, 64 or 128,
 // every mask.  This is the path of fp32 tensors: fp32 operands, fp32 products, fp32 accumulation (the 1e-4
 // relative bar), at the fp32 matrix rate (157 TFLOP/s peak) instead of the fp32 vector rate of the VALU kernels.
 //
@@ -687,7 +687,7 @@ hipError_t launch_f32_fwd(const GenericTdpArgs& a, hipStream_t st) {
 
 }  // namespace
 
-bool f32_mfma_tdp_supported(int D) { return D == 32 || D == 64; }
+bool f32_mfma_tdp_supported(int D) { return D == 32 || D == 64 || D == 128; }
 
 // The first query tiles of a 16-bit backward, in fp32 (see the comment above tdp_f32_bwd_kernel).
 template <typename E, int D>
@@ -784,6 +784,7 @@ hipError_t f32_mfma_tdp_bwd_first_tile(const FirstTileArgs& a, hipStream_t st) {
 hipError_t f32_mfma_tdp_fwd(const GenericTdpArgs& a, hipStream_t st) {
     if (a.D == 32) return launch_f32_fwd<32>(a, st);
     if (a.D == 64) return launch_f32_fwd<64>(a, st);
+    if (a.D == 128) return launch_f32_fwd<128>(a, st);
     return hipErrorInvalidValue;
 }
 
@@ -792,6 +793,7 @@ size_t f32_mfma_tdp_bwd_scratch_elems(int BH, int T, int D) { return 4 * (size_t
 hipError_t f32_mfma_tdp_bwd(const GenericTdpArgs& a, long long* scratch, hipStream_t st) {
     if (a.D == 32) return launch_f32_bwd<32>(a, scratch, st);
     if (a.D == 64) return launch_f32_bwd<64>(a, scratch, st);
+    if (a.D == 128) return launch_f32_bwd<128>(a, scratch, st);
     return hipErrorInvalidValue;
 }
 

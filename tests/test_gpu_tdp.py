@@ -62,6 +62,25 @@ def test_head_dims_fp32(D):
     check_all(inputs, 1 / math.sqrt(D), True)
 
 
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("causal,windows", [(True, (None,) * 4), (False, (None,) * 4), (True, (100, 40, 24, 7)),
+                                            (True, (3, 200, 0, 2))])
+def test_fp32_tensors_on_the_matrix_cores(D, causal, windows, tune):
+    """fp32 tensors on the fp32 MFMA kernels (enough query tiles for the launcher to pick them; ragged length):
+    forward and all five gradients at the fp32 bar, and against the fp32 VALU kernels of the same library."""
+    print(f"case fp32 mfma D={D} causal={causal} {windows}", flush=True)
+    inputs = orc.make_inputs(2, 4, 250, D, torch.float32, seed=D + 3)
+    alpha = 1 / math.sqrt(D)
+    check_all(inputs, alpha, causal, windows)
+    out, g = util.run_tdp(inputs, alpha, causal, windows)
+    tune(_lib.TUNE_F32_VALU, 1)
+    out_v, g_v = util.run_tdp(inputs, alpha, causal, windows)
+    assert not torch.equal(out, out_v), "both runs took the same kernels"
+    util.assert_close("out vs VALU kernels", out, out_v, **FP32)
+    for name, a, b in zip(util.NAMES, g, g_v):
+        util.assert_close(f"{name} vs VALU kernels", a, b, **FP32)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_config2_lowp_forward_backward(dtype):
     """B=2 H=4 T=256 D=64, 16-bit tensors with fp32 accumulation, all five gradients."""
