@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
-from .. import _lib
+from .. import _lib, _ops
 from ..triple_dot_product.utils import clamp_window
 
 
@@ -39,22 +39,15 @@ class TrittentionTritonFunction(torch.autograd.Function):
         B, H, T, D = q.shape
         if D not in (16, 32, 64, 128):
             raise ValueError(f"head_dim must be one of 16, 32, 64, 128, got {D}")
-        code = _lib.dtype_code(q.dtype)
-        _lib.require_gpu(q, "TrittentionTriton")
-        q, k1, k2, v1, v2 = (_lib.dense(t) for t in (q, k1, k2, v1, v2))
+        _lib.dtype_code(q.dtype)
+        q, k1, k2, v1, v2 = (t.contiguous() for t in (q, k1, k2, v1, v2))
         k_diff = clamp_window(k_diff, T, "k_diff")
-        flags = getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
+        compiling = _ops.compiling()
+        flags = _lib.FLAG_AUTO if compiling else getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
         if convert_to_float32 and not flags & _lib.FLAG_FORCE_MFMA:
             flags |= _lib.FLAG_FORCE_GENERIC  # fp32 operands throughout (trittention_triton.py:92-98 of the reference)
-        lib = _lib.lib()
-        o = torch.empty_like(q)
-        m = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
-        with torch.cuda.device(q.device):
-            ws = _lib.workspace(lib.tritt_dps_fwd_workspace_bytes(B, H, T, D, code, flags), q.device)
-            st = lib.tritt_dps_fwd(_lib.ptr(q), _lib.ptr(k1), _lib.ptr(k2), _lib.ptr(v1), _lib.ptr(v2), _lib.ptr(o),
-                                   _lib.ptr(m), B, H, T, D, code, float(softmax_scale), int(bool(causal)), k_diff,
-                                   _lib.ptr(ws), ws.numel(), flags, _lib.stream_ptr(q.device))
-        _lib.check(st, "tritt_dps_fwd")
+        call = torch.ops.flash_trittention.dps_fwd if compiling else _ops.dps_fwd_impl
+        o, m = call(q, k1, k2, v1, v2, float(softmax_scale), bool(causal), k_diff, flags)
         ctx.save_for_backward(q, k1, k2, v1, v2, o, m)
         ctx.causal = bool(causal)
         ctx.softmax_scale = float(softmax_scale)
@@ -66,21 +59,13 @@ class TrittentionTritonFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output, m_grad=None):
         q, k1, k2, v1, v2, o, m = ctx.saved_tensors
-        B, H, T, D = q.shape
         assert grad_output.shape == o.shape, f"Shape mismatch: O={o.shape}, dO={grad_output.shape}"
         assert o.device == grad_output.device, "O and dO must be on the same device"
         assert o.dtype == grad_output.dtype, "O and dO must have the same dtype"
-        grad_output = _lib.dense(grad_output)
-        lib = _lib.lib()
-        code = _lib.dtype_code(q.dtype)
-        dq, dk1, dk2, dv1, dv2 = (torch.empty_like(q) for _ in range(5))
-        with torch.cuda.device(q.device):
-            ws = _lib.workspace(lib.tritt_dps_bwd_workspace_bytes(B, H, T, D, code, ctx.flags), q.device)
-            st = lib.tritt_dps_bwd(_lib.ptr(q), _lib.ptr(k1), _lib.ptr(k2), _lib.ptr(v1), _lib.ptr(v2), _lib.ptr(o),
-                                   _lib.ptr(m), _lib.ptr(grad_output), _lib.ptr(dq), _lib.ptr(dk1), _lib.ptr(dk2),
-                                   _lib.ptr(dv1), _lib.ptr(dv2), B, H, T, D, code, ctx.softmax_scale, int(ctx.causal),
-                                   ctx.k_diff, _lib.ptr(ws), ws.numel(), ctx.flags, _lib.stream_ptr(q.device))
-        _lib.check(st, "tritt_dps_bwd")
+        grad_output = grad_output.contiguous()
+        call = torch.ops.flash_trittention.dps_bwd if _ops.compiling() else _ops.dps_bwd_impl
+        dq, dk1, dk2, dv1, dv2 = call(q, k1, k2, v1, v2, o, m, grad_output, ctx.softmax_scale, ctx.causal, ctx.k_diff,
+                                      ctx.flags)
         return dq, dk1, dk2, dv1, dv2, None, None, None, None, None
 
 

@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
-from .. import _lib
+from .. import _lib, _ops
 from .utils import process_masking_variables
 
 
@@ -48,31 +48,20 @@ class FlashTrittention(torch.autograd.Function):
     def forward(ctx, Q, K1, K2, V1, V2, softmax_scale, kk_left, kk_right, k1_window, k2_window, causal,
                 convert_to_float32):
         _validate(Q, (("K1", K1), ("K2", K2), ("V1", V1), ("V2", V2)))
-        _lib.require_gpu(Q, "flash_trittention")
-        B, H, T, D = Q.shape
-        Q, K1, K2, V1, V2 = (_lib.dense(t) for t in (Q, K1, K2, V1, V2))
+        T = Q.shape[2]
+        Q, K1, K2, V1, V2 = (t.contiguous() for t in (Q, K1, K2, V1, V2))
         k1_window, k2_window, kk_left, kk_right = process_masking_variables(T, k1_window, k2_window, kk_left, kk_right)
         causal = bool(causal)
-        flags = getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
+        compiling = _ops.compiling()  # tracing: the implementation flags are the class default
+        flags = _lib.FLAG_AUTO if compiling else getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
         if torch.are_deterministic_algorithms_enabled():
             flags &= ~_lib.FLAG_FLOAT_ATOMICS  # the default (fixed-point accumulation) is bitwise reproducible
         if convert_to_float32 and not flags & _lib.FLAG_FORCE_MFMA:
             # the reference forms its scores in fp32 under this flag (flash_trittention.py:408, bwd_dq.py:197); here
             # 16-bit tensors then take the fp32 kernels: fp32 operands and products throughout, 16-bit results
             flags |= _lib.FLAG_FORCE_GENERIC
-        lib = _lib.lib()
-        code = _lib.dtype_code(Q.dtype)
-        O = torch.empty_like(Q)
-        LSE = torch.empty((B, H, T), dtype=torch.float32, device=Q.device)
-        with torch.cuda.device(Q.device):
-            need = lib.tritt_tdp_fwd_workspace_bytes(B, H, T, D, code, int(causal), k1_window, k2_window, kk_left,
-                                                     kk_right, flags)
-            ws = _lib.workspace(need, Q.device)
-            st = lib.tritt_tdp_fwd(_lib.ptr(Q), _lib.ptr(K1), _lib.ptr(K2), _lib.ptr(V1), _lib.ptr(V2), _lib.ptr(O),
-                                   _lib.ptr(LSE), B, H, T, D, code, float(softmax_scale), int(causal), k1_window,
-                                   k2_window, kk_left, kk_right, _lib.ptr(ws), ws.numel(), flags,
-                                   _lib.stream_ptr(Q.device))
-        _lib.check(st, "tritt_tdp_fwd")
+        call = torch.ops.flash_trittention.tdp_fwd if compiling else _ops.tdp_fwd_impl
+        O, LSE = call(Q, K1, K2, V1, V2, float(softmax_scale), causal, k1_window, k2_window, kk_left, kk_right, flags)
         ctx.save_for_backward(Q, K1, K2, V1, V2, O, LSE)
         ctx.softmax_scale = float(softmax_scale)
         ctx.windows = (k1_window, k2_window, kk_left, kk_right)
@@ -83,30 +72,22 @@ class FlashTrittention(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dO):
         Q, K1, K2, V1, V2, O, LSE = ctx.saved_tensors
-        B, H, T, D = Q.shape
         if dO.dtype != Q.dtype:
             dO = dO.to(Q.dtype)
-        dO = _lib.dense(dO)
+        dO = dO.contiguous()
         k1_window, k2_window, kk_left, kk_right = ctx.windows
-        lib = _lib.lib()
-        code = _lib.dtype_code(Q.dtype)
-        # only the gradients autograd asks for: a null pointer tells the library to skip one (and the kernel launch
-        # that serves nothing else)
-        wanted = list(getattr(ctx, "needs_input_grad", (True,) * 5)[:5])
-        grads = [torch.empty_like(Q) if w else None for w in wanted]
-        dq, dk1, dk2, dv1, dv2 = grads
-        gptr = lambda t: _lib.ptr(t) if t is not None else None
-        with torch.cuda.device(Q.device):
-            need = lib.tritt_tdp_bwd_workspace_bytes(B, H, T, D, code, int(ctx.causal), k1_window, k2_window, kk_left,
-                                                     kk_right, ctx.flags)
-            ws = _lib.workspace(need, Q.device)
-            st = lib.tritt_tdp_bwd(_lib.ptr(Q), _lib.ptr(K1), _lib.ptr(K2), _lib.ptr(V1), _lib.ptr(V2), _lib.ptr(O),
-                                   _lib.ptr(LSE), _lib.ptr(dO), gptr(dq), gptr(dk1), gptr(dk2),
-                                   gptr(dv1), gptr(dv2), B, H, T, D, code, ctx.softmax_scale, int(ctx.causal),
-                                   k1_window, k2_window, kk_left, kk_right, _lib.ptr(ws), ws.numel(), ctx.flags,
-                                   _lib.stream_ptr(Q.device))
-        _lib.check(st, "tritt_tdp_bwd")
-        return dq, dk1, dk2, dv1, dv2, None, None, None, None, None, None, None
+        # only the gradients autograd asks for: the library skips the others (and the kernel launch that serves
+        # nothing else)
+        needs = getattr(ctx, "needs_input_grad", (True,) * 5)
+        wanted = sum(1 << i for i in range(5) if needs[i])
+        if _ops.compiling():
+            grads = torch.ops.flash_trittention.tdp_bwd(Q, K1, K2, V1, V2, O, LSE, dO, ctx.softmax_scale, ctx.causal,
+                                                        k1_window, k2_window, kk_left, kk_right, ctx.flags, wanted)
+            grads = [g if needs[i] else None for i, g in enumerate(grads)]
+        else:
+            grads = _ops.tdp_bwd_impl(Q, K1, K2, V1, V2, O, LSE, dO, ctx.softmax_scale, ctx.causal, k1_window, k2_window,
+                                      kk_left, kk_right, ctx.flags, wanted)
+        return (*grads, None, None, None, None, None, None, None)
 
 
 def flash_trittention(q, k1, k2, v1, v2, softmax_scale=1 / 8, kk_left=1, kk_right=1, k1_window=1, k2_window=1,
