@@ -19,11 +19,21 @@ __device__ __forceinline__ constexpr int swz_perm(int r) {
 }
 __device__ __forceinline__ constexpr int swz_seq(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 
-// one 1 KB block: `gbase` is wave-uniform, `byte_off` per lane, `lds_dst` wave-uniform
+// one 1 KB block: `gbase` is wave-uniform, `byte_off` per lane, `lds_dst` wave-uniform.
+// Written as inline assembly on purpose.  The compiler treats the builtin form of this load as an access that may
+// touch both global memory and LDS, and while one is outstanding its wait-count insertion turns every wait for an
+// LDS read into lgkmcnt(0): in loops that keep stage loads in flight all the time (every kernel here) an operand
+// read issued a phase ahead was then waited for together with the reads issued after it, and the prefetch bought
+// nothing.  Seen as an opaque statement, the load leaves the compiler's counting of LDS reads exact; the callers
+// wait for these loads themselves (wait_vmcnt / barrier_keep_loads), as they had to before.  A wait that the
+// compiler computes for its own vector-memory loads can only become more conservative by loads it does not know.
+// M0 (the LDS base of the load) is a reserved register that nothing else in these kernels uses.
 __device__ __forceinline__ void direct_load_16(const void* gbase, unsigned byte_off, void* lds_dst) {
-    __builtin_amdgcn_global_load_lds(
-        (const __attribute__((address_space(1))) void*)(static_cast<const char*>(gbase) + byte_off),
-        (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
+    const unsigned lds = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds), "v"(byte_off), "s"(gbase)
+                 : "memory");
 }
 
 // make a wave-uniform pointer provably scalar (keeps it in SGPRs instead of spilled VGPR pairs)

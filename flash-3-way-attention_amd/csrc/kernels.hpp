@@ -11,7 +11,7 @@ struct Knobs {
     int fwd_splits;      // TRITT_TUNE_FWD_SPLITS / env TRITT_FWD_SPLITS: workgroups per query tile, forward (1..8)
     int fwd_band;        // TRITT_TUNE_FWD_BAND / env TRITT_FWD_BAND: -1 switches the band-resident forward off
     int bwd_splits;      // TRITT_TUNE_BWD_SPLITS / env TRITT_BWD_SPLITS: workgroups per query tile, backward (1..16)
-    int bwd128_variant;  // TRITT_TUNE_BWD128_WAVES / env TRITT_BWD128_VARIANT=w8|w4: 8 or 4 waves per workgroup
+    int bwd128_variant;  // TRITT_TUNE_BWD128_WAVES / env TRITT_BWD128_VARIANT=w8|w4: the 32-query kernels (default: 16 queries per wave)
     int f32_valu;        // TRITT_TUNE_F32_VALU: 1 = fp32 tensors take the VALU kernels at every head dimension
 };
 Knobs knobs();

@@ -65,6 +65,7 @@ __device__ __forceinline__ void accumulate(const BwdParams<E>& p, float* acc, si
 }  // namespace tritt
 
 #include "tdp_bwd_rows_general.hpp"
+#include "tdp_bwd_rows_q16.hpp"
 
 namespace tritt {
 
@@ -633,12 +634,16 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         kern_nodq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), false, 8, 64, true>;
         col_parts = D / 64;
     } else if constexpr (D == 128) {
-        // Two waves per SIMD, 64 gradient columns per workgroup (S and dP computed by both column halves) is the
-        // faster shape at every grid size measured, now that it fits the register file without scratch memory;
-        // the one-wave-per-SIMD shape with all 128 columns stays selectable.
-        // TRITT_BWD128_VARIANT=w8 / w4 overrides the choice.
-        const bool w8 = knobs().bwd128_variant != 4;
-        if (w8) {
+        // Default: 16 queries per wave on 16x16x32 tiles, every gradient column in one wave, S and dP formed once
+        // (tdp_bwd_rows_q16.hpp).  The two 32-query shapes stay selectable (TRITT_TUNE_BWD128_WAVES = 8 | 4,
+        // TRITT_BWD128_VARIANT=w8 | w4): two waves per SIMD with 64 gradient columns per workgroup (S and dP
+        // computed by both column halves), or one wave per SIMD with all 128 columns.
+        const int variant = knobs().bwd128_variant;
+        if (variant != 4 && variant != 8) {
+            smem = bwd_q16_smem();
+            kern_dq = tdp_bwd_rows_q16_kernel<E, true>;
+            kern_nodq = tdp_bwd_rows_q16_kernel<E, false>;
+        } else if (variant == 8) {
             smem = bwdg_smem(128, 8, 64, true);
             kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 8, 64, false>;
             kern_nodq = tdp_bwd_rows_general_kernel<E, 128, false, 8, 64, false>;

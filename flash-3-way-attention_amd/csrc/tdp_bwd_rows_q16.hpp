@@ -1,0 +1,412 @@
+// Triple-dot-product trittention backward on MFMA, head dimension 128, full causal windows or no mask
+// (included by tdp_bwd_mfma.hip after BwdParams): the rows kernel on 16x16x32 tiles.
+//
+// Same decomposition as tdp_bwd_rows_kernel (one K2/V2 row k per wave and round, K1 / U streamed over j in
+// stages shared by the workgroup), but a wave owns 16 queries instead of 32.  The accumulators Yq / Tv of
+// all 128 gradient columns are then 2 x 32 registers, so one wave holds every column and S and dP are
+// computed once per (query, row, key): a 32-key step is 16 + 16 MFMAs of 16x16x32 = the work of 16
+// 32x32x16 MFMAs, where the 32-query form, which has to split the columns over two workgroups that both
+// form S and dP, executes 26.  The price is LDS operand traffic: every MFMA reads one operand from LDS
+// (32 KB per step and wave), twice the bytes per flop of the 32x32 form.
+//
+// v_mfma_f32_16x16x32_{bf16,f16}: D[16x16] = A[16x32] * B[32x16] + C.
+//   A operand: lane l holds A[row = l%16][k = 8*(l/16) .. +8]
+//   B operand: lane l holds B[k = 8*(l/16) .. +8][col = l%16]
+//   C/D:       lane l holds D[row = 4*(l/16) + i][col = l%16], i = 0..3
+// Score tiles are computed transposed (rows = keys, columns = queries), two 16-key tiles per step, and
+// the K1 rows fed to tile t are permuted (MFMA row r holds key 8 (r / 4) + 4 t + r % 4) so that the eight
+// values a lane gets from the two tiles are keys 8 (l/16) .. +7: exactly its k-slots of the A operand of
+// the gradient products, no cross-lane movement.  -LSE2[q] and -Delta[q] are lane constants (column =
+// query) and enter as resident 4-register C operands; an invalid (q, j, k) gets -3e4 there instead.
+//
+// Workgroup = 32 queries x 4 rows per round: wave w takes query half w & 1 and row w >> 1.  Stages are 32
+// keys of K1, U (row-major, 128-byte tile rows, 16-byte chunks swizzled for the permuted 16-row reads) and
+// K1^T, U^T ([128 d][32 keys], 64-byte rows); three buffers, fetched direct-to-LDS two steps ahead, one
+// workgroup barrier per step.  dQ is summed over the rounds in registers and over the waves at the end.
+#pragma once
+
+namespace tritt {
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <typename E>
+struct Mma16;
+template <>
+struct Mma16<__bf16> {
+    static __device__ __forceinline__ f32x4 mma(bf16x8 a, bf16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma16<_Float16> {
+    static __device__ __forceinline__ f32x4 mma(f16x8 a, f16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// key offset (0..31) that sits in MFMA row r of the K1-style operand of 16-key tile t
+__device__ __forceinline__ constexpr int q16_key(int t, int r) { return 8 * (r >> 2) + 4 * t + (r & 3); }
+// Chunk swizzles of the stage tiles.  A 16-byte LDS read is served in four passes of 16 lanes, {0-3, 12-15, 20-27},
+// {32-35, 44-47, 52-59}, {4-11, 16-19, 28-31}, {36-43, 48-51, 60-63} (measured: lanes of different passes never
+// collide), and the 16 lanes of a pass must fall on 16 distinct 16-byte bank groups (address / 16 mod 16).
+// Row-major tiles (128-byte rows): chunk c of key row r sits at position c ^ swz_q16(r); transposed tiles (64-byte
+// rows): chunk c of column d at c ^ swz_t16(d).  Both were found by searching the xor swizzles under that rule
+// for the 16-row operand reads below and confirmed on the hardware (2.8 cycles per wave-wide read, the rate of a
+// linear read; the swizzles of the 32-row kernels cost 4.3-5 cycles under these reads).
+__device__ __forceinline__ constexpr int swz_q16(int r) { return (r & 2) | ((r >> 1) & 4); }
+__device__ __forceinline__ constexpr int swz_t16(int d) { return (d >> 1) & 2; }
+
+constexpr size_t bwd_q16_smem() {
+    return 3 * (size_t)(4 * 32 * 128 * 2)    // stage buffers
+           + 2 * (size_t)(2 * 4 * 128 * 2)   // K2 / V2 rows of two rounds
+           + 2 * (size_t)(32 * (128 + 8) * 2);  // Q and dO tiles
+}
+
+template <typename E, bool WITH_DQ>
+__global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
+    using M = Mma<E>;
+    using M16 = Mma16<E>;
+    using v8 = typename M::v8;
+    using v2 = typename M::v2;
+    constexpr int D = 128, KS = D / 32, DT = D / 16, BQ = 32, NW = 8, RPR = 4, NTH = 64 * NW;
+    constexpr int LDK = D + 8;
+    constexpr int NBUF = 3, LW = 4;  // stage buffers; direct loads per wave per stage (32 blocks of 1 KB)
+    constexpr int TILE = 32 * D;     // elements of one tensor's part of a stage
+    constexpr int STAGE = 4 * TILE;
+
+    extern __shared__ __align__(16) char smem[];
+    E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows | U rows | K1^T | U^T]
+    E* sKr = sStage + NBUF * STAGE;          // [2][RPR][D]
+    E* sVr = sKr + 2 * RPR * D;
+    E* sQb = sVr + 2 * RPR * D;              // [BQ][LDK]
+    E* sOb = sQb + BQ * LDK;
+
+    const int groups = (p.BH + 7) / 8;
+    const int xcd = blockIdx.x & 7;
+    int slot = blockIdx.x >> 3;
+    const int split = slot % p.splits;  // which share of the tile's rounds this workgroup walks
+    slot /= p.splits;
+    const int bh = (slot % groups) * 8 + xcd;
+    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
+    if (bh >= p.BH) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, grp = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = wave & 1, rrow = wave >> 1;
+    const int T = p.T;
+    const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
+    const E* __restrict__ K2 = p.row_k + base;
+    const E* __restrict__ V2 = p.row_v + base;
+
+    const int q0 = qt * BQ;
+    const int qlast = min(T - 1, q0 + BQ - 1);
+    const int jend = p.causal ? qlast : T - 1;
+    const int jfull = p.causal ? q0 : T - 1;
+    const int nsteps = jend / 32 + 1, nrounds = jend / RPR + 1;
+    const int per_split = (nrounds + p.splits - 1) / p.splits;
+    const int m_lo = split * per_split, m_hi = min(nrounds, m_lo + per_split);
+    if (m_lo >= m_hi) return;  // fewer rounds than shares (uniform over the workgroup, before any barrier)
+    const int q = q0 + 16 * half + n;
+    const bool q_ok = q < T;
+    const int jq = p.causal ? min(q, T - 1) : T - 1;
+    const float scale_log2 = p.alpha * kLog2e;
+
+    // ---- stage loader: wave w fetches blocks 4 w .. 4 w + 3 of
+    //   8 blocks of K1 rows, 8 of U rows (tile rows 8 b .. 8 b + 7), 8 of K1^T, 8 of U^T (16 d-rows each);
+    //   row-major tensors: blocks 0..3 are keys 0..31 of columns 0..63, blocks 4..7 the same keys of columns 64..127
+    const bool row_major = wave < 4;
+    const E* gsrc = uniform_ptr(wave < 2 ? p.st_k + base : wave < 4 ? p.st_v + base : wave < 6 ? p.st_kt + tbase : p.st_vt + tbase);
+    unsigned grest[LW];  // per-lane byte offset apart from the key term
+    int gkey[LW];        // row-major blocks: key offset of this lane's row inside the stage
+#pragma unroll
+    for (int c = 0; c < LW; ++c) {
+        const int b = (wave & 1) * LW + c;  // block inside its tensor
+        if (row_major) {
+            const int R = b * 8 + (lane >> 3), hh = R >> 5, r = R & 31;
+            gkey[c] = r;
+            grest[c] = (unsigned)(hh * 64 + (((lane & 7) ^ swz_q16(r)) * 8)) * 2;
+        } else {
+            const int dl = b * 16 + (lane >> 2);
+            gkey[c] = 0;
+            grest[c] = ((unsigned)dl * p.Tp + (((lane & 3) ^ swz_t16(dl)) * 8)) * 2;
+        }
+    }
+    auto issue_stage = [&](int st, int buf) {
+        const int jb = st * 32;
+        char* dst = reinterpret_cast<char*>(sStage + buf * STAGE) + wave * LW * 1024;
+#pragma unroll
+        for (int c = 0; c < LW; ++c) {
+            // row-major rows past the end of the sequence are clamped (their keys are masked); the transposed
+            // tensors are zero padded
+            const unsigned off = grest[c] + (row_major ? (unsigned)min(jb + gkey[c], T - 1) * (D * 2) : (unsigned)jb * 2);
+            direct_load_16(gsrc, off, dst + c * 1024);
+        }
+    };
+    // the round's K2 / V2 rows RPR m .. RPR m + 3: one 1 KB load per tensor
+    auto issue_round = [&](int m, int buf) {
+        if (wave < 2) {
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const unsigned off = (unsigned)min(m * RPR + (ln >> 4), T - 1) * (D * 2) + (ln & 15) * 16;
+            direct_load_16(uniform_ptr(wave ? V2 : K2), off, (wave ? sVr : sKr) + buf * RPR * D);
+        }
+    };
+
+    // ---- prologue
+    for (int idx = tid; idx < BQ * D; idx += NTH) {
+        const int r = idx / D, d = idx % D;
+        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
+        sQb[r * LDK + d] = p.q[off];
+        sOb[r * LDK + d] = p.d_o[off];
+    }
+    int st_ahead = 0;
+    auto advance = [&]() { st_ahead = st_ahead + 1 < nsteps ? st_ahead + 1 : 0; };
+    issue_round(m_lo, m_lo & 1);
+    issue_stage(st_ahead, 0);
+    advance();
+    issue_stage(st_ahead, 1);
+    advance();
+    int gstage = 0;
+
+    const float lse2 = q_ok ? p.lse[(size_t)bh * T + q] * kLog2e : 3.0e4f;
+    const float delta = q_ok ? p.delta[(size_t)bh * T + q] : 0.f;
+    const f32x4 c_lse = {-lse2, -lse2, -lse2, -lse2};
+    const f32x4 c_delta = {-delta, -delta, -delta, -delta};
+
+    [[maybe_unused]] f32x4 accDQ[DT];
+    if constexpr (WITH_DQ) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) accDQ[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // per-lane element offsets of the operand reads inside a stage tile
+    int roff[2];  // row operands of j-tile t: row q16_key(t, n), chunk position (c ^ swizzle) added per k-step
+#pragma unroll
+    for (int t = 0; t < 2; ++t) roff[t] = q16_key(t, n) * 64;
+    const int rswz = swz_q16(q16_key(0, n));  // the same for both tiles: the swizzle ignores bit 2 of the key
+
+    // Operand registers: two sets of eight 16-byte operands.  Every LDS batch is issued one phase before the MFMAs
+    // that use it: while one set feeds the matrix pipe the other is being filled.
+    //   rows batch b of a stage: set.a[2 t + kk] = K1 operand of key tile t, k-step 2 b + kk; set.u = the same of U
+    //   column batch b:          set.a[x] = U^T operand of column tile 4 b + x; set.u[x] = the same of K1^T
+    struct OperandSet {
+        v8 a[4], u[4];
+    };
+    OperandSet X, Y;
+    auto read_rows = [&](const E* sb, int b, OperandSet& o) {
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const int ks = 2 * b + kk;
+            const int coff = (ks >> 1) * 32 * 64 + ((((ks & 1) * 4 + grp) ^ rswz) * 8);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                o.a[2 * t + kk] = *reinterpret_cast<const v8*>(sb + roff[t] + coff);
+                o.u[2 * t + kk] = *reinterpret_cast<const v8*>(sb + TILE + roff[t] + coff);
+            }
+        }
+    };
+    auto read_cols = [&](const E* sb, int b, OperandSet& o) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int d = (4 * b + x) * 16 + n;
+            const int toff = d * 32 + ((grp ^ swz_t16(d)) * 8);
+            o.a[x] = *reinterpret_cast<const v8*>(sb + 3 * TILE + toff);
+            o.u[x] = *reinterpret_cast<const v8*>(sb + 2 * TILE + toff);
+        }
+    };
+    // stage 0 and the first round's rows have landed for every wave
+    barrier_keep_loads<LW>();
+    read_rows(sStage, 0, X);
+
+    for (int m = m_lo; m < m_hi; ++m) {
+        const int mb = m & 1;
+        const int k = m * RPR + rrow;
+
+        // B operands of the score products of this round: alpha log2e Q (.) K2[k] and dO (.) V2[k]
+        v8 bq[KS], bg[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int off = ks * 32 + grp * 8;
+            const v8 kv = *reinterpret_cast<const v8*>(sKr + (mb * RPR + rrow) * D + off);
+            const v8 vv = *reinterpret_cast<const v8*>(sVr + (mb * RPR + rrow) * D + off);
+            const v8 qv = *reinterpret_cast<const v8*>(sQb + (16 * half + n) * LDK + off);
+            const v8 dv = *reinterpret_cast<const v8*>(sOb + (16 * half + n) * LDK + off);
+            v8 a, b;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                const v2 pa = M::pack((float)kv[e] * ((float)qv[e] * scale_log2),
+                                      (float)kv[e + 1] * ((float)qv[e + 1] * scale_log2));
+                const v2 pb = M::pack((float)vv[e] * (float)dv[e], (float)vv[e + 1] * (float)dv[e + 1]);
+                a[e] = pa[0]; a[e + 1] = pa[1];
+                b[e] = pb[0]; b[e + 1] = pb[1];
+            }
+            bq[ks] = a;
+            bg[ks] = b;
+        }
+        f32x4 accQ[DT], accT[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            accQ[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            accT[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+
+        for (int st = 0; st < nsteps; ++st, ++gstage) {
+            const E* sb = sStage + (gstage % NBUF) * STAGE;
+            const E* sb_next = sStage + ((gstage + 1) % NBUF) * STAGE;
+            const int jb = st * 32;
+            const bool need_mask = (k > jfull) || (jb + 31 > jfull);
+
+            // ---- score products, k-steps 0 and 1 (X: rows batch 0, read during the previous step); Y <- rows batch 1
+            read_rows(sb, 1, Y);
+            __builtin_amdgcn_sched_barrier(0);
+            // S starts from -LSE2[q], or from -3e4 where (q, j, k) is invalid; register i of tile t is key
+            // jb + 8 grp + 4 t + i.  dP starts from -Delta[q].
+            f32x4 s[2], dp[2];
+            if (need_mask) {
+                const int lim = (k <= jq) ? jq - jb - 8 * grp : -1;
+                f32x4 c0, c1;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    c0[i] = i <= lim ? -lse2 : -3.0e4f;
+                    c1[i] = 4 + i <= lim ? -lse2 : -3.0e4f;
+                }
+                s[0] = M16::mma(X.a[0], bq[0], c0);
+                s[1] = M16::mma(X.a[2], bq[0], c1);
+            } else {
+                s[0] = M16::mma(X.a[0], bq[0], c_lse);
+                s[1] = M16::mma(X.a[2], bq[0], c_lse);
+            }
+            dp[0] = M16::mma(X.u[0], bg[0], c_delta);
+            dp[1] = M16::mma(X.u[2], bg[0], c_delta);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                s[t] = M16::mma(X.a[2 * t + 1], bq[1], s[t]);
+                dp[t] = M16::mma(X.u[2 * t + 1], bg[1], dp[t]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- k-steps 2 and 3 (Y); X <- column batch 0
+            read_cols(sb, 0, X);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    s[t] = M16::mma(Y.a[2 * t + kk], bq[2 + kk], s[t]);
+                    dp[t] = M16::mma(Y.u[2 * t + kk], bg[2 + kk], dp[t]);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- the next stage has landed (this wave's part: fetched a step ago), and after the barrier every
+            // wave's; every wave is also done with the buffer the fetch below overwrites (the previous step's).
+            // LDS reads stay in flight across the barrier.
+            asm volatile("" ::: "memory");
+            wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (st == 0 && m + 1 < m_hi) issue_round(m + 1, mb ^ 1);
+            issue_stage(st_ahead, (gstage + 2) % NBUF);
+            advance();
+            // ---- Y <- column batch 1; P = exp2(S), dS = P dP, packed: k-slots 0..3 of a lane come from tile 0,
+            // 4..7 from tile 1
+            read_cols(sb, 1, Y);
+            __builtin_amdgcn_sched_barrier(0);
+            v8 pa, da;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; i += 2) {
+                    const float p0 = fast_exp2(s[t][i]), p1 = fast_exp2(s[t][i + 1]);
+                    const v2 pp = M::pack(p0, p1);
+                    const v2 dd = M::pack(p0 * dp[t][i], p1 * dp[t][i + 1]);
+                    pa[4 * t + i] = pp[0]; pa[4 * t + i + 1] = pp[1];
+                    da[4 * t + i] = dd[0]; da[4 * t + i + 1] = dd[1];
+                }
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- gradient products of column tiles 0..3 (X); X <- rows batch 0 of the next stage
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                accT[x] = M16::mma(pa, X.a[x], accT[x]);
+                accQ[x] = M16::mma(da, X.u[x], accQ[x]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            read_rows(sb_next, 0, X);
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- column tiles 4..7 (Y)
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                accT[4 + x] = M16::mma(pa, Y.a[x], accT[4 + x]);
+                accQ[4 + x] = M16::mma(da, Y.u[x], accQ[4 + x]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // ---- round epilogue: register i of column tile dt = query 16 half + 4 grp + i, column 16 dt + n
+        if (k <= jend) {
+            float outk[2] = {0.f, 0.f}, outv[2] = {0.f, 0.f};
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = dt * 16 + n;
+                float sk = 0.f, sv = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int ql = 16 * half + 4 * grp + i;
+                    sk += accQ[dt][i] * (float)sQb[ql * LDK + d];
+                    sv += accT[dt][i] * (float)sOb[ql * LDK + d];
+                }
+                sk += __shfl_xor(sk, 16, 64);
+                sv += __shfl_xor(sv, 16, 64);
+                sk += __shfl_xor(sk, 32, 64);
+                sv += __shfl_xor(sv, 32, 64);
+                // lane group g keeps column tiles g and g + 4: four full-wave atomics instead of sixteen quarter ones
+                if (grp == (dt & 3)) {
+                    outk[dt >> 2] = sk;
+                    outv[dt >> 2] = sv;
+                }
+            }
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const int d = (grp + 4 * x) * 16 + n;
+                accumulate(p, p.acc_k, base + (size_t)k * D + d, outk[x] * p.alpha);
+                accumulate(p, p.acc_v, base + (size_t)k * D + d, outv[x]);
+            }
+            if constexpr (WITH_DQ) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const float kd = (float)sKr[(mb * RPR + rrow) * D + dt * 16 + n];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) accDQ[dt][i] += accQ[dt][i] * kd;
+                }
+            }
+        }
+        // the next round's rows (fetched at this round's first step) have landed for every wave: they are older than
+        // the one stage fetch that stays in flight
+        barrier_keep_loads<LW>();
+    }
+    wait_vmcnt<0>();  // the stages fetched ahead land in LDS before the buffers are reused
+    __syncthreads();
+
+    if constexpr (WITH_DQ) {
+        // dQ: the four waves of a query half meet in LDS (the stage buffers are free now)
+        float* red = reinterpret_cast<float*>(smem);  // [wave][dt][i][lane]
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[((wave * DT + dt) * 4 + i) * 64 + lane] = accDQ[dt][i];
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < BQ * D / NTH; ++e) {
+            const int idx = e * NTH + tid;
+            const int ln = idx & 63, i = (idx >> 6) & 3, dt = (idx >> 8) & 7, hf = idx >> 11;
+            float v = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v += red[(((2 * r + hf) * DT + dt) * 4 + i) * 64 + ln];
+            const int qq = q0 + 16 * hf + 4 * (ln >> 4) + i, d = dt * 16 + (ln & 15);
+            if (qq < T) {
+                const size_t off = base + (size_t)qq * D + d;
+                if (p.splits > 1) accumulate(p, p.acc_q, off, v);  // scaled by alpha when converted
+                else p.dq[off] = (E)(v * p.alpha);
+            }
+        }
+    }
+}
+
+}  // namespace tritt

@@ -67,9 +67,10 @@ const char* tritt_status_string(int status);
  *   TRITT_TUNE_FWD_BAND     (env TRITT_FWD_BAND=0)     -1: narrow windowed masks take the streaming forward
  *                                                      instead of the band-resident one
  *   TRITT_TUNE_BWD_SPLITS   (env TRITT_BWD_SPLITS)     workgroups per query tile in the triple-dot backward, 1..16
- *   TRITT_TUNE_BWD128_WAVES (env TRITT_BWD128_VARIANT=w8|w4)  workgroup shape of the D = 128 backward: 8 or 4
+ *   TRITT_TUNE_BWD128_WAVES (env TRITT_BWD128_VARIANT=w8|w4)  the D = 128 backward under full windows: 0 = 16 queries per
+ *                           wave on 16x16x32 tiles (the default); 8 | 4 = the 32-query kernels with 8 or 4 waves
  *   TRITT_TUNE_F32_VALU     1: the fp32 path runs the VALU kernels at every head dimension (instead of the
- *                           fp32 MFMA kernels at D = 32 and 64) */
+ *                           fp32 MFMA kernels at D = 32, 64 and 128) */
 enum { TRITT_TUNE_FWD_SPLITS = 0, TRITT_TUNE_FWD_BAND = 1, TRITT_TUNE_BWD_SPLITS = 2, TRITT_TUNE_BWD128_WAVES = 3,
        TRITT_TUNE_F32_VALU = 4, TRITT_TUNE_COUNT_ = 5 };
 int tritt_set_tuning(int knob, int value);

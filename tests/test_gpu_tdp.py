@@ -476,12 +476,13 @@ def test_mfma_backward_bf16(seq_len, causal):
 
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("seq_len", [1, 33, 100, 256, 300])
-@pytest.mark.parametrize("shape", ["w4", "w8"])
+@pytest.mark.parametrize("shape", ["w4", "w8", "q16"])
 def test_mfma_backward_d128_bf16(seq_len, causal, shape, tune):
-    """Head dimension 128, both workgroup shapes of the backward kernel (one wave per SIMD with all
-    128 gradient columns / two waves per SIMD with one half of them)."""
+    """Head dimension 128, the three shapes of the backward kernel: 32 queries per wave with one wave per SIMD and
+    all 128 gradient columns / two waves per SIMD and one half of them, and 16 queries per wave on 16x16x32
+    tiles (the default)."""
     print(f"case mfma bwd D=128 T={seq_len} causal={causal} shape={shape}", flush=True)
-    tune(_lib.TUNE_BWD128_WAVES, int(shape[1]))
+    tune(_lib.TUNE_BWD128_WAVES, int(shape[1:]))
     inputs = orc.make_inputs(1, 3, seq_len, 128, torch.bfloat16, seed=seq_len + 7)
     alpha = 1 / math.sqrt(128)
     z, _, grads = util.oracle_tdp(inputs, alpha, causal)
