@@ -18,7 +18,6 @@ __device__ __forceinline__ constexpr int swz_perm(int r) {
     return ((r >> 1) & 1) | (((r >> 3) & 1) << 1) | (((r ^ (r >> 2)) & 1) << 2);
 }
 __device__ __forceinline__ constexpr int swz_seq(int r) { return (r & 7) ^ ((r >> 3) & 1); }
-
 // one 1 KB block: `gbase` is wave-uniform, `byte_off` per lane, `lds_dst` wave-uniform.
 // Written as inline assembly on purpose.  The compiler treats the builtin form of this load as an access that may
 // touch both global memory and LDS, and while one is outstanding its wait-count insertion turns every wait for an

@@ -20,9 +20,10 @@
 // query) and enter as resident 4-register C operands; an invalid (q, j, k) gets -3e4 there instead.
 //
 // Workgroup = 32 queries x 4 rows per round: wave w takes query half w & 1 and row w >> 1.  Stages are 32
-// keys of K1, U (row-major, 128-byte tile rows, 16-byte chunks swizzled for the permuted 16-row reads) and
-// K1^T, U^T ([128 d][32 keys], 64-byte rows); three buffers, fetched direct-to-LDS two steps ahead, one
-// workgroup barrier per step.  dQ is summed over the rounds in registers and over the waves at the end.
+// keys of K1 and U, row-major (128-byte tile rows, 16-byte chunks swizzled for the permuted 16-row reads); the
+// gradient products read the same tiles transposed (ds_read_b64_tr_b16).  Three buffers, fetched direct-to-LDS
+// two steps ahead, one workgroup barrier per step.  dQ is summed over the rounds in registers and over the
+// waves at the end.
 #pragma once
 
 namespace tritt {
@@ -49,15 +50,15 @@ __device__ __forceinline__ constexpr int q16_key(int t, int r) { return 8 * (r >
 // Chunk swizzles of the stage tiles.  A 16-byte LDS read is served in four passes of 16 lanes, {0-3, 12-15, 20-27},
 // {32-35, 44-47, 52-59}, {4-11, 16-19, 28-31}, {36-43, 48-51, 60-63} (measured: lanes of different passes never
 // collide), and the 16 lanes of a pass must fall on 16 distinct 16-byte bank groups (address / 16 mod 16).
-// Row-major tiles (128-byte rows): chunk c of key row r sits at position c ^ swz_q16(r); transposed tiles (64-byte
-// rows): chunk c of column d at c ^ swz_t16(d).  Both were found by searching the xor swizzles under that rule
-// for the 16-row operand reads below and confirmed on the hardware (2.8 cycles per wave-wide read, the rate of a
-// linear read; the swizzles of the 32-row kernels cost 4.3-5 cycles under these reads).
+// Chunk c of key row r (128-byte rows) sits at position c ^ swz_q16(r): found by searching the xor swizzles under
+// that rule for the 16-row operand reads below and confirmed on the hardware (2.8 cycles per wave-wide read, the
+// rate of a linear read; the swizzle of the 32-row kernels costs 4.3-5 cycles under these reads).  The 8-byte
+// transposed reads of the gradient products run at the linear rate under the same swizzle too (1.5 cycles per
+// 512-byte read; 4.5 without a swizzle).
 __device__ __forceinline__ constexpr int swz_q16(int r) { return (r & 2) | ((r >> 1) & 4); }
-__device__ __forceinline__ constexpr int swz_t16(int d) { return (d >> 1) & 2; }
 
 constexpr size_t bwd_q16_smem() {
-    return 3 * (size_t)(4 * 32 * 128 * 2)    // stage buffers
+    return 3 * (size_t)(2 * 32 * 128 * 2)    // stage buffers
            + 2 * (size_t)(2 * 4 * 128 * 2)   // K2 / V2 rows of two rounds
            + 2 * (size_t)(32 * (128 + 8) * 2);  // Q and dO tiles
 }
@@ -70,12 +71,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     using v2 = typename M::v2;
     constexpr int D = 128, KS = D / 32, DT = D / 16, BQ = 32, NW = 8, RPR = 4, NTH = 64 * NW;
     constexpr int LDK = D + 8;
-    constexpr int NBUF = 3, LW = 4;  // stage buffers; direct loads per wave per stage (32 blocks of 1 KB)
-    constexpr int TILE = 32 * D;     // elements of one tensor's part of a stage
-    constexpr int STAGE = 4 * TILE;
+    constexpr int NBUF = 3, LW = 2;  // stage buffers; direct loads per wave per stage (16 blocks of 1 KB)
+    constexpr int SK = 32;           // keys per stage: one step
+    constexpr int TILE = SK * D;     // elements of one tensor's part of a stage
+    constexpr int STAGE = 2 * TILE;
 
     extern __shared__ __align__(16) char smem[];
-    E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows | U rows | K1^T | U^T]
+    E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows | U rows]
     E* sKr = sStage + NBUF * STAGE;          // [2][RPR][D]
     E* sVr = sKr + 2 * RPR * D;
     E* sQb = sVr + 2 * RPR * D;              // [BQ][LDK]
@@ -111,36 +113,24 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     const int jq = p.causal ? min(q, T - 1) : T - 1;
     const float scale_log2 = p.alpha * kLog2e;
 
-    // ---- stage loader: wave w fetches blocks 4 w .. 4 w + 3 of
-    //   8 blocks of K1 rows, 8 of U rows (tile rows 8 b .. 8 b + 7), 8 of K1^T, 8 of U^T (16 d-rows each);
-    //   row-major tensors: blocks 0..3 are keys 0..31 of columns 0..63, blocks 4..7 the same keys of columns 64..127
-    const bool row_major = wave < 4;
-    const E* gsrc = uniform_ptr(wave < 2 ? p.st_k + base : wave < 4 ? p.st_v + base : wave < 6 ? p.st_kt + tbase : p.st_vt + tbase);
+    // ---- stage loader: wave w fetches blocks 2 w, 2 w + 1 of 8 blocks of K1 rows and 8 of U rows (tile rows
+    //   8 b .. 8 b + 7; blocks 0..3 are keys 0..31 of columns 0..63, blocks 4..7 the same keys of columns 64..127)
+    const E* gsrc = uniform_ptr((wave < 4 ? p.st_k : p.st_v) + base);
     unsigned grest[LW];  // per-lane byte offset apart from the key term
-    int gkey[LW];        // row-major blocks: key offset of this lane's row inside the stage
+    int gkey[LW];        // key offset of this lane's row inside the stage
 #pragma unroll
     for (int c = 0; c < LW; ++c) {
-        const int b = (wave & 1) * LW + c;  // block inside its tensor
-        if (row_major) {
-            const int R = b * 8 + (lane >> 3), hh = R >> 5, r = R & 31;
-            gkey[c] = r;
-            grest[c] = (unsigned)(hh * 64 + (((lane & 7) ^ swz_q16(r)) * 8)) * 2;
-        } else {
-            const int dl = b * 16 + (lane >> 2);
-            gkey[c] = 0;
-            grest[c] = ((unsigned)dl * p.Tp + (((lane & 3) ^ swz_t16(dl)) * 8)) * 2;
-        }
+        const int b = (wave & 3) * LW + c;  // block inside its tensor
+        const int R = b * 8 + (lane >> 3), hh = R / SK, r = R % SK;
+        gkey[c] = r;
+        grest[c] = (unsigned)(hh * 64 + (((lane & 7) ^ swz_q16(r)) * 8)) * 2;
     }
-    auto issue_stage = [&](int st, int buf) {
-        const int jb = st * 32;
+    auto issue_stage = [&](int sg, int buf) {
+        const int jb = sg * SK;
         char* dst = reinterpret_cast<char*>(sStage + buf * STAGE) + wave * LW * 1024;
 #pragma unroll
-        for (int c = 0; c < LW; ++c) {
-            // row-major rows past the end of the sequence are clamped (their keys are masked); the transposed
-            // tensors are zero padded
-            const unsigned off = grest[c] + (row_major ? (unsigned)min(jb + gkey[c], T - 1) * (D * 2) : (unsigned)jb * 2);
-            direct_load_16(gsrc, off, dst + c * 1024);
-        }
+        for (int c = 0; c < LW; ++c)  // rows past the end of the sequence are clamped (their keys are masked)
+            direct_load_16(gsrc, grest[c] + (unsigned)min(jb + gkey[c], T - 1) * (D * 2), dst + c * 1024);
     };
     // the round's K2 / V2 rows RPR m .. RPR m + 3: one 1 KB load per tensor
     auto issue_round = [&](int m, int buf) {
@@ -159,14 +149,14 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
         sQb[r * LDK + d] = p.q[off];
         sOb[r * LDK + d] = p.d_o[off];
     }
-    int st_ahead = 0;
+    int st_ahead = 0;  // stage fetched next: the sequence the rounds walk, 0 .. nsteps - 1 over and over
     auto advance = [&]() { st_ahead = st_ahead + 1 < nsteps ? st_ahead + 1 : 0; };
     issue_round(m_lo, m_lo & 1);
     issue_stage(st_ahead, 0);
     advance();
     issue_stage(st_ahead, 1);
     advance();
-    int gstage = 0;
+    int gstage = 0;  // stages consumed so far (buffer = gstage % NBUF)
 
     const float lse2 = q_ok ? p.lse[(size_t)bh * T + q] * kLog2e : 3.0e4f;
     const float delta = q_ok ? p.delta[(size_t)bh * T + q] : 0.f;
@@ -197,7 +187,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
             const int ks = 2 * b + kk;
-            const int coff = (ks >> 1) * 32 * 64 + ((((ks & 1) * 4 + grp) ^ rswz) * 8);
+            const int coff = (ks >> 1) * SK * 64 + ((((ks & 1) * 4 + grp) ^ rswz) * 8);
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 o.a[2 * t + kk] = *reinterpret_cast<const v8*>(sb + roff[t] + coff);
@@ -205,13 +195,32 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
             }
         }
     };
+    // The gradient products contract over the keys, so their streamed operand wants eight keys of one column per
+    // lane: a transposed read of the row-major tile.  ds_read_b64_tr_b16 does that in the LDS unit: in every group
+    // of 16 lanes, lane i supplies the address of four consecutive 16-bit elements and lane l receives element
+    // l % 4 of lanes l / 4, 4 + l / 4, 8 + l / 4, 12 + l / 4.  With lane i of group g pointing at columns
+    // 16 dt + 4 (i % 4) .. + 3 of key 8 g + i / 4, lane l gets column 16 dt + l of keys 8 g .. 8 g + 3; a second read
+    // four rows further down completes the eight k-slots.  (No transposed copies of K1 and U in the stages: half
+    // the bytes fetched per step.)
+    typedef __attribute__((ext_vector_type(4))) short s4;
+    typedef __attribute__((ext_vector_type(8))) short s8;
+    auto tr_read8 = [&](const E* ptr) {
+        const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4*)ptr);
+        const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4*)(ptr + 4 * 64));
+        return __builtin_bit_cast(v8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    int cbase[4];  // element offset of this lane's piece for column tiles dt = 0..3 (dt + 4: the other 64-column half)
+    {
+        const int i = lane & 15, key = 8 * grp + (i >> 2);
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            cbase[v] = key * 64 + ((((2 * v) ^ swz_q16(key)) + ((i & 3) >> 1)) * 8) + (i & 1) * 4;
+    }
     auto read_cols = [&](const E* sb, int b, OperandSet& o) {
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
-            const int d = (4 * b + x) * 16 + n;
-            const int toff = d * 32 + ((grp ^ swz_t16(d)) * 8);
-            o.a[x] = *reinterpret_cast<const v8*>(sb + 3 * TILE + toff);
-            o.u[x] = *reinterpret_cast<const v8*>(sb + 2 * TILE + toff);
+            o.a[x] = tr_read8(sb + TILE + b * (SK * 64) + cbase[x]);
+            o.u[x] = tr_read8(sb + b * (SK * 64) + cbase[x]);
         }
     };
     // stage 0 and the first round's rows have landed for every wave
