@@ -51,6 +51,13 @@ __device__ __forceinline__ bool block_to_tile(int BH, int& bh, int& tile) {
     return bh < BH;
 }
 
+// Under a full causal mask the owner tiles of a launch are a triangle: the longest walks nt streamed tiles, the
+// shortest one, and with one tile per workgroup the launch lasts as long as its longest tile while most SIMDs
+// idle.  Paired, a workgroup takes tile `tile` and then tile nt - 1 - tile of the launch order: nt + 1 streamed
+// tiles for every workgroup.  Returns how many owner tiles this workgroup walks; `part` selects one.
+__device__ __forceinline__ int owner_tiles(int pair, int nt, int tile) { return (pair && tile != nt - 1 - tile) ? 2 : 1; }
+__device__ __forceinline__ int owner_tile(int nt, int tile, int part) { return part ? nt - 1 - tile : tile; }
+
 // element offsets of (row, d) in the two packings
 template <int D>
 __device__ __forceinline__ size_t p1_index(int row, int d) {
@@ -122,6 +129,7 @@ struct AttnFwdP {
     int T, Tp;
     float scale_log2;
     int causal, k_diff;
+    int pair;           // a workgroup takes two owner tiles, a long and a short one (see owner_tiles)
 };
 
 // kW: waves per workgroup (they split the streamed tiles of one owner tile)
@@ -135,8 +143,12 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     float* sM = sO + kW * D * kLdr;                  // [kW][32]
     float* sL = sM + kW * 32;                        // [kW][32]
 
-    int bh, tile;
-    if (!block_to_tile(p.BH, bh, tile)) return;
+    int bh, tile0;
+    if (!block_to_tile(p.BH, bh, tile0)) return;
+    const int nparts = owner_tiles(p.pair, p.Tp / 32, tile0);
+    for (int op = 0; op < nparts; ++op) {
+    if (op) __syncthreads();  // the merge tiles of the first owner tile have been read
+    const int tile = owner_tile(p.Tp / 32, tile0, op);
     const int r0 = (p.Tp / 32 - 1 - tile) * 32;  // longest rows first
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -316,6 +328,7 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
                 for (int j = 0; j < 8; ++j) p.outm_p2[tb + p2_index<D>(row, d0 + j)] = wv[j];
         }
     }
+    }  // owner tiles of this workgroup
 }
 
 // ------------------------------------------------------------------------------ backward, rows
@@ -332,6 +345,7 @@ struct AttnBwdP {
     int BH, T, Tp;
     float alpha;
     int causal, k_diff;
+    int pair;                // a workgroup takes two owner tiles, a long and a short one (see owner_tiles)
     // row kernel output: dx = alpha * sum + addend
     const float* addend;     // fp32 [BH][T][D] or null
     E* dx;
@@ -356,8 +370,12 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
     extern __shared__ __align__(16) char smem_raw[];
     float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
 
-    int bh, tile;
-    if (!block_to_tile(p.BH, bh, tile)) return;
+    int bh, tile0;
+    if (!block_to_tile(p.BH, bh, tile0)) return;
+    const int nparts = owner_tiles(p.pair, p.Tp / 32, tile0);
+    for (int op = 0; op < nparts; ++op) {
+    if (op) __syncthreads();  // the merge tiles of the first owner tile have been read
+    const int tile = owner_tile(p.Tp / 32, tile0, op);
     const int r0 = (p.Tp / 32 - 1 - tile) * 32;
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -465,9 +483,9 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
     spill_tiles<D>(sO, wave, acc, n, g);
     __syncthreads();
     const int rr = tid & 31, dg = tid >> 5, row = r0 + rr;
-    if (row >= T) return;
 #pragma unroll
     for (int c = dg; c < D / 8; c += 2 * kW) {  // 16-byte pieces dg, dg + 2 kW, ... of the row
+        if (row >= T) break;
         const int d0 = 8 * c;
         const size_t off = base + (size_t)row * D + d0;
         v8 ov;
@@ -482,6 +500,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
         }
         *reinterpret_cast<v8*>(p.dx + off) = ov;
     }
+    }  // owner tiles of this workgroup
 }
 
 // --------------------------------------------------------------------------- backward, columns
@@ -495,8 +514,12 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     float* sB = sO + kW * D * kLdr;                  // [kW][32]  dbias partials
     float* sR = sB + kW * 32;                        // [2 kW][32]   delta1 partials
 
-    int bh, tile;
-    if (!block_to_tile(p.BH, bh, tile)) return;
+    int bh, tile0;
+    if (!block_to_tile(p.BH, bh, tile0)) return;
+    const int nparts = owner_tiles(p.pair, p.Tp / 32, tile0);
+    for (int op = 0; op < nparts; ++op) {
+    if (op) __syncthreads();  // the merge tiles of the first owner tile have been read
+    const int tile = owner_tile(p.Tp / 32, tile0, op);
     const int c0 = tile * 32;  // lowest key rows are the longest
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -712,6 +735,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
             p.delta1[vb + c0 + tid] = (c0 + tid < T) ? d1 : 0.f;
         }
     }
+    }  // owner tiles of this workgroup
 }
 
 // --------------------------------------------------------------------------------------- prep
@@ -855,7 +879,18 @@ constexpr size_t row_smem() { return 4 * (size_t)(kW * D * kLdr); }
 
 template <typename F>
 hipError_t allow_smem(F kern, size_t bytes) {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    return ensure_dynamic_smem(reinterpret_cast<const void*>(kern), bytes);
+}
+// Owner tiles are paired (owner_tiles) when the pass is a full causal triangle of at least 32 tiles and the halved
+// grid still gives every CU two workgroups; measured together with the wave count (dps_waves below).
+bool pair_tiles(const MfmaDpsArgs& a, int k_diff, int workgroups, bool backward) {
+    const int knob = knobs().dps_pair;
+    if (knob) return knob > 0;
+    return a.causal && k_diff >= a.T - 1 && workgroups >= 1024 && a.T >= (backward ? 2048 : 1024);
+}
+dim3 attn_grid(const MfmaDpsArgs& a, int Tp, bool pair) {
+    const int nt = Tp / 32;
+    return dim3(8 * ((a.BH + 7) / 8) * (pair ? (nt + 1) / 2 : nt));
 }
 
 template <typename E, int D, int kW>
@@ -864,6 +899,7 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     const Layout l = layout(a.BH, a.T, D, for_bwd);
     char* ws = static_cast<char*>(a.workspace);
     const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
+    const bool pair_in = pair_tiles(a, a.k_diff, grid.x, for_bwd), pair_out = pair_tiles(a, a.T, grid.x, for_bwd);
     auto kern = attn_fwd_mfma_kernel<E, D, kW>;
     hipError_t e = allow_smem(kern, fwd_smem<D, kW>());
     if (e != hipSuccess) return e;
@@ -884,15 +920,15 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     p.outm_p1 = for_bwd ? (E*)(ws + l.wp1) : nullptr;
     p.outm_p2 = (E*)(ws + l.wp2);
     p.lse = (float*)(ws + l.lse1); p.lse_stride = Tp; p.lse_scale = 1.0f;
-    p.BH = a.BH; p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff;
-    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), (fwd_smem<D, kW>()), st, p);
+    p.BH = a.BH; p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff; p.pair = pair_in;
+    hipLaunchKernelGGL(kern, attn_grid(a, Tp, pair_in), dim3(64 * kW), (fwd_smem<D, kW>()), st, p);
     if (for_bwd) return hipGetLastError();
     // outer: rows Q[q], keys K2 with bias lse1, values W; O and LSE (natural log)
     AttnFwdP<E> o{};
     o.x = (const E*)a.q; o.kp = (const E*)(ws + l.k2p1); o.vp2 = (const E*)(ws + l.wp2); o.bias = (const float*)(ws + l.lse1);
     o.out = (E*)a.o_out; o.lse = a.lse_out; o.lse_stride = a.T; o.lse_scale = kLn2;
-    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T;
-    hipLaunchKernelGGL(kern, grid, dim3(64 * kW), (fwd_smem<D, kW>()), st, o);
+    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T; o.pair = pair_out;
+    hipLaunchKernelGGL(kern, attn_grid(a, Tp, pair_out), dim3(64 * kW), (fwd_smem<D, kW>()), st, o);
     return hipGetLastError();
 }
 
@@ -902,6 +938,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     const Layout l = layout(a.BH, a.T, D, true);
     char* ws = static_cast<char*>(a.workspace);
     const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
+    const bool pair_in = pair_tiles(a, a.k_diff, grid.x, true), pair_out = pair_tiles(a, a.T, grid.x, true);
     auto krow = attn_bwd_row_mfma_kernel<E, D, kW>;
     auto kcol_link = attn_bwd_col_mfma_kernel<E, D, kW, true>;
     auto kcol = attn_bwd_col_mfma_kernel<E, D, kW, false>;
@@ -932,13 +969,13 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     o.xp = (const E*)(ws + l.qp1); o.gp = (const E*)(ws + l.dop1);
     o.xp2 = (const E*)(ws + l.qp2); o.gp2 = (const E*)(ws + l.dop2);
     o.bias = (const float*)(ws + l.lse1); o.lse2 = (const float*)(ws + l.lse2); o.delta = (const float*)(ws + l.delta);
-    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T;
+    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T; o.pair = pair_out;
     o.dx = (E*)a.dq;
     o.dk_f32 = (float*)(ws + l.dk2p);
     o.r_f32 = (const float*)(ws + l.r); o.v2 = (const E*)a.v2; o.dv2 = (E*)a.dv2;
     o.dr = (E*)(ws + l.dr); o.dr_p1 = (E*)(ws + l.drp1); o.dr_p2 = (E*)(ws + l.drp2); o.delta1 = (float*)(ws + l.delta1);
-    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), (row_smem<D, kW>()), st, o);
-    hipLaunchKernelGGL(kcol_link, grid, dim3(64 * kW), (col_smem<D, kW>()), st, o);
+    hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_out), dim3(64 * kW), (row_smem<D, kW>()), st, o);
+    hipLaunchKernelGGL(kcol_link, attn_grid(a, Tp, pair_out), dim3(64 * kW), (col_smem<D, kW>()), st, o);
 
     // inner pass: X = K2, G = dR, K = K1, V = U
     AttnBwdP<E> i{};
@@ -947,11 +984,11 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     i.xp = (const E*)(ws + l.k2p1); i.gp = (const E*)(ws + l.drp1);
     i.xp2 = (const E*)(ws + l.k2p2); i.gp2 = (const E*)(ws + l.drp2);
     i.lse2 = (const float*)(ws + l.lse1); i.delta = (const float*)(ws + l.delta1);
-    i.BH = a.BH; i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff;
+    i.BH = a.BH; i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff; i.pair = pair_in;
     i.addend = (const float*)(ws + l.dk2p); i.dx = (E*)a.dk2;
     i.dk = (E*)a.dk1; i.v1 = (const E*)a.v1; i.dv = (E*)a.dv1;
-    hipLaunchKernelGGL(krow, grid, dim3(64 * kW), (row_smem<D, kW>()), st, i);
-    hipLaunchKernelGGL(kcol, grid, dim3(64 * kW), (col_smem<D, kW>()), st, i);
+    hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_in), dim3(64 * kW), (row_smem<D, kW>()), st, i);
+    hipLaunchKernelGGL(kcol, attn_grid(a, Tp, pair_in), dim3(64 * kW), (col_smem<D, kW>()), st, i);
     return hipGetLastError();
 }
 
@@ -961,21 +998,30 @@ bool mfma_dps_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D
 size_t mfma_dps_fwd_workspace(int BH, int T, int D) { return layout(BH, T, D, false).total; }
 size_t mfma_dps_bwd_workspace(int BH, int T, int D) { return layout(BH, T, D, true).total; }
 
-// Waves per workgroup, measured: two at D = 128 and for long sequences at D = 64 (fewer partial results to
-// merge, longer-lived waves), four otherwise (short sequences and D = 32 want the parallelism).
-static bool two_waves(const MfmaDpsArgs& a) { return a.D == 128 || (a.D == 64 && a.T >= 1024); }
+// Waves per workgroup (they split the streamed tiles of an owner tile), measured at B*H = 32..64, bf16, forward /
+// backward in us, (waves, paired) = (2, no) | (4, no) | (4, yes):  T=512: 29 / 100 | 32 / 118 | 31 / 115;
+// T=1024: 42 / 137 | 39 / 145 | 38 / 142;  T=2048: 65 / 208 | 54 / 199 | 52 / 197;  T=4096: 112 / 351 | 84 / 309 | 81 / 308.
+// Two waves at D = 128 (fewer partial results to merge); at D = 64 four waves from T = 2048 on, and from T = 1024 in
+// the forward, or when the grid is too small to give every CU four workgroups of two waves.
+static bool two_waves(const MfmaDpsArgs& a, bool backward) {
+    if (a.D == 128) return true;
+    if (a.D == 64 && knobs().dps_waves) return knobs().dps_waves == 2;
+    const int workgroups = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32);
+    if (workgroups < 1024) return false;
+    return a.T < (backward ? 2048 : 1024);
+}
 
 template <typename E>
 static hipError_t dps_fwd_typed(const MfmaDpsArgs& a, hipStream_t st) {
     if (a.D == 32) return run_fwd<E, 32, 4>(a, st, false);
-    if (a.D == 64) return two_waves(a) ? run_fwd<E, 64, 2>(a, st, false) : run_fwd<E, 64, 4>(a, st, false);
+    if (a.D == 64) return two_waves(a, false) ? run_fwd<E, 64, 2>(a, st, false) : run_fwd<E, 64, 4>(a, st, false);
     if (a.D == 128) return run_fwd<E, 128, 2>(a, st, false);
     return hipErrorInvalidValue;
 }
 template <typename E>
 static hipError_t dps_bwd_typed(const MfmaDpsArgs& a, hipStream_t st) {
     if (a.D == 32) return run_bwd<E, 32, 4>(a, st);
-    if (a.D == 64) return two_waves(a) ? run_bwd<E, 64, 2>(a, st) : run_bwd<E, 64, 4>(a, st);
+    if (a.D == 64) return two_waves(a, true) ? run_bwd<E, 64, 2>(a, st) : run_bwd<E, 64, 4>(a, st);
     if (a.D == 128) return run_bwd<E, 128, 2>(a, st);
     return hipErrorInvalidValue;
 }

@@ -13,6 +13,8 @@ struct Knobs {
     int bwd_splits;      // TRITT_TUNE_BWD_SPLITS / env TRITT_BWD_SPLITS: workgroups per query tile, backward (1..16)
     int bwd128_variant;  // TRITT_TUNE_BWD128_WAVES / env TRITT_BWD128_VARIANT=w8|w4: the 32-query kernels (default: 16 queries per wave)
     int f32_valu;        // TRITT_TUNE_F32_VALU: 1 = fp32 tensors take the VALU kernels at every head dimension
+    int dps_waves;       // TRITT_TUNE_DPS_WAVES: waves per workgroup of the dot-product-sum MFMA kernels at D = 64 (2 | 4)
+    int dps_pair;        // TRITT_TUNE_DPS_PAIR: 1 / -1 = owner tiles always / never paired in those kernels
 };
 Knobs knobs();
 

@@ -67,7 +67,7 @@ def exported_symbols():
     return list(_PROTOS)
 
 
-TUNE_FWD_SPLITS, TUNE_FWD_BAND, TUNE_BWD_SPLITS, TUNE_BWD128_WAVES, TUNE_F32_VALU = 0, 1, 2, 3, 4
+TUNE_FWD_SPLITS, TUNE_FWD_BAND, TUNE_BWD_SPLITS, TUNE_BWD128_WAVES, TUNE_F32_VALU, TUNE_DPS_WAVES, TUNE_DPS_PAIR = range(7)
 
 
 class tuning:

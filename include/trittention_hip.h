@@ -70,9 +70,12 @@ const char* tritt_status_string(int status);
  *   TRITT_TUNE_BWD128_WAVES (env TRITT_BWD128_VARIANT=w8|w4)  the D = 128 backward under full windows: 0 = 16 queries per
  *                           wave on 16x16x32 tiles (the default); 8 | 4 = the 32-query kernels with 8 or 4 waves
  *   TRITT_TUNE_F32_VALU     1: the fp32 path runs the VALU kernels at every head dimension (instead of the
- *                           fp32 MFMA kernels at D = 32, 64 and 128) */
+ *                           fp32 MFMA kernels at D = 32, 64 and 128)
+ *   TRITT_TUNE_DPS_WAVES    waves per workgroup of the dot-product-sum MFMA kernels at D = 64: 2 | 4
+ *   TRITT_TUNE_DPS_PAIR     dot-product-sum MFMA kernels: 1 = a workgroup always takes two owner tiles (a long and a
+ *                           short one), -1 = never */
 enum { TRITT_TUNE_FWD_SPLITS = 0, TRITT_TUNE_FWD_BAND = 1, TRITT_TUNE_BWD_SPLITS = 2, TRITT_TUNE_BWD128_WAVES = 3,
-       TRITT_TUNE_F32_VALU = 4, TRITT_TUNE_COUNT_ = 5 };
+       TRITT_TUNE_F32_VALU = 4, TRITT_TUNE_DPS_WAVES = 5, TRITT_TUNE_DPS_PAIR = 6, TRITT_TUNE_COUNT_ = 7 };
 int tritt_set_tuning(int knob, int value);
 
 /* ---- triple-dot-product:  s[q,j,k] = alpha * sum_d Q[q,d] K1[j,d] K2[k,d] ----------------

@@ -160,6 +160,32 @@ def test_bitwise_reproducible():
         assert torch.equal(x, y)
 
 
+@pytest.mark.parametrize("T,D,k_diff,causal", [(203, 64, 203, True), (160, 64, 50, True), (96, 128, 1024, True),
+                                               (130, 32, 130, True), (64, 64, 64, False), (33, 64, 33, True)])
+@pytest.mark.parametrize("waves", [2, 4])
+def test_paired_owner_tiles_change_nothing(T, D, k_diff, causal, waves, tune):
+    """A workgroup of the MFMA kernels that takes two owner tiles (the long-and-short pairing of full causal
+    launches) computes each tile exactly as a workgroup of its own would: forced on and off, every result is
+    bitwise the same, odd and even tile counts, banded and unmasked passes included; and it matches the oracle."""
+    from flash_trittention import _lib
+
+    print(f"case dps pairing T={T} D={D} k_diff={k_diff} causal={causal} waves={waves}", flush=True)
+    inputs = orc.make_inputs(2, 3, T, D, torch.bfloat16, seed=T + D)
+    alpha = 1 / math.sqrt(D)
+    tune(_lib.TUNE_DPS_WAVES, waves)
+    tune(_lib.TUNE_DPS_PAIR, -1)
+    a = util.run_dps(inputs, alpha, causal, k_diff, flags=_lib.FLAG_FORCE_MFMA)
+    tune(_lib.TUNE_DPS_PAIR, 1)
+    b = util.run_dps(inputs, alpha, causal, k_diff, flags=_lib.FLAG_FORCE_MFMA)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    for name, x, y in zip(util.NAMES, a[2], b[2]):
+        assert torch.equal(x, y), name
+    z, lse, grads = util.oracle_dps(inputs, alpha, causal, k_diff)
+    util.assert_close("out", b[0], z, **LOWP)
+    for name, x, y in zip(util.NAMES, b[2], grads):
+        util.assert_close(name, x, y, **LOWP)
+
+
 def test_rejects_mismatched_shapes():
     from flash_trittention import TrittentionTriton
 
