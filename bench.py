@@ -31,9 +31,10 @@ NOMINAL_CLOCK_MHZ = 2400.0  # the clock behind the published peak
 # profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt).  Reported only when the workload is the default one.
 TRAFFIC_SOURCE = "profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt (rocprofv3 --pmc, default workload only)"
 TRAFFIC_FWD = 25.6e6        # 20.3 MiB fetched + 4.1 MiB written
-# average of the two launches: ~530 MiB written by 64-bit atomics each, 46 / 442 MiB fetched (the first launch's accumulators
-# fall out of their XCD's L2; the bytes are L2 <-> fabric traffic, which the 256 MB Infinity Cache absorbs)
-TRAFFIC_BWD_ROWS = 811e6
+# average of the two launches: ~530 MiB written by 64-bit atomics each, 36 / 78 MiB fetched (some runs: up to 440 MiB in the first
+# launch, when its accumulators fall out of their XCD's L2; the bytes are L2 <-> fabric traffic, which the 256 MB Infinity
+# Cache absorbs)
+TRAFFIC_BWD_ROWS = 614e6
 
 
 def triples(B, H, T, causal=True):
