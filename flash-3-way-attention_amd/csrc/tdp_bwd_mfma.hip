@@ -628,6 +628,13 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         smem = bwdg_smem(32, 8, 32, true);
         kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true>;
         kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true>;
+    } else if (a.windowed && D == 128 && knobs().bwd128_variant != 8) {
+        // the 16-query kernel (tdp_bwd_rows_q16.hpp), banded instantiation
+        if constexpr (D == 128) {
+            smem = bwd_q16_smem();
+            kern_dq = tdp_bwd_rows_q16_kernel<E, true, true>;
+            kern_nodq = tdp_bwd_rows_q16_kernel<E, false, true>;
+        }
     } else if (a.windowed) {
         smem = bwdg_smem(D, 8, 64, true);
         kern_dq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), true, 8, 64, true>;
@@ -641,8 +648,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         const int variant = knobs().bwd128_variant;
         if (variant != 4 && variant != 8) {
             smem = bwd_q16_smem();
-            kern_dq = tdp_bwd_rows_q16_kernel<E, true>;
-            kern_nodq = tdp_bwd_rows_q16_kernel<E, false>;
+            kern_dq = tdp_bwd_rows_q16_kernel<E, true, false>;
+            kern_nodq = tdp_bwd_rows_q16_kernel<E, false, false>;
         } else if (variant == 8) {
             smem = bwdg_smem(128, 8, 64, true);
             kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 8, 64, false>;

@@ -1,5 +1,6 @@
-// Triple-dot-product trittention backward on MFMA, head dimension 128, full causal windows or no mask
-// (included by tdp_bwd_mfma.hip after BwdParams): the rows kernel on 16x16x32 tiles.
+// Triple-dot-product trittention backward on MFMA, head dimension 128, every mask (included by tdp_bwd_mfma.hip
+// after BwdParams): the rows kernel on 16x16x32 tiles.  WIN: windowed causal masks; rounds and steps then cover the
+// band only, and a key outside the window of its (q, k) is masked like one past the causal bound.
 //
 // Same decomposition as tdp_bwd_rows_kernel (one K2/V2 row k per wave and round, K1 / U streamed over j in
 // stages shared by the workgroup), but a wave owns 16 queries instead of 32.  The accumulators Yq / Tv of
@@ -63,7 +64,7 @@ constexpr size_t bwd_q16_smem() {
            + 2 * (size_t)(32 * (128 + 8) * 2);  // Q and dO tiles
 }
 
-template <typename E, bool WITH_DQ>
+template <typename E, bool WITH_DQ, bool WIN>
 __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using M16 = Mma16<E>;
@@ -105,8 +106,15 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     const int jend = p.causal ? qlast : T - 1;
     const int jfull = p.causal ? q0 : T - 1;
     const int nsteps = jend / 32 + 1, nrounds = jend / RPR + 1;
-    const int per_split = (nrounds + p.splits - 1) / p.splits;
-    const int m_lo = split * per_split, m_hi = min(nrounds, m_lo + per_split);
+    // WIN, with a = streamed index (j), b = row index (k):  (q, a, b) takes part iff a, b <= q,
+    // q - a <= wa, q - b <= wb, b - a <= lab, a - b <= rab.  Rounds below m_first are outside the band
+    // of every query here; a round's sweep over a covers step_lo(m) .. step_hi(m) (never empty).
+    const bool banded = WIN && p.causal;
+    const int m_first = banded ? max(0, max(q0 - p.wb, q0 - p.wa - p.rab)) / RPR : 0;
+    auto step_lo = [&](int m) { return banded ? max(0, max(q0 - p.wa, m * RPR - p.lab)) / 32 : 0; };
+    auto step_hi = [&](int m) { return banded ? min(jend, m * RPR + RPR - 1 + p.rab) / 32 : nsteps - 1; };
+    const int per_split = (nrounds - m_first + p.splits - 1) / p.splits;
+    const int m_lo = m_first + split * per_split, m_hi = min(nrounds, m_lo + per_split);
     if (m_lo >= m_hi) return;  // fewer rounds than shares (uniform over the workgroup, before any barrier)
     const int q = q0 + 16 * half + n;
     const bool q_ok = q < T;
@@ -149,8 +157,17 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
         sQb[r * LDK + d] = p.q[off];
         sOb[r * LDK + d] = p.d_o[off];
     }
-    int st_ahead = 0;  // stage fetched next: the sequence the rounds walk, 0 .. nsteps - 1 over and over
-    auto advance = [&]() { st_ahead = st_ahead + 1 < nsteps ? st_ahead + 1 : 0; };
+    // (round, step) of the stage fetched next: the sequence the main loop walks, wrapping to the first round after
+    // the last (those fetches are never used)
+    int m_ahead = m_lo, st_ahead = step_lo(m_lo);
+    auto advance = [&]() {
+        if (st_ahead < step_hi(m_ahead)) {
+            ++st_ahead;
+        } else {
+            m_ahead = m_ahead + 1 < m_hi ? m_ahead + 1 : m_lo;
+            st_ahead = step_lo(m_ahead);
+        }
+    };
     issue_round(m_lo, m_lo & 1);
     issue_stage(st_ahead, 0);
     advance();
@@ -230,6 +247,15 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     for (int m = m_lo; m < m_hi; ++m) {
         const int mb = m & 1;
         const int k = m * RPR + rrow;
+        const int st_first = step_lo(m), st_last = step_hi(m);
+        // WIN: this lane's window of streamed keys for (q, k); empty if k itself is outside the band of q
+        [[maybe_unused]] int wlo = 0, whi = -1;
+        if constexpr (WIN) {
+            if (k <= jq && (!banded || q <= k + p.wb)) {
+                wlo = banded ? max(q - p.wa, k - p.lab) : 0;
+                whi = banded ? min(jq, k + p.rab) : jq;
+            }
+        }
 
         // B operands of the score products of this round: alpha log2e Q (.) K2[k] and dO (.) V2[k]
         v8 bq[KS], bg[KS];
@@ -259,11 +285,17 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
             accT[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
 
-        for (int st = 0; st < nsteps; ++st, ++gstage) {
+        for (int st = st_first; st <= st_last; ++st, ++gstage) {
             const E* sb = sStage + (gstage % NBUF) * STAGE;
             const E* sb_next = sStage + ((gstage + 1) % NBUF) * STAGE;
             const int jb = st * 32;
-            const bool need_mask = (k > jfull) || (jb + 31 > jfull);
+            bool need_mask = (k > jfull) || (jb + 31 > jfull);
+            if constexpr (WIN) {
+                // inside the band of every query of the tile (q0 .. q0 + 31), for this wave's row k
+                if (banded)
+                    need_mask = !((k <= q0) && (q0 + 31 <= k + p.wb) && (jb >= max(q0 + 31 - p.wa, k - p.lab)) &&
+                                  (jb + 31 <= min(q0, k + p.rab)));
+            }
 
             // ---- score products, k-steps 0 and 1 (X: rows batch 0, read during the previous step); Y <- rows batch 1
             read_rows(sb, 1, Y);
@@ -272,12 +304,21 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
             // jb + 8 grp + 4 t + i.  dP starts from -Delta[q].
             f32x4 s[2], dp[2];
             if (need_mask) {
-                const int lim = (k <= jq) ? jq - jb - 8 * grp : -1;
                 f32x4 c0, c1;
+                if constexpr (WIN) {
+                    const int lo = wlo - jb - 8 * grp, hi = whi - jb - 8 * grp;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    c0[i] = i <= lim ? -lse2 : -3.0e4f;
-                    c1[i] = 4 + i <= lim ? -lse2 : -3.0e4f;
+                    for (int i = 0; i < 4; ++i) {
+                        c0[i] = (i >= lo && i <= hi) ? -lse2 : -3.0e4f;
+                        c1[i] = (4 + i >= lo && 4 + i <= hi) ? -lse2 : -3.0e4f;
+                    }
+                } else {
+                    const int lim = (k <= jq) ? jq - jb - 8 * grp : -1;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        c0[i] = i <= lim ? -lse2 : -3.0e4f;
+                        c1[i] = 4 + i <= lim ? -lse2 : -3.0e4f;
+                    }
                 }
                 s[0] = M16::mma(X.a[0], bq[0], c0);
                 s[1] = M16::mma(X.a[2], bq[0], c1);
@@ -311,7 +352,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
             wait_vmcnt<0>();
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (st == 0 && m + 1 < m_hi) issue_round(m + 1, mb ^ 1);
+            if (st == st_first && m + 1 < m_hi) issue_round(m + 1, mb ^ 1);
             issue_stage(st_ahead, (gstage + 2) % NBUF);
             advance();
             // ---- Y <- column batch 1; P = exp2(S), dS = P dP, packed: k-slots 0..3 of a lane come from tile 0,
