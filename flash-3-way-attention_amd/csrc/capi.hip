@@ -81,7 +81,7 @@ size_t elem_size(int dtype) { return dtype == TRITT_F32 ? 4 : 2; }
 int check_common(int B, int H, int T, int D, int dtype) {
     if (B <= 0 || H <= 0 || T <= 0) return TRITT_ERR_INVALID;
     if (dtype != TRITT_F32 && dtype != TRITT_BF16 && dtype != TRITT_F16) return TRITT_ERR_INVALID;
-    if (D != 16 && D != 32 && D != 64 && D != 128) return TRITT_ERR_HEAD_DIM;
+    if (D != 8 && D != 16 && D != 32 && D != 64 && D != 128) return TRITT_ERR_HEAD_DIM;
     if ((long long)B * H > 65535) return TRITT_ERR_INVALID;
     if ((long long)B * H * T > 0x7fffffffLL) return TRITT_ERR_INVALID;  // row indices are 32-bit; element offsets are not
     return TRITT_OK;
@@ -424,7 +424,7 @@ const char* tritt_status_string(int status) {
     switch (status) {
         case TRITT_OK: return "ok";
         case TRITT_ERR_INVALID: return "invalid argument (null or misaligned pointer, non-positive size, negative window or unknown dtype)";
-        case TRITT_ERR_HEAD_DIM: return "head dimension must be 16, 32, 64 or 128";
+        case TRITT_ERR_HEAD_DIM: return "head dimension must be 8, 16, 32, 64 or 128";
         case TRITT_ERR_WORKSPACE: return "workspace missing or too small";
         case TRITT_ERR_UNSUPPORTED: return "requested implementation does not support this configuration";
         case TRITT_ERR_SCRATCH_LIMIT: return "problem needs more scratch than the library's static buffer holds";

@@ -307,6 +307,7 @@ static hipError_t bwd_impl(const DpsArgs& a, hipStream_t st) {
 
 hipError_t dps_fwd(const DpsArgs& a, hipStream_t st) {
     switch (a.D) {
+        case 8: return fwd_impl<8>(a, st);
         case 16: return fwd_impl<16>(a, st);
         case 32: return fwd_impl<32>(a, st);
         case 64: return fwd_impl<64>(a, st);
@@ -317,6 +318,7 @@ hipError_t dps_fwd(const DpsArgs& a, hipStream_t st) {
 
 hipError_t dps_bwd(const DpsArgs& a, hipStream_t st) {
     switch (a.D) {
+        case 8: return bwd_impl<8>(a, st);
         case 16: return bwd_impl<16>(a, st);
         case 32: return bwd_impl<32>(a, st);
         case 64: return bwd_impl<64>(a, st);

@@ -358,6 +358,7 @@ static hipError_t launch_bwd(const GenericTdpArgs& a, hipStream_t st) {
 
 hipError_t generic_tdp_fwd(const GenericTdpArgs& a, hipStream_t st) {
     switch (a.D) {
+        case 8: return launch_fwd<8>(a, st);
         case 16: return launch_fwd<16>(a, st);
         case 32: return launch_fwd<32>(a, st);
         case 64: return launch_fwd<64>(a, st);
@@ -368,6 +369,7 @@ hipError_t generic_tdp_fwd(const GenericTdpArgs& a, hipStream_t st) {
 
 hipError_t generic_tdp_bwd(const GenericTdpArgs& a, hipStream_t st) {
     switch (a.D) {
+        case 8: return launch_bwd<8>(a, st);
         case 16: return launch_bwd<16>(a, st);
         case 32: return launch_bwd<32>(a, st);
         case 64: return launch_bwd<64>(a, st);

@@ -37,8 +37,8 @@ class TrittentionTritonFunction(torch.autograd.Function):
         if q.dim() != 4:
             raise ValueError(f"expected [batch, heads, seq_len, head_dim] tensors, got shape {tuple(q.shape)}")
         B, H, T, D = q.shape
-        if D not in (16, 32, 64, 128):
-            raise ValueError(f"head_dim must be one of 16, 32, 64, 128, got {D}")
+        if D not in (8, 16, 32, 64, 128):
+            raise ValueError(f"head_dim must be one of 8, 16, 32, 64, 128, got {D}")
         _lib.dtype_code(q.dtype)
         q, k1, k2, v1, v2 = (t.contiguous() for t in (q, k1, k2, v1, v2))
         k_diff = clamp_window(k_diff, T, "k_diff")

@@ -29,8 +29,8 @@ def _validate(Q, others):
     head_dim = Q.shape[-1]
     if head_dim <= 0 or head_dim & (head_dim - 1):
         raise ValueError(f"head_dim must be a power of 2, got {head_dim}")
-    if head_dim not in (16, 32, 64, 128):
-        raise ValueError(f"head_dim must be one of 16, 32, 64, 128, got {head_dim}")
+    if head_dim not in (8, 16, 32, 64, 128):
+        raise ValueError(f"head_dim must be one of 8, 16, 32, 64, 128, got {head_dim}")
     _lib.dtype_code(Q.dtype)
 
 

@@ -36,7 +36,7 @@ enum {
     TRITT_OK = 0,
     TRITT_ERR_INVALID = -1,     /* null or misaligned pointer, negative size, bad dtype,
                                    B*H above 65535 or B*H*T above 2^31-1                    */
-    TRITT_ERR_HEAD_DIM = -2,    /* D not one of 16, 32, 64, 128                            */
+    TRITT_ERR_HEAD_DIM = -2,    /* D not one of 8, 16, 32, 64, 128                         */
     TRITT_ERR_WORKSPACE = -3,   /* workspace missing or smaller than *_workspace_bytes     */
     TRITT_ERR_UNSUPPORTED = -4, /* requested implementation cannot run this configuration */
     TRITT_ERR_SCRATCH_LIMIT = -5 /* tritt_tdp_fwd_static_scratch: the problem needs more scratch

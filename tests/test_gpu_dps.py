@@ -40,7 +40,7 @@ def test_narrow_k_diff_causal(k_diff):
     check_all(inputs, 1 / 8, True, k_diff)
 
 
-@pytest.mark.parametrize("D", [16, 64, 128])
+@pytest.mark.parametrize("D", [8, 16, 64, 128])
 def test_head_dims_fp32(D):
     inputs = orc.make_inputs(1, 2, 80, D, torch.float32, seed=D + 1)
     check_all(inputs, 1 / math.sqrt(D), True, 80)
@@ -149,6 +149,12 @@ def test_force_mfma_refused_for_fp32():
     inputs = orc.make_inputs(1, 1, 32, 64, torch.float32, seed=34)
     with pytest.raises(RuntimeError):
         util.run_dps(inputs, 1 / 8, True, 32, flags=_lib.FLAG_FORCE_MFMA)
+
+
+def test_head_dim_8_bf16():
+    """16-bit tensors with the smallest head dimension: computed by the fp32 kernels, held to the 16-bit bar."""
+    inputs = orc.make_inputs(2, 3, 70, 8, torch.bfloat16, seed=8)
+    check_all(inputs, 1 / math.sqrt(8), True, 40, tol=LOWP, rel=5e-2)
 
 
 def test_bitwise_reproducible():

@@ -55,11 +55,22 @@ def test_config1_forward_fp32():
     assert util.rel_err(out, z) <= 1e-4
 
 
-@pytest.mark.parametrize("D", [16, 64, 128])
+@pytest.mark.parametrize("D", [8, 16, 64, 128])
 def test_head_dims_fp32(D):
     print(f"case fp32 D={D}", flush=True)
     inputs = orc.make_inputs(1, 2, 48, D, torch.float32, seed=D)
     check_all(inputs, 1 / math.sqrt(D), True)
+
+
+def test_head_dim_8_bf16():
+    """16-bit tensors with the smallest head dimension: computed by the fp32 kernels, held to the 16-bit bar."""
+    inputs = orc.make_inputs(2, 3, 70, 8, torch.bfloat16, seed=8)
+    alpha = 1 / math.sqrt(8)
+    z, _, grads = util.oracle_tdp(inputs, alpha, True)
+    out, g = util.run_tdp(inputs, alpha, True)
+    util.assert_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_close(name, a, b, **LOWP)
 
 
 @pytest.mark.parametrize("D", [32, 64, 128])
