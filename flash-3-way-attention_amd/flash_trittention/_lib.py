@@ -70,6 +70,12 @@ def exported_symbols():
 TUNE_FWD_SPLITS, TUNE_FWD_BAND, TUNE_BWD_SPLITS, TUNE_BWD128_WAVES, TUNE_F32_VALU, TUNE_DPS_WAVES, TUNE_DPS_PAIR = range(7)
 
 
+def set_tuning(knob: int, value: int) -> int:
+    """tritt_set_tuning, returning the previous value; remembered workspace sizes may depend on the knobs."""
+    _workspace_sizes.clear()
+    return lib().tritt_set_tuning(knob, value)
+
+
 class tuning:
     """``with _lib.tuning(_lib.TUNE_BWD_SPLITS, 4): ...`` (tests and sweeps): sets a knob of the library and
     puts the previous value back on exit."""
@@ -78,11 +84,11 @@ class tuning:
         self.knob, self.value = knob, value
 
     def __enter__(self):
-        self.previous = lib().tritt_set_tuning(self.knob, self.value)
+        self.previous = set_tuning(self.knob, self.value)
         return self
 
     def __exit__(self, *exc):
-        lib().tritt_set_tuning(self.knob, self.previous)
+        set_tuning(self.knob, self.previous)
         return False
 
 
@@ -138,3 +144,37 @@ def stream_ptr(device):
 
 def workspace(nbytes: int, device):
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+class on_device:
+    """``with on_device(t.device):`` makes the tensor's GPU current around a library call (the backward may run on
+    an autograd thread whose current device is another one).  When it already is current, which is the usual case,
+    nothing is switched: torch's own guard costs several microseconds per call, as much as a small launch."""
+
+    __slots__ = ("guard",)
+
+    def __init__(self, device):
+        self.guard = None if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            return self.guard.__exit__(*exc)
+        return False
+
+
+_workspace_sizes = {}
+
+
+def workspace_bytes(query: str, *args) -> int:
+    """A `*_workspace_bytes` query of the library, remembered per argument tuple (the answer depends on nothing
+    else, except the tuning knobs: `tuning` and the tests' knob changes clear the memory)."""
+    key = (query, args)
+    size = _workspace_sizes.get(key)
+    if size is None:
+        size = _workspace_sizes[key] = getattr(lib(), query)(*args)
+    return size

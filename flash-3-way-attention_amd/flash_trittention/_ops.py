@@ -25,9 +25,9 @@ def tdp_fwd_impl(q, k1, k2, v1, v2, softmax_scale: float, causal: bool, k1_windo
     code = _lib.dtype_code(q.dtype)
     o = _empty_like_bhtd(q)
     lse = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
-        need = lib.tritt_tdp_fwd_workspace_bytes(B, H, T, D, code, int(causal), k1_window, k2_window, kk_left, kk_right,
-                                                 flags)
+    with _lib.on_device(q.device):
+        need = _lib.workspace_bytes("tritt_tdp_fwd_workspace_bytes", B, H, T, D, code, int(causal), k1_window, k2_window,
+                                    kk_left, kk_right, flags)
         ws = _lib.workspace(need, q.device)
         st = lib.tritt_tdp_fwd(_lib.ptr(q), _lib.ptr(k1), _lib.ptr(k2), _lib.ptr(v1), _lib.ptr(v2), _lib.ptr(o),
                                _lib.ptr(lse), B, H, T, D, code, float(softmax_scale), int(causal), k1_window, k2_window,
@@ -45,9 +45,9 @@ def tdp_bwd_impl(q, k1, k2, v1, v2, o, lse, d_o, softmax_scale: float, causal: b
     code = _lib.dtype_code(q.dtype)
     grads = [_empty_like_bhtd(q) if (wanted >> i) & 1 else None for i in range(5)]
     gptr = [_lib.ptr(t) if t is not None else None for t in grads]
-    with torch.cuda.device(q.device):
-        need = lib.tritt_tdp_bwd_workspace_bytes(B, H, T, D, code, int(causal), k1_window, k2_window, kk_left, kk_right,
-                                                 flags)
+    with _lib.on_device(q.device):
+        need = _lib.workspace_bytes("tritt_tdp_bwd_workspace_bytes", B, H, T, D, code, int(causal), k1_window, k2_window,
+                                    kk_left, kk_right, flags)
         ws = _lib.workspace(need, q.device)
         st = lib.tritt_tdp_bwd(_lib.ptr(q), _lib.ptr(k1), _lib.ptr(k2), _lib.ptr(v1), _lib.ptr(v2), _lib.ptr(o),
                                _lib.ptr(lse), _lib.ptr(d_o), *gptr, B, H, T, D, code, float(softmax_scale), int(causal),
@@ -65,8 +65,8 @@ def dps_fwd_impl(q, k1, k2, v1, v2, softmax_scale: float, causal: bool, k_diff: 
     code = _lib.dtype_code(q.dtype)
     o = _empty_like_bhtd(q)
     m = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
-        ws = _lib.workspace(lib.tritt_dps_fwd_workspace_bytes(B, H, T, D, code, flags), q.device)
+    with _lib.on_device(q.device):
+        ws = _lib.workspace(_lib.workspace_bytes("tritt_dps_fwd_workspace_bytes", B, H, T, D, code, flags), q.device)
         st = lib.tritt_dps_fwd(_lib.ptr(q), _lib.ptr(k1), _lib.ptr(k2), _lib.ptr(v1), _lib.ptr(v2), _lib.ptr(o),
                                _lib.ptr(m), B, H, T, D, code, float(softmax_scale), int(causal), k_diff, _lib.ptr(ws),
                                ws.numel(), flags, _lib.stream_ptr(q.device))
@@ -80,8 +80,8 @@ def dps_bwd_impl(q, k1, k2, v1, v2, o, m, d_o, softmax_scale: float, causal: boo
     lib = _lib.lib()
     code = _lib.dtype_code(q.dtype)
     grads = [_empty_like_bhtd(q) for _ in range(5)]
-    with torch.cuda.device(q.device):
-        ws = _lib.workspace(lib.tritt_dps_bwd_workspace_bytes(B, H, T, D, code, flags), q.device)
+    with _lib.on_device(q.device):
+        ws = _lib.workspace(_lib.workspace_bytes("tritt_dps_bwd_workspace_bytes", B, H, T, D, code, flags), q.device)
         st = lib.tritt_dps_bwd(_lib.ptr(q), _lib.ptr(k1), _lib.ptr(k2), _lib.ptr(v1), _lib.ptr(v2), _lib.ptr(o),
                                _lib.ptr(m), _lib.ptr(d_o), *(_lib.ptr(t) for t in grads), B, H, T, D, code,
                                float(softmax_scale), int(causal), k_diff, _lib.ptr(ws), ws.numel(), flags,

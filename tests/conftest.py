@@ -23,9 +23,9 @@ def tune():
     first = {}
 
     def set_knob(knob, value):
-        previous = _lib.lib().tritt_set_tuning(knob, value)
+        previous = _lib.set_tuning(knob, value)
         first.setdefault(knob, previous)
 
     yield set_knob
     for knob, previous in first.items():
-        _lib.lib().tritt_set_tuning(knob, previous)
+        _lib.set_tuning(knob, previous)
