@@ -804,6 +804,28 @@ def test_config3_headline_backward_subset():
             assert util.rel_err(a[b, h], ref) <= 2e-2, (name, util.rel_err(a[b, h], ref))
 
 
+def test_d128_backward_at_sweep_size_subset():
+    """B=1 H=16 T=1024 D=128 bf16 causal (a shape of the sequence-length sweep, with its backward): forward and all
+    five gradients of two heads, all rows, against the chunked dense fp32 oracle; the other heads through the
+    bitwise head-permutation property."""
+    print("case D=128 T=1024 backward", flush=True)
+    alpha = 1 / math.sqrt(128)
+    inputs = orc.make_inputs(1, 16, 1024, 128, torch.bfloat16, seed=9)
+    out, g = util.run_tdp(inputs, alpha, True)
+    for h in (2, 13):
+        z, lse, grads = orc.tdp_forward_backward_chunked(*(t[0, h].float() for t in inputs), alpha, True, q_chunk=64,
+                                                         need_grads=True)
+        util.assert_close(f"out[{h}]", out[0, h], z, **LOWP)
+        for name, a, ref in zip(util.NAMES, g, grads):
+            util.assert_close(f"{name}[{h}]", a[0, h], ref, **LOWP)
+            assert util.rel_err(a[0, h], ref) <= 2e-2, (name, util.rel_err(a[0, h], ref))
+    perm = torch.randperm(16, generator=torch.Generator().manual_seed(2))
+    out2, g2 = util.run_tdp([t[:, perm].contiguous() for t in inputs], alpha, True)
+    assert torch.equal(out2, out[:, perm])
+    for name, a, b in zip(util.NAMES, g2, g):
+        assert torch.equal(a, b[:, perm]), name
+
+
 # ------------------------------------------------- full-size properties (no oracle: every head is checked)
 def _headline_inputs(seed=5):
     return orc.make_inputs(4, 8, 1024, 64, torch.bfloat16, seed=seed)
