@@ -30,7 +30,7 @@ def test_check_perf_harness_passes_and_prints_the_reference_format():
     assert all(pat.match(l) for l in checks), checks
     assert len(perfs) == 4 and all(re.match(r"^PERF s=\d+ \S+ mi355x_ms=\d+\.\d+ ", l) for l in perfs)
     assert lines[-1] == "RESULT correctness=PASS"
-    # kept for the record of a GPU run (gpurun_out/ is scratch space on the GPU box)
+    # the harness output of this run is kept as a text file in the run's scratch output folder
     os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
     with open(os.path.join(ROOT, "gpurun_out", "harness_check_perf.txt"), "w") as f:
         f.write("\n".join(lines) + "\n")
