@@ -23,6 +23,7 @@ void init_knobs() {
         if (const char* e = getenv("TRITT_BWD_SPLITS")) g_knobs[TRITT_TUNE_BWD_SPLITS] = atoi(e);
         if (const char* e = getenv("TRITT_BWD128_VARIANT"))
             g_knobs[TRITT_TUNE_BWD128_WAVES] = strcmp(e, "w4") == 0 ? 4 : strcmp(e, "w8") == 0 ? 8 : 0;
+        if (const char* e = getenv("TRITT_F32_VALU")) g_knobs[TRITT_TUNE_F32_VALU] = atoi(e) != 0 ? 1 : 0;
     });
 }
 }  // namespace
@@ -414,10 +415,12 @@ extern "C" {
 
 int tritt_version(void) { return 200; }
 
-int tritt_set_tuning(int knob, int value) {
+int tritt_set_tuning(int knob, int value, int* previous) {
     if (knob < 0 || knob >= TRITT_TUNE_COUNT_) return TRITT_ERR_INVALID;
     init_knobs();
-    return g_knobs[knob].exchange(value);
+    const int old = g_knobs[knob].exchange(value);
+    if (previous) *previous = old;
+    return TRITT_OK;
 }
 
 const char* tritt_status_string(int status) {

@@ -96,6 +96,74 @@ __device__ __forceinline__ void transpose_store(E* __restrict__ dst, const E* ti
     }
 }
 
+// ---- 64-bit fixed-point gradient accumulators (backward kernels whose workgroups add shares of one gradient
+// element to a common sum; integer addition is associative, so the sums do not depend on the order of arrival).
+// The scale is a power of two chosen per (batch, head) slice from the largest finite |dO| of that slice,
+// 2^e <= max|dO| < 2^(e+1): a share v is added as round(v * 2^(bias - e)), so the accumulators resolve steps of
+// 2^-bias relative to the incoming gradient whatever its magnitude (loss scaling, mean-reduced losses) and cover
+// sums up to 2^(63 - bias) times it.  Scaling dO by a power of two scales every gradient by exactly that power.
+// The producer of the scale leaves kScaleParts partial maxima per slice (bit patterns of |dO|, non-finite values
+// skipped); every consumer joins them.  A share that is not finite, or too large for the accumulator, cannot be
+// represented in it: it sets a bit in the row's poison word instead, and the kernel that converts the
+// accumulators writes NaN for that row of that gradient (the fp32 sums these accumulators stand in for would
+// have been non-finite as well).
+constexpr int kScaleParts = 8;
+enum : unsigned { kPoisonDK1 = 1, kPoisonDU = 2, kPoisonDK2 = 4, kPoisonDV2 = 8, kPoisonDQ = 16 };
+
+__device__ __forceinline__ unsigned finite_abs_bits(float v) {
+    const unsigned b = __float_as_uint(v) & 0x7fffffffu;
+    return b < 0x7f800000u ? b : 0u;
+}
+// exponent field f of the scale 2^(f - 127) of slice bh.  UNIFORM: bh is the same in every lane of the wave (the
+// result is then kept in a scalar register); the kernels that convert the accumulators walk elements of several
+// slices in one wave and pass false.
+template <bool UNIFORM = true>
+__device__ __forceinline__ int fixed_scale_field(const unsigned* __restrict__ parts, int bh, int bias) {
+    const uint4 a = reinterpret_cast<const uint4*>(parts)[bh * 2], b = reinterpret_cast<const uint4*>(parts)[bh * 2 + 1];
+    unsigned m = max(max(max(a.x, a.y), max(a.z, a.w)), max(max(b.x, b.y), max(b.z, b.w)));
+    if (UNIFORM) m = __builtin_amdgcn_readfirstlane(m);
+    const int f = bias + 254 - (int)(m >> 23);  // bias - (exponent - 127) + 127
+    return min(max(f, 1), 254);
+}
+__device__ __forceinline__ float fixed_scale_value(int field) { return __uint_as_float((unsigned)field << 23); }
+__device__ __forceinline__ double fixed_scale_inverse(int field) {
+    return __longlong_as_double((long long)(1023 + 127 - field) << 52);
+}
+// One share of a common sum.  fscale == 0: the accumulator is fp32 (float atomics; non-finite values propagate by
+// themselves).  poison_row: the poison word of the element's row; bit: which gradient.
+__device__ __forceinline__ void shared_add(void* acc, size_t idx, float v, float fscale, unsigned* poison_row,
+                                           unsigned bit) {
+    if (fscale != 0.f) {
+        const float x = v * fscale;
+        if (!(fabsf(x) < 9.0e18f)) {  // NaN, Inf or beyond 2^63
+            atomicOr(poison_row, bit);
+            return;
+        }
+        atomicAdd(reinterpret_cast<unsigned long long*>(acc) + idx, (unsigned long long)__float2ll_rn(x));
+    } else {
+        unsafeAtomicAdd(reinterpret_cast<float*>(acc) + idx, v);
+    }
+}
+// block-wide maximum of the finite |x| bit patterns of `count` 16-byte pieces (E8 = 8 elements of E, or 4 floats)
+// starting at src; every thread of the 256-thread block returns the same value; `red` = 4 words of LDS
+template <typename E>
+__device__ __forceinline__ unsigned block_absmax_bits(const E* __restrict__ src, size_t count, unsigned* red) {
+    constexpr int PER = 16 / sizeof(E);
+    typedef __attribute__((ext_vector_type(PER))) E ev;
+    unsigned m = 0;
+    for (size_t i = threadIdx.x; i < count; i += 256) {
+        const ev x = *reinterpret_cast<const ev*>(src + i * PER);
+#pragma unroll
+        for (int e = 0; e < PER; ++e) m = max(m, finite_abs_bits((float)x[e]));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, off, 64));
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    return max(max(red[0], red[1]), max(red[2], red[3]));
+}
+
 // Window parameters of the triple-dot causal mask, expressed for a "staged"
 // index a and an "owner" index b (a = j, b = k in the natural orientation):
 //   valid  <=>  a<=q, b<=q, q<=a+wa, q<=b+wb, b<=a+lab, a<=b+rab

@@ -58,7 +58,11 @@ struct FirstTileArgs {
     void* dq;                                 // written when acc_q is null
     void *acc_k2, *acc_v2, *acc_k1, *acc_u;   // fixed point (long long) or float
     void* acc_q;                              // dQ / alpha accumulator of a split backward, or null
-    float fixed_scale;                        // 0: float accumulators
+    // fixed-point accumulators (common.hpp): the slices' scale partials, the rows' poison words and the bias of the
+    // scale; scale_parts null: float accumulators
+    const unsigned* scale_parts;
+    unsigned* poison;
+    int scale_bias;
     int BH, T, D, is_bf16;
     float alpha;
     int causal, k1_window, k2_window, kk_left, kk_right;

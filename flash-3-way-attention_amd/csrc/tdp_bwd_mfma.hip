@@ -38,10 +38,13 @@ struct BwdParams {
     // one, dQ / alpha is accumulated into acc_q (fp32, zero on entry) instead of being written to dq
     float* acc_q;
     int splits;
-    // accumulate the row gradients (and a split dQ) as 64-bit fixed point with integer atomics: integer addition is
-    // associative, so the sums are bitwise the same whatever order the workgroups arrive in.  The accumulators
-    // then hold long long where they otherwise hold float (twice the bytes, same element index).
+    // accumulate the row gradients (and a split dQ) as 64-bit fixed point with integer atomics (common.hpp: the
+    // sums are bitwise the same whatever order the workgroups arrive in).  The accumulators then hold long long
+    // where they otherwise hold float (twice the bytes, same element index); scale_parts / poison: see common.hpp
     int fixed_point;
+    const unsigned* scale_parts;  // [BH][kScaleParts]
+    unsigned* poison;             // [BH][T]
+    unsigned bit_k, bit_v;        // poison bits of acc_k / acc_v
     int T, Tp, BH, nqt;
     float alpha;
     int causal;
@@ -50,16 +53,13 @@ struct BwdParams {
     int wa, wb, lab, rab;
 };
 
-// 2^30: the accumulators cover |sum| < 8.6e9 in steps of 9.3e-10
-constexpr float kFixedScale = 1073741824.0f;
+// the 16-bit kernels' accumulators resolve 2^-30 of the slice's max |dO| and cover sums up to 2^33 times it
+constexpr int kFixedBias = 30;
 
-// One contribution to a gradient accumulator that several workgroups add to.
+// scale of the fixed-point accumulators of slice bh (0: the accumulators are fp32)
 template <typename E>
-__device__ __forceinline__ void accumulate(const BwdParams<E>& p, float* acc, size_t idx, float v) {
-    if (p.fixed_point)
-        atomicAdd(reinterpret_cast<unsigned long long*>(acc) + idx, (unsigned long long)__float2ll_rn(v * kFixedScale));
-    else
-        unsafeAtomicAdd(acc + idx, v);
+__device__ __forceinline__ float acc_scale(const BwdParams<E>& p, int bh) {
+    return p.fixed_point ? fixed_scale_value(fixed_scale_field(p.scale_parts, bh, kFixedBias)) : 0.f;
 }
 
 }  // namespace tritt
@@ -155,6 +155,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     const bool q_ok = q < T;
     const int jq = p.causal ? min(q, T - 1) : T - 1;  // per-lane bound on j and k
     const float scale_log2 = p.alpha * kLog2e;
+    const float fscale = acc_scale(p, bh);
 
     // stage loader: wave w fetches blocks 4*(w%2) .. +3 (8 rows each) of tensor w/2, direct to LDS
     const int tensor = wave >> 1;
@@ -424,8 +425,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
                 sk += __shfl_xor(sk, 32, 64);
                 sv += __shfl_xor(sv, 32, 64);
                 if (g == 0) {
-                    accumulate(p, p.acc_k, base + (size_t)k * D + d, sk * p.alpha);
-                    accumulate(p, p.acc_v, base + (size_t)k * D + d, sv);
+                    unsigned* prow = p.poison + (size_t)bh * T + k;
+                    shared_add(p.acc_k, base + (size_t)k * D + d, sk * p.alpha, fscale, prow, p.bit_k);
+                    shared_add(p.acc_v, base + (size_t)k * D + d, sv, fscale, prow, p.bit_v);
                 }
             }
         }
@@ -457,7 +459,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         for (int e = 0; e < 4; ++e)
             if (q0 + r0 + e < T) {
                 const size_t off = base + (size_t)(q0 + r0 + e) * D + d;
-                if (p.splits > 1) accumulate(p, p.acc_q, off, out[e]);  // scaled by alpha when converted
+                if (p.splits > 1)  // scaled by alpha when converted
+                    shared_add(p.acc_q, off, out[e], fscale, p.poison + (size_t)bh * T + q0 + r0 + e, kPoisonDQ);
                 else p.dq[off] = (E)(out[e] * p.alpha);
             }
     }
@@ -476,9 +479,23 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
                                                        float* __restrict__ delta, float* __restrict__ zero_a,
                                                        float* __restrict__ zero_b, float* __restrict__ zero_c,
                                                        float* __restrict__ zero_d, float* __restrict__ zero_e, int T,
-                                                       int Tp, int D, int zero_width) {
+                                                       int Tp, int D, int zero_width,
+                                                       unsigned* __restrict__ scale_parts,
+                                                       unsigned* __restrict__ poison) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * Tp;
+    if (scale_parts) {
+        // fixed-point accumulators: clear the poison words of this block's rows; the first blocks of a slice
+        // also leave the partial maxima of |dO| that fix the slice's scale (part s = 64-row blocks s, s + 8, ...)
+        __shared__ unsigned red[4];
+        if (threadIdx.x < 64 && j0 + threadIdx.x < T) poison[(size_t)bh * T + j0 + threadIdx.x] = 0;
+        for (int part = blockIdx.x; part < kScaleParts; part += gridDim.x) {
+            unsigned m = 0;
+            for (int r0 = part * 64; r0 < T; r0 += kScaleParts * 64)
+                m = max(m, block_absmax_bits<E>(d_o + base + (size_t)r0 * D, (size_t)min(64, T - r0) * D / 8, red));
+            if (threadIdx.x == 0) scale_parts[bh * kScaleParts + part] = m;
+        }
+    }
     // two tiles at a time (static LDS stays under 64 KB at D = 128): their loads are in flight together
     constexpr int kTile = 64 * (128 + 2);
     __shared__ E tiles[2 * kTile];
@@ -533,27 +550,36 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
                                                          E* __restrict__ dq, const E* __restrict__ v1,
                                                          E* __restrict__ dk1, E* __restrict__ dv1, E* __restrict__ dk2,
                                                          E* __restrict__ dv2, size_t n, int fixed_point,
-                                                         const float* __restrict__ dq0acc, int T, int D) {
-    auto value = [&](const float* acc, size_t i) {
-        if (!fixed_point) return acc[i];
-        return (float)((double)reinterpret_cast<const long long*>(acc)[i] * (1.0 / (double)kFixedScale));
-    };
+                                                         const float* __restrict__ dq0acc, int T, int D,
+                                                         const unsigned* __restrict__ scale_parts,
+                                                         const unsigned* __restrict__ poison) {
     // a null output is a gradient the caller does not want
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        if (dk1) dk1[i] = (E)value(dk1acc, i);
-        if (dv1) dv1[i] = (E)(value(duacc, i) * silu_grad_f((float)v1[i]));
-        if (dk2) dk2[i] = (E)value(dk2acc, i);
-        if (dv2) dv2[i] = (E)value(dv2acc, i);
-        if (dqacc && dq) dq[i] = (E)(value(dqacc, i) * alpha);
-        if (dq0acc && dq) {  // query tile 0 was summed over its rounds in a [BH][32][D] accumulator
-            const size_t row = i / D, t = row % T;
-            if (t < 32) dq[i] = (E)(value(dq0acc, (row / T * 32 + t) * D + i % D) * alpha);
+        const size_t row = i / D, t = row % T;
+        double inv = 0.0;
+        unsigned bad = 0;
+        if (fixed_point) {
+            inv = fixed_scale_inverse(fixed_scale_field<false>(scale_parts, (int)(row / T), kFixedBias));
+            bad = poison[row];
         }
+        auto value = [&](const float* acc, size_t at, unsigned bit) {
+            if (!fixed_point) return acc[at];
+            if (bad & bit) return __builtin_nanf("");
+            return (float)((double)reinterpret_cast<const long long*>(acc)[at] * inv);
+        };
+        if (dk1) dk1[i] = (E)value(dk1acc, i, kPoisonDK1);
+        if (dv1) dv1[i] = (E)(value(duacc, i, kPoisonDU) * silu_grad_f((float)v1[i]));
+        if (dk2) dk2[i] = (E)value(dk2acc, i, kPoisonDK2);
+        if (dv2) dv2[i] = (E)value(dv2acc, i, kPoisonDV2);
+        if (dqacc && dq) dq[i] = (E)(value(dqacc, i, kPoisonDQ) * alpha);
+        // query tile 0 was summed over its rounds in a [BH][32][D] accumulator
+        if (dq0acc && dq && t < 32) dq[i] = (E)(value(dq0acc, (row / T * 32 + t) * D + i % D, kPoisonDQ) * alpha);
     }
 }
 
 struct BwdLayout {
-    size_t u, ut, k1t, k2t, v2t, delta, lse_f32, delta_f32, dq0acc, dk1acc, duacc, dk2acc, dv2acc, dqacc, total;
+    size_t u, ut, k1t, k2t, v2t, delta, lse_f32, delta_f32, dq0acc, scale_parts, poison, dk1acc, duacc, dk2acc, dv2acc,
+        dqacc, total;
 };
 static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     const size_t Tp = (size_t)(T + 63) / 64 * 64, n = (size_t)BH * T * D;
@@ -574,6 +600,8 @@ static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     l.lse_f32 = take((size_t)BH * T * 4);    // fp32 tiles of the backward: their rows' LSE and Delta in fp32
     l.delta_f32 = take(std::max((size_t)BH * T, (size_t)BH * 32 * 4 * 3) * 4);
     l.dq0acc = take((size_t)BH * 32 * D * 8);  // dQ / alpha of query tile 0, summed over its rounds
+    l.scale_parts = take((size_t)BH * kScaleParts * 4);  // fixed point: see common.hpp
+    l.poison = take((size_t)BH * T * 4);
     const size_t acc = fixed_point ? 8 : 4;
     l.dk1acc = take(n * acc);
     l.duacc = take(n * acc);
@@ -607,7 +635,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
                        (const E*)a.k2, (const E*)a.v2, (const E*)a.o, (const E*)a.d_o, (E*)(ws + l.u),
                        (E*)(ws + l.ut), (E*)(ws + l.k1t), (E*)(ws + l.k2t), (E*)(ws + l.v2t),
                        (float*)(ws + l.delta), dk1acc, duacc, dk2acc, dv2acc, dqacc, a.T, Tp, D,
-                       a.deterministic ? 2 * D : D);
+                       a.deterministic ? 2 * D : D, a.deterministic ? (unsigned*)(ws + l.scale_parts) : nullptr,
+                       (unsigned*)(ws + l.poison));
 
     BwdParams<E> p;
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o;
@@ -616,6 +645,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha; p.causal = a.causal;
     p.acc_q = dqacc; p.splits = splits; p.fixed_point = a.deterministic ? 1 : 0;
+    p.scale_parts = (const unsigned*)(ws + l.scale_parts); p.poison = (unsigned*)(ws + l.poison);
 
     // D = 64, full windows: three stage buffers of four 64x64 tiles, two rounds of 8 K2 / V2 rows, the Q and dO
     // tiles (twice: operand and epilogue layout), four dQ slices.  Otherwise: tdp_bwd_rows_general.hpp
@@ -685,7 +715,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         f.lse_f32 = (float*)(ws + l.lse_f32); f.delta_f32 = (float*)(ws + l.delta_f32);
         f.dq0_acc = ws + l.dq0acc;
         f.dq = a.dq; f.acc_k2 = dk2acc; f.acc_v2 = dv2acc; f.acc_k1 = dk1acc; f.acc_u = duacc; f.acc_q = dqacc;
-        f.fixed_scale = a.deterministic ? kFixedScale : 0.f;
+        f.scale_parts = a.deterministic ? p.scale_parts : nullptr; f.poison = p.poison; f.scale_bias = kFixedBias;
         f.BH = a.BH; f.T = a.T; f.D = D; f.is_bf16 = a.is_bf16;
         f.alpha = a.alpha; f.causal = a.causal;
         f.k1_window = a.k1_window; f.k2_window = a.k2_window; f.kk_left = a.kk_left; f.kk_right = a.kk_right;
@@ -699,7 +729,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
-    p.acc_k = dk2acc; p.acc_v = dv2acc;
+    p.acc_k = dk2acc; p.acc_v = dv2acc; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
     // a launch whose gradients the caller does not want (null outputs) is skipped
     if (tiles_here > 0 && want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
@@ -707,7 +737,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     // rows = (K1, U), streamed = (K2, V2): dK1, dU
     p.row_k = (const E*)a.k1; p.row_v = u;
     p.st_k = (const E*)a.k2; p.st_v = (const E*)a.v2; p.st_kt = k2t; p.st_vt = v2t;
-    p.acc_k = dk1acc; p.acc_v = duacc;
+    p.acc_k = dk1acc; p.acc_v = duacc; p.bit_k = kPoisonDK1; p.bit_v = kPoisonDU;
     p.wa = a.k2_window; p.wb = a.k1_window; p.lab = a.kk_right; p.rab = a.kk_left;  // the mask with j and k exchanged
     if (tiles_here > 0 && want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
 
@@ -718,7 +748,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
                        (const float*)duacc, (const float*)dk2acc, (const float*)dv2acc, (const float*)dqacc, a.alpha,
                        (E*)a.dq, (const E*)a.v1, (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n,
                        a.deterministic ? 1 : 0,
-                       (first_in_f32 && !all_in_f32 && !dqacc) ? (const float*)(ws + l.dq0acc) : nullptr, a.T, D);
+                       (first_in_f32 && !all_in_f32 && !dqacc) ? (const float*)(ws + l.dq0acc) : nullptr, a.T, D,
+                       p.scale_parts, p.poison);
     return hipGetLastError();
 }
 

@@ -122,6 +122,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
+    const float fscale = acc_scale(p, bh);
     const E* __restrict__ K2 = p.row_k + base;
     const E* __restrict__ V2 = p.row_v + base;
 
@@ -469,8 +470,9 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                 sk += __shfl_xor(sk, 32, 64);
                 sv += __shfl_xor(sv, 32, 64);
                 if (g == 0) {
-                    accumulate(p, p.acc_k, base + (size_t)k * D + d, sk * p.alpha);
-                    accumulate(p, p.acc_v, base + (size_t)k * D + d, sv);
+                    unsigned* prow = p.poison + (size_t)bh * T + k;
+                    shared_add(p.acc_k, base + (size_t)k * D + d, sk * p.alpha, fscale, prow, p.bit_k);
+                    shared_add(p.acc_v, base + (size_t)k * D + d, sv, fscale, prow, p.bit_v);
                 }
             }
         }
@@ -506,7 +508,8 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             for (int e = 0; e < 4; ++e)
                 if (q0 + r0 + e < T) {
                     const size_t off = base + (size_t)(q0 + r0 + e) * D + d;
-                    if (p.splits > 1) accumulate(p, p.acc_q, off, out[e]);  // scaled by alpha when converted
+                    if (p.splits > 1)  // scaled by alpha when converted
+                        shared_add(p.acc_q, off, out[e], fscale, p.poison + (size_t)bh * T + q0 + r0 + e, kPoisonDQ);
                     else p.dq[off] = (E)(out[e] * p.alpha);
                 }
         }

@@ -98,6 +98,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     const int half = wave & 1, rrow = wave >> 1;
     const int T = p.T;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
+    const float fscale = acc_scale(p, bh);
     const E* __restrict__ K2 = p.row_k + base;
     const E* __restrict__ V2 = p.row_v + base;
 
@@ -415,8 +416,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
                 const int d = (grp + 4 * x) * 16 + n;
-                accumulate(p, p.acc_k, base + (size_t)k * D + d, outk[x] * p.alpha);
-                accumulate(p, p.acc_v, base + (size_t)k * D + d, outv[x]);
+                unsigned* prow = p.poison + (size_t)bh * T + k;
+                shared_add(p.acc_k, base + (size_t)k * D + d, outk[x] * p.alpha, fscale, prow, p.bit_k);
+                shared_add(p.acc_v, base + (size_t)k * D + d, outv[x], fscale, prow, p.bit_v);
             }
             if constexpr (WITH_DQ) {
 #pragma unroll
@@ -452,7 +454,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
             const int qq = q0 + 16 * hf + 4 * (ln >> 4) + i, d = dt * 16 + (ln & 15);
             if (qq < T) {
                 const size_t off = base + (size_t)qq * D + d;
-                if (p.splits > 1) accumulate(p, p.acc_q, off, v);  // scaled by alpha when converted
+                if (p.splits > 1)  // scaled by alpha when converted
+                    shared_add(p.acc_q, off, v, fscale, p.poison + (size_t)bh * T + qq, kPoisonDQ);
                 else p.dq[off] = (E)(v * p.alpha);
             }
         }

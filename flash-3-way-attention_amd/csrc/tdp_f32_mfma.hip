@@ -338,7 +338,8 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
 // kernels (dO * V2 rounded to 16 bit) cannot resolve.
 // D = 128: a workgroup produces DOUT = 64 of the gradient columns (blockIdx.y picks the half), and the B operands
 // of the score products are formed as they are used instead of being held in registers.
-constexpr float kF32FixedScale = 68719476736.0f;  // 2^36: |sum| < 1.3e8 in steps of 1.5e-11
+// the fp32 tensors' accumulators resolve 2^-36 of the slice's max |dO| and cover sums up to 2^27 times it
+constexpr int kF32FixedBias = 36;
 
 template <typename E>
 struct F32BwdParams {
@@ -351,7 +352,11 @@ struct F32BwdParams {
     // when non-null, LSE and Delta of query tile 0 come from the partials the split STATS launch left here
     const float* stats_part;
     int split_rounds;      // tile 0 only: rounds dealt out to workgroups (see tdp_f32_tile0_kernel), else 0
-    float fixed_scale;     // scale of the fixed-point accumulators; 0: the accumulators are float
+    // fixed-point accumulators (common.hpp); scale_parts null: the accumulators are float
+    const unsigned* scale_parts;
+    unsigned* poison;
+    int scale_bias;
+    unsigned bit_k, bit_v;  // poison bits of acc_k / acc_v
     int T, BH, nqt;        // nqt: query tiles this launch covers (tiles 0 .. nqt - 1)
     float alpha;
     TdpMask mask;
@@ -361,13 +366,6 @@ __device__ __forceinline__ float half_sum(float v) {  // over the 32 lanes of a 
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
-}
-
-__device__ __forceinline__ void shared_add(void* acc, size_t idx, float v, float fixed_scale) {
-    if (fixed_scale != 0.f)
-        atomicAdd(reinterpret_cast<unsigned long long*>(acc) + idx, (unsigned long long)__float2ll_rn(v * fixed_scale));
-    else
-        unsafeAtomicAdd(reinterpret_cast<float*>(acc) + idx, v);
 }
 
 // `only_round` >= 0: this workgroup walks that round of rows only
@@ -401,6 +399,7 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
     const E* __restrict__ VB = p.vb + base;
     const TdpMask mask = p.mask;
     const float scale_log2 = p.alpha * kLog2e;
+    const float fscale = p.scale_parts ? fixed_scale_value(fixed_scale_field(p.scale_parts, bh, p.scale_bias)) : 0.f;
 
     const int q0 = qt * 32, q1 = min(T - 1, q0 + 31);
     const int q = q0 + n;
@@ -537,8 +536,9 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
                     const float rv = half_sum(accT[dt][i] * sDO[n * LD + d]);
                     if (n == 0) {
                         const size_t idx = base + (size_t)b * D + d;
-                        shared_add(p.acc_k, idx, rk, p.fixed_scale);
-                        shared_add(p.acc_v, idx, rv, p.fixed_scale);
+                        unsigned* prow = p.poison + (size_t)bh * T + b;
+                        shared_add(p.acc_k, idx, rk, fscale, prow, p.bit_k);
+                        shared_add(p.acc_v, idx, rv, fscale, prow, p.bit_v);
                     }
                 }
         }
@@ -563,7 +563,7 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
                 const size_t off = base + (size_t)(q0 + r) * D + c0 + d;
                 if (p.acc_q)
                     shared_add(p.acc_q, p.acc_q_rows ? ((size_t)bh * p.acc_q_rows + q0 + r) * D + c0 + d : off,
-                               sO[d * 33 + r], p.fixed_scale);
+                               sO[d * 33 + r], fscale, p.poison + (size_t)bh * T + q0 + r, kPoisonDQ);
                 else
                     p.dq[off] = (E)(sO[d * 33 + r] * p.alpha);
             }
@@ -594,13 +594,27 @@ __global__ __launch_bounds__(512) void tdp_f32_tile0_kernel(F32BwdParams<E> r0, 
 __global__ __launch_bounds__(256) void f32_zero_kernel(long long* __restrict__ a, size_t n) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) a[i] = 0;
 }
+// the partial maxima of |dO| that fix the scale of a slice's accumulators: grid (kScaleParts, BH)
+__global__ __launch_bounds__(256) void f32_scale_kernel(const float* __restrict__ d_o, unsigned* __restrict__ parts,
+                                                        size_t per_slice) {
+    __shared__ unsigned red[4];
+    const size_t pieces = per_slice / 4, per_part = (pieces + kScaleParts - 1) / kScaleParts;
+    const size_t lo = min(pieces, blockIdx.x * per_part), hi = min(pieces, lo + per_part);
+    const unsigned m = block_absmax_bits<float>(d_o + blockIdx.y * per_slice + lo * 4, hi - lo, red);
+    if (threadIdx.x == 0) parts[blockIdx.y * kScaleParts + blockIdx.x] = m;
+}
 // fixed point -> fp32
 __global__ __launch_bounds__(256) void f32_finish_kernel(const long long* __restrict__ acc, float* __restrict__ dk_rows,
-                                                         float* __restrict__ dv_rows, size_t n) {
-    const double inv = 1.0 / (double)kF32FixedScale;
+                                                         float* __restrict__ dv_rows, size_t n, int T, int D,
+                                                         const unsigned* __restrict__ scale_parts,
+                                                         const unsigned* __restrict__ poison, unsigned bit_k,
+                                                         unsigned bit_v) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-        dk_rows[i] = (float)((double)acc[i] * inv);
-        dv_rows[i] = (float)((double)acc[n + i] * inv);
+        const size_t row = i / D;
+        const double inv = fixed_scale_inverse(fixed_scale_field<false>(scale_parts, (int)(row / T), kF32FixedBias));
+        const unsigned bad = poison[row];
+        dk_rows[i] = (bad & bit_k) ? __builtin_nanf("") : (float)((double)acc[i] * inv);
+        dv_rows[i] = (bad & bit_v) ? __builtin_nanf("") : (float)((double)acc[n + i] * inv);
     }
 }
 
@@ -625,13 +639,13 @@ hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, cons
     const dim3 grid(8 * groups * p.nqt, D / DOUT);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.ka = k1; p.va = u; p.kb = k2; p.vb = v2;
-    p.acc_k = acc_k2; p.acc_v = acc_v2;
+    p.acc_k = acc_k2; p.acc_v = acc_v2; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
     p.mask = natural;
     if (want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(512), smem, st, p);
     else if (want_k2) hipLaunchKernelGGL(kern_nodq, grid, dim3(512), smem, st, p);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU (the mask with the two key indices exchanged)
     p.ka = k2; p.va = v2; p.kb = k1; p.vb = u;
-    p.acc_k = acc_k1; p.acc_v = acc_u;
+    p.acc_k = acc_k1; p.acc_v = acc_u; p.bit_k = kPoisonDK1; p.bit_v = kPoisonDU;
     p.mask = TdpMask{natural.causal, natural.wb, natural.wa, natural.rab, natural.lab};
     if (want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(512), smem, st, p);
     return hipGetLastError();
@@ -644,12 +658,17 @@ hipError_t launch_f32_bwd(const GenericTdpArgs& a, long long* acc, hipStream_t s
     F32BwdParams<float> p{};
     p.q = a.q; p.d_o = a.d_o; p.lse = a.lse_in; p.delta = a.delta;
     p.dq = a.dq; p.acc_q = nullptr; p.acc_q_rows = 0; p.stats_part = nullptr; p.split_rounds = 0;
-    p.fixed_scale = kF32FixedScale;
+    // scratch: four accumulators, the rows' poison words, the slices' scale partials
+    const size_t rows = (size_t)a.BH * a.T, zero_n = 4 * n + (rows + 3) / 4 * 2;  // 16-byte aligned parts
+    unsigned* poison = reinterpret_cast<unsigned*>(acc + 4 * n);
+    unsigned* parts = reinterpret_cast<unsigned*>(acc + zero_n);
+    p.scale_parts = parts; p.poison = poison; p.scale_bias = kF32FixedBias;
     p.T = a.T; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
     p.alpha = a.alpha;
-    size_t gz = (4 * n + 255) / 256;
+    size_t gz = (zero_n + 255) / 256;
     if (gz > 8192) gz = 8192;
-    hipLaunchKernelGGL(f32_zero_kernel, dim3((unsigned)gz), dim3(256), 0, st, acc, 4 * n);
+    hipLaunchKernelGGL(f32_zero_kernel, dim3((unsigned)gz), dim3(256), 0, st, acc, zero_n);
+    hipLaunchKernelGGL(f32_scale_kernel, dim3(kScaleParts, a.BH), dim3(256), 0, st, a.d_o, parts, (size_t)a.T * D);
     const TdpMask natural{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
     if (hipError_t e = launch_f32_bwd_tiles<float, D>(p, a.k1, a.u, a.k2, a.v2, acc, acc + n, acc + 2 * n, acc + 3 * n,
                                                       natural, want_q, want_k2, want_k1, st);
@@ -657,8 +676,12 @@ hipError_t launch_f32_bwd(const GenericTdpArgs& a, long long* acc, hipStream_t s
         return e;
     size_t gf = (n + 255) / 256;
     if (gf > 4096) gf = 4096;
-    if (want_k2) hipLaunchKernelGGL(f32_finish_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc, a.dk2, a.dv2, n);
-    if (want_k1) hipLaunchKernelGGL(f32_finish_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc + 2 * n, a.dk1, a.du, n);
+    if (want_k2)
+        hipLaunchKernelGGL(f32_finish_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc, a.dk2, a.dv2, n, a.T, D, parts,
+                           poison, kPoisonDK2, kPoisonDV2);
+    if (want_k1)
+        hipLaunchKernelGGL(f32_finish_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc + 2 * n, a.dk1, a.du, n, a.T, D,
+                           parts, poison, kPoisonDK1, kPoisonDU);
     return hipGetLastError();
 }
 
@@ -720,7 +743,7 @@ static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
         p.o = nullptr; p.lse = nullptr; p.d_o = (const E*)a.d_o; p.delta = a.delta_f32;
         p.split_rounds = rounds;
         p.zero_ptr = own_dq_acc ? (unsigned*)a.dq0_acc : nullptr;
-        p.zero_words = own_dq_acc ? 32 * D * (a.fixed_scale != 0.f ? 2 : 1) : 0;
+        p.zero_words = own_dq_acc ? 32 * D * (a.scale_parts ? 2 : 1) : 0;
         p.T = a.T; p.BH = a.BH; p.nqt = 1;
         p.scale_log2 = a.alpha * kLog2e;
         p.mask = natural;
@@ -733,13 +756,13 @@ static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
     r0.q = (const E*)a.q; r0.d_o = (const E*)a.d_o; r0.lse = nullptr; r0.delta = nullptr;
     r0.stats_part = a.delta_f32; r0.split_rounds = rounds;
     r0.dq = (E*)a.dq; r0.acc_q = a.acc_q ? a.acc_q : a.dq0_acc; r0.acc_q_rows = a.acc_q ? 0 : 32;
-    r0.fixed_scale = a.fixed_scale;
+    r0.scale_parts = a.scale_parts; r0.poison = a.poison; r0.scale_bias = a.scale_bias;
     r0.T = a.T; r0.BH = a.BH; r0.nqt = 1; r0.alpha = a.alpha;
     F32BwdParams<E> r1 = r0;
     r0.ka = (const E*)a.k1; r0.va = (const E*)a.u; r0.kb = (const E*)a.k2; r0.vb = (const E*)a.v2;
-    r0.acc_k = a.acc_k2; r0.acc_v = a.acc_v2; r0.mask = natural;
+    r0.acc_k = a.acc_k2; r0.acc_v = a.acc_v2; r0.bit_k = kPoisonDK2; r0.bit_v = kPoisonDV2; r0.mask = natural;
     r1.ka = (const E*)a.k2; r1.va = (const E*)a.v2; r1.kb = (const E*)a.k1; r1.vb = (const E*)a.u;
-    r1.acc_k = a.acc_k1; r1.acc_v = a.acc_u;
+    r1.acc_k = a.acc_k1; r1.acc_v = a.acc_u; r1.bit_k = kPoisonDK1; r1.bit_v = kPoisonDU;
     r1.mask = TdpMask{natural.causal, natural.wb, natural.wa, natural.rab, natural.lab};
     const int roles = ((a.want_q || a.want_k2) ? 1 : 0) | (a.want_k1 ? 2 : 0) | (a.want_q ? 4 : 0);
     auto kern = tdp_f32_tile0_kernel<E, D, DOUT>;
@@ -763,7 +786,7 @@ static hipError_t first_tile_typed(const FirstTileArgs& a, hipStream_t st) {
     F32BwdParams<E> p{};
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o; p.lse = a.lse_f32; p.delta = a.delta_f32;
     p.dq = (E*)a.dq; p.acc_q = a.acc_q; p.acc_q_rows = 0; p.stats_part = nullptr; p.split_rounds = 0;
-    p.fixed_scale = a.fixed_scale;
+    p.scale_parts = a.scale_parts; p.poison = a.poison; p.scale_bias = a.scale_bias;
     p.T = a.T; p.BH = a.BH; p.nqt = a.tiles;
     p.alpha = a.alpha;
     const TdpMask natural{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
@@ -788,7 +811,9 @@ hipError_t f32_mfma_tdp_fwd(const GenericTdpArgs& a, hipStream_t st) {
     return hipErrorInvalidValue;
 }
 
-size_t f32_mfma_tdp_bwd_scratch_elems(int BH, int T, int D) { return 4 * (size_t)BH * T * D; }
+size_t f32_mfma_tdp_bwd_scratch_elems(int BH, int T, int D) {
+    return 4 * (size_t)BH * T * D + ((size_t)BH * T + 3) / 4 * 2 + (size_t)BH * kScaleParts / 2;
+}
 
 hipError_t f32_mfma_tdp_bwd(const GenericTdpArgs& a, long long* scratch, hipStream_t st) {
     if (a.D == 32) return launch_f32_bwd<32>(a, scratch, st);

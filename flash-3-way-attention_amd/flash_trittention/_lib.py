@@ -24,7 +24,7 @@ _vp, _i, _f, _sz, _u = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_s
 _PROTOS = {
     "tritt_version": (_i, []),
     "tritt_status_string": (ctypes.c_char_p, [_i]),
-    "tritt_set_tuning": (_i, [_i, _i]),
+    "tritt_set_tuning": (_i, [_i, _i, ctypes.POINTER(_i)]),
     "tritt_probe_mfma": (_i, [_vp, _i, _i, _vp]),
     "tritt_tdp_fwd_workspace_bytes": (_sz, [_i] * 10 + [_u]),
     "tritt_tdp_fwd": (_i, [_vp] * 7 + [_i] * 5 + [_f] + [_i] * 5 + [_vp, _sz, _u, _vp]),
@@ -73,7 +73,9 @@ TUNE_FWD_SPLITS, TUNE_FWD_BAND, TUNE_BWD_SPLITS, TUNE_BWD128_WAVES, TUNE_F32_VAL
 def set_tuning(knob: int, value: int) -> int:
     """tritt_set_tuning, returning the previous value; remembered workspace sizes may depend on the knobs."""
     _workspace_sizes.clear()
-    return lib().tritt_set_tuning(knob, value)
+    previous = _i(0)
+    check(lib().tritt_set_tuning(knob, value, ctypes.byref(previous)), "tritt_set_tuning")
+    return previous.value
 
 
 class tuning:

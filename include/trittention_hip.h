@@ -60,23 +60,23 @@ const char* tritt_status_string(int status);
 /* Tuning overrides for sweeps and tests; production callers never need them.  Each knob
  * starts from an environment variable that is read once per process (the first time any
  * entry point needs it), so a *_workspace_bytes query and the launch that follows always see
- * the same value; tritt_set_tuning changes a knob afterwards and returns its previous value
- * (TRITT_ERR_INVALID for an unknown knob).  0 = automatic.  Process-wide: do not change a knob
- * while another thread is inside the library.
+ * the same value; tritt_set_tuning changes a knob afterwards, stores its previous value in
+ * *previous (which may be NULL) and returns TRITT_OK, or TRITT_ERR_INVALID for an unknown knob.
+ * 0 = automatic.  Process-wide: do not change a knob while another thread is inside the library.
  *   TRITT_TUNE_FWD_SPLITS   (env TRITT_FWD_SPLITS)     workgroups per query tile in the triple-dot forward, 1..8
  *   TRITT_TUNE_FWD_BAND     (env TRITT_FWD_BAND=0)     -1: narrow windowed masks take the streaming forward
  *                                                      instead of the band-resident one
  *   TRITT_TUNE_BWD_SPLITS   (env TRITT_BWD_SPLITS)     workgroups per query tile in the triple-dot backward, 1..16
  *   TRITT_TUNE_BWD128_WAVES (env TRITT_BWD128_VARIANT=w8|w4)  the D = 128 backward under full windows: 0 = 16 queries per
  *                           wave on 16x16x32 tiles (the default); 8 | 4 = the 32-query kernels with 8 or 4 waves
- *   TRITT_TUNE_F32_VALU     1: the fp32 path runs the VALU kernels at every head dimension (instead of the
+ *   TRITT_TUNE_F32_VALU     (env TRITT_F32_VALU=1)     1: the fp32 path runs the VALU kernels at every head dimension (instead of the
  *                           fp32 MFMA kernels at D = 32, 64 and 128)
  *   TRITT_TUNE_DPS_WAVES    waves per workgroup of the dot-product-sum MFMA kernels at D = 64: 2 | 4
  *   TRITT_TUNE_DPS_PAIR     dot-product-sum MFMA kernels: 1 = a workgroup always takes two owner tiles (a long and a
  *                           short one), -1 = never */
 enum { TRITT_TUNE_FWD_SPLITS = 0, TRITT_TUNE_FWD_BAND = 1, TRITT_TUNE_BWD_SPLITS = 2, TRITT_TUNE_BWD128_WAVES = 3,
        TRITT_TUNE_F32_VALU = 4, TRITT_TUNE_DPS_WAVES = 5, TRITT_TUNE_DPS_PAIR = 6, TRITT_TUNE_COUNT_ = 7 };
-int tritt_set_tuning(int knob, int value);
+int tritt_set_tuning(int knob, int value, int* previous);
 
 /* ---- triple-dot-product:  s[q,j,k] = alpha * sum_d Q[q,d] K1[j,d] K2[k,d] ----------------
  * O[q] = sum_{j,k} softmax_{(j,k)}(s[q]) * SiLU(V1[j]) * V2[k].
@@ -95,13 +95,18 @@ int tritt_set_tuning(int knob, int value);
  *   {dk2, dv2} and {dk1, dv1}).  On the 16-bit MFMA path
  *   (16-bit tensors, D = 32, 64 or 128, any mask) the workgroups of different query tiles add their
  *   shares of dK1/dV1/dK2/dV2 (and of dQ, when a small grid splits a tile's rows) to common
- *   accumulators.  The shares are added as 64-bit fixed point (steps of 2^-30, |sum| below 8.6e9)
- *   with integer atomics, whose result does not depend on the order of arrival: like the
- *   reference's owner-computes kernels, and like every other entry point here, the call is
- *   bitwise reproducible from run to run (measured cost against fp32 atomics: none).
- *   TRITT_FLAG_FLOAT_ATOMICS selects fp32 atomics instead (reproducible to rounding only; no
- *   bound on the magnitude of the sums; accumulators half the size: pass the same flags to
- *   tritt_tdp_bwd_workspace_bytes).  Workspace of the MFMA path: about 15 (fixed point: 25) times
+ *   accumulators.  The shares are added as 64-bit fixed point with integer atomics, whose result
+ *   does not depend on the order of arrival: like the reference's owner-computes kernels, and
+ *   like every other entry point here, the call is bitwise reproducible from run to run
+ *   (measured cost against fp32 atomics: none).  The fixed-point scale is a power of two chosen
+ *   per (batch, head) slice from the largest finite |dO| of the slice: steps of 2^-30 of that
+ *   magnitude (2^-36 on the fp32 matrix-core kernels), sums up to 2^33 (2^27) times it, so the
+ *   backward is exactly homogeneous in dO for powers of two (loss scaling, mean-reduced losses)
+ *   and has no absolute floor, like the reference's fp32 accumulators
+ *   (triple_dot_product/kernels/bwd_dk1.py:239-258).  A share that is NaN, Inf or beyond the
+ *   accumulator's range makes that row of that gradient NaN in the output.
+ *   TRITT_FLAG_FLOAT_ATOMICS selects fp32 atomics instead (reproducible to rounding only;
+ *   accumulators half the size: pass the same flags to tritt_tdp_bwd_workspace_bytes).  Workspace of the MFMA path: about 15 (fixed point: 25) times
  *   one 16-bit [B,H,T,D] tensor (five accumulators, four transposed copies, SiLU(V1)).
  */
 size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,

@@ -871,3 +871,78 @@ def test_config3_rows_sum_to_one():
     out, _ = util.run_tdp(inputs, 1 / 8, True, backward=False)
     want = torch.nn.functional.silu(v1.float()).to(torch.bfloat16).float()
     util.assert_close("out", out, want, rtol=2e-2, atol=2e-2)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Range of the backward's common accumulators.  The reference accumulates every gradient in fp32
+# (triple_dot_product/kernels/bwd_dk1.py:239-258): no floor under small gradients, non-finite values propagate.
+# Here the shares of dK1/dV1/dK2/dV2 (and of a split dQ) are 64-bit fixed point whose scale follows the largest
+# |dO| of each (batch, head) slice, so the whole backward is exactly homogeneous in dO for powers of two.
+
+@pytest.mark.parametrize("case", ["config2 bf16 (rows split, dQ accumulated)", "fp32 tensors on the fp32 matrix-core kernels",
+                                  "bf16, one workgroup per query tile", "bf16 D=128", "bf16 windowed D=64"])
+def test_backward_is_exactly_homogeneous_in_dO(case, tune):
+    """dO * 2^-40 (a mean-reduced loss over many tokens, no loss scaling) and dO * 2^+20 (loss scaling) give all
+    five gradients bitwise equal to the unscaled run's times that power of two: nothing in the path has an
+    absolute resolution or an absolute range."""
+    print(f"case homogeneous: {case}", flush=True)
+    windows = (None,) * 4
+    if case.startswith("config2"):
+        inputs, alpha = orc.make_inputs(2, 4, 256, 64, torch.bfloat16, seed=2), 1 / 8
+    elif case.startswith("fp32"):
+        inputs, alpha = orc.make_inputs(2, 4, 256, 64, torch.float32, seed=3), 1 / 8
+    elif case.endswith("per query tile"):
+        inputs, alpha = orc.make_inputs(1, 2, 300, 64, torch.bfloat16, seed=4), 1 / 8
+        tune(_lib.TUNE_BWD_SPLITS, 1)
+    elif case.endswith("D=128"):
+        inputs, alpha = orc.make_inputs(1, 3, 203, 128, torch.bfloat16, seed=5), 1 / math.sqrt(128)
+    else:
+        inputs, alpha, windows = orc.make_inputs(1, 4, 400, 64, torch.bfloat16, seed=6), 1 / 8, (200, 150, 60, 90)
+    run = lambda power: util.run_tdp(list(inputs[:5]) + [inputs[5] * 2.0 ** power], alpha, True, windows)[1]
+    base = run(0)
+    for power in (-40, 20):
+        got = run(power)
+        for name, a, b in zip(util.NAMES, got, base):
+            assert torch.isfinite(a).all(), (name, power)
+            assert torch.equal(a, b * 2.0 ** power), (name, power, (a - b * 2.0 ** power).abs().max().item())
+
+
+@pytest.mark.parametrize("dtype,factor", [(torch.bfloat16, 1e-6), (torch.bfloat16, 1e4), (torch.float32, 4.8e-7),
+                                          (torch.float32, 1e4)])
+def test_small_and_large_incoming_gradients_against_oracle(dtype, factor):
+    """dO of the size `out.mean().backward()` leaves at the headline shape (4.8e-7), and of a scaled loss: every
+    gradient meets the usual bar relative to its own magnitude (the tolerances scale with dO)."""
+    print(f"case dO x {factor} {dtype}", flush=True)
+    inputs = orc.make_inputs(2, 4, 256, 64, dtype, seed=11)
+    inputs = list(inputs[:5]) + [(inputs[5].float() * factor).to(dtype)]
+    tol = FP32 if dtype == torch.float32 else LOWP
+    _, _, grads = util.oracle_tdp(inputs, 1 / 8, True)
+    _, g = util.run_tdp(inputs, 1 / 8, True)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a / factor, b / factor, **tol)
+        assert util.rel_err(a, b) <= (1e-4 if dtype == torch.float32 else 2e-2), (name, util.rel_err(a, b))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("bad", [float("nan"), float("inf")])
+def test_non_finite_dO_gives_non_finite_gradients(dtype, bad):
+    """A NaN or Inf in dO[b, h, q] reaches dQ[q] and every row j <= q, k <= q of that head's dK1/dV1/dK2/dV2 as
+    a non-finite value, as it does through the reference's fp32 accumulators (fp16 training with a GradScaler
+    skips the step on exactly that); the other heads keep their gradients bit for bit, and so do the rows of
+    the same head past the query tile of q."""
+    print(f"case non-finite dO {dtype} {bad}", flush=True)
+    B, H, T, D, q = 2, 4, 256, 64, 100
+    inputs = orc.make_inputs(B, H, T, D, dtype, seed=13)
+    _, base = util.run_tdp(inputs, 1 / 8, True)
+    do = inputs[5].clone()
+    do[1, 2, q, 5] = bad
+    _, g = util.run_tdp(list(inputs[:5]) + [do], 1 / 8, True)
+    for name, a, b in zip(util.NAMES, g, base):
+        if name == "dq":
+            assert not torch.isfinite(a[1, 2, q]).any(), name
+        else:
+            assert not torch.isfinite(a[1, 2, : q + 1]).any(), name
+            assert torch.equal(a[1, 2, 128:], b[1, 2, 128:]), name
+        a = a.clone()
+        a[1, 2] = b[1, 2]
+        assert torch.equal(a, b), f"{name}: another head changed"
