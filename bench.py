@@ -232,12 +232,14 @@ def dps_times(torch, dev, B, H, T, D, steps, warmup):
             "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} bf16 causal"}}
 
 
-def tdp_times(torch, flash_trittention, dev, B, H, T, D, dtype, steps, warmup, backward=True):
-    """Triple-dot forward (and backward) milliseconds at one shape, full windows."""
+def tdp_times(torch, flash_trittention, dev, B, H, T, D, dtype, steps, warmup, backward=True, convert=False):
+    """Triple-dot forward (and backward) milliseconds at one shape, full windows.  `convert`: the reference's
+    convert_to_float32=True (what its own benchmark scripts pass: scripts/benchmark_triple_dot_product.py:172)."""
     alpha = 1 / math.sqrt(D)
     q, k1, k2, v1, v2, do = (t.to(dev) for t in make_inputs(B, H, T, D, dtype, seed=0))
     leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
-    kw = dict(softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True)
+    kw = dict(softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True,
+              convert_to_float32=convert)
     hold = {}
 
     def fwd():
@@ -248,7 +250,8 @@ def tdp_times(torch, flash_trittention, dev, B, H, T, D, dtype, steps, warmup, b
         hold["o"].backward(do, retain_graph=True)
 
     n = triples(B, H, T)
-    row = {"workload": f"triple-dot B={B} H={H} T={T} D={D} {str(dtype).split('.')[-1]} causal",
+    row = {"workload": f"triple-dot B={B} H={H} T={T} D={D} {str(dtype).split('.')[-1]} causal"
+                       + (" convert_to_float32=True" if convert else ""),
            "fwd_ms": time_events(fwd, steps, warmup, torch)}
     row["fwd_tflops"] = 4 * D * n / row["fwd_ms"] / 1e9
     if backward:
@@ -276,6 +279,7 @@ def main():
                          "T=256/512/1024 full windows, T=2048 windows 128,128,32,32), its best H100 / B200 figures beside ours")
     ap.add_argument("--windows", default="", help="k1_window,k2_window,kk_left,kk_right for --mode tdp (empty: full)")
     ap.add_argument("--dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="tensor type for --mode tdp")
+    ap.add_argument("--convert", action="store_true", help="--mode tdp: pass convert_to_float32=True")
     ap.add_argument("--B", type=int, default=4)
     ap.add_argument("--H", type=int, default=8)
     ap.add_argument("--T", type=int, default=1024)
@@ -338,6 +342,8 @@ def main():
     q, k1, k2, v1, v2, do = (t.to(dev) for t in make_inputs(B, H, T, D, tdtype, seed=0))
     leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
     kw = dict(softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None, kk_right=None, causal=True)
+    if args.mode == "tdp" and args.convert:
+        kw["convert_to_float32"] = True
 
     def fwd_only():
         with torch.no_grad():
@@ -370,7 +376,7 @@ def main():
         print(json.dumps({"metric": "triple-dot trittention fwd / bwd", "unit": "ms", "fwd_ms": ms_fwd, "bwd_ms": ms_bwd,
                           "fwd_tflops": f_fwd / ms_fwd / 1e9, "bwd_tflops": f_bwd / ms_bwd / 1e9, "valid_triples": n,
                           "config": {"workload": f"triple-dot fwd+bwd B={B} H={H} T={T} D={D} {args.dtype} causal",
-                                     "windows": win}}), flush=True)
+                                     "windows": win, "convert_to_float32": bool(args.convert)}}), flush=True)
         return
 
     if args.mode == "fwd":
@@ -447,6 +453,10 @@ def main():
             "config1_tdp_fwd_fp32": tdp_times(torch, flash_trittention, dev, 1, 2, 64, 32, torch.float32, 20, 5,
                                               backward=False),
             "config2_tdp_fwd_bwd": tdp_times(torch, flash_trittention, dev, 2, 4, 256, 64, torch.bfloat16, 20, 5),
+            # the headline shape as the reference's own scripts call it (convert_to_float32=True): the score
+            # operands as hi + lo pairs on the same matrix-core kernels
+            "config3_tdp_fwd_bwd_convert_to_float32": tdp_times(torch, flash_trittention, dev, 4, 8, 1024, 64,
+                                                               torch.bfloat16, short, 2, convert=True),
             "config4_dps_fwd_bwd": dps_times(torch, dev, 4, 8, 1024, 64, 20, 5),
             "config5_tdp_fwd_sweep": {"workload": "triple-dot fwd B=1 H=16 D=128 bf16 causal",
                                       "rows": sweep_rows(torch, flash_trittention, dev, short)},

@@ -350,6 +350,12 @@ bool full_windows(int T, int causal, int w1, int w2, int kl, int kr) {
     return !causal || (w1 >= T - 1 && w2 >= T - 1 && kl >= T - 1 && kr >= T - 1);
 }
 
+// TRITT_FLAG_SPLIT_OPERANDS applies where the 16-bit MFMA kernels have a split-operand form
+bool use_split(int D, int dtype, unsigned flags) {
+    return (flags & TRITT_FLAG_SPLIT_OPERANDS) && !(flags & TRITT_FLAG_FORCE_GENERIC) &&
+           mfma_tdp_split_supported(D, dtype != TRITT_F32);
+}
+
 bool use_mfma_fwd(int T, int D, int dtype, int causal, int w1, int w2, int kl, int kr, unsigned flags) {
     if (flags & TRITT_FLAG_FORCE_GENERIC) return false;
     (void)T; (void)causal; (void)w1; (void)w2; (void)kl; (void)kr;  // any mask: windows take the banded instantiation
@@ -438,13 +444,14 @@ const char* tritt_status_string(int status) {
 
 // the fields of MfmaFwdArgs that describe the problem (no pointers)
 static MfmaFwdArgs mfma_fwd_shape(int B, int H, int T, int D, int dtype, int causal, int k1_window, int k2_window,
-                                  int kk_left, int kk_right) {
+                                  int kk_left, int kk_right, unsigned flags) {
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
     MfmaFwdArgs a{};
     a.BH = B * H; a.T = T; a.D = D; a.causal = causal ? 1 : 0;
     a.is_bf16 = dtype == TRITT_BF16;
     a.windowed = full_windows(T, causal, w1, w2, kl, kr) ? 0 : 1;
     a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+    a.split = use_split(D, dtype, flags) ? 1 : 0;
     return a;
 }
 
@@ -452,7 +459,7 @@ size_t tritt_tdp_fwd_workspace_bytes(int B, int H, int T, int D, int dtype, int 
                                      int kk_left, int kk_right, unsigned flags) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
     if (use_mfma_fwd(T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags))
-        return mfma_tdp_fwd_workspace(mfma_fwd_shape(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right));
+        return mfma_tdp_fwd_workspace(mfma_fwd_shape(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags));
     Arena ar(nullptr);
     tdp_fwd_generic(ar, false, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, B, H, T, D, dtype, 0.f,
                     causal, k1_window, k2_window, kk_left, kk_right, nullptr);
@@ -472,10 +479,12 @@ int tritt_tdp_fwd(const void* q, const void* k1, const void* k2, const void* v1,
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
     const bool mfma = use_mfma_fwd(T, D, dtype, causal, w1, w2, kl, kr, flags);
     if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;
+    // the caller sized `o` for two tensors: a path that writes one would leave the residual undefined
+    if ((flags & TRITT_FLAG_SPLIT_OPERANDS) && !(mfma && use_split(D, dtype, flags))) return TRITT_ERR_UNSUPPORTED;
     const size_t need = tritt_tdp_fwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
     if (need && (!workspace || workspace_bytes < need)) return TRITT_ERR_WORKSPACE;
     if (mfma) {
-        MfmaFwdArgs a = mfma_fwd_shape(B, H, T, D, dtype, causal, w1, w2, kl, kr);
+        MfmaFwdArgs a = mfma_fwd_shape(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
         a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.lse = lse; a.ut = workspace;
         a.alpha = alpha;
         return (int)mfma_tdp_fwd(a, (hipStream_t)stream);
@@ -533,6 +542,7 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
     const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
     const bool mfma = use_mfma_bwd(T, D, dtype, causal, w1, w2, kl, kr, flags);
     if ((flags & TRITT_FLAG_FORCE_MFMA) && !mfma) return TRITT_ERR_UNSUPPORTED;
+    if ((flags & TRITT_FLAG_SPLIT_OPERANDS) && !(mfma && use_split(D, dtype, flags))) return TRITT_ERR_UNSUPPORTED;
     const size_t need = tritt_tdp_bwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
     if (need && (!workspace || workspace_bytes < need)) return TRITT_ERR_WORKSPACE;
     if (mfma) {
@@ -544,6 +554,7 @@ int tritt_tdp_bwd(const void* q, const void* k1, const void* k2, const void* v1,
         a.windowed = full_windows(T, causal, w1, w2, kl, kr) ? 0 : 1;
         a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
         a.deterministic = (flags & TRITT_FLAG_FLOAT_ATOMICS) ? 0 : 1;
+        a.split = use_split(D, dtype, flags) ? 1 : 0;
         return (int)mfma_tdp_bwd(a, (hipStream_t)stream);
     }
     Arena ar(workspace);

@@ -100,8 +100,12 @@ struct MfmaFwdArgs {
     int is_bf16;  // else fp16
     int windowed;  // some window can exclude a pair with j, k <= q: the banded instantiation
     int k1_window, k2_window, kk_left, kk_right;
+    // split operands (D = 32, 64): the Q (.) K2 operand of the score products as a hi + lo pair of 16-bit numbers;
+    // `o` then holds two [BH][T][D] tensors, the output and its rounding residual
+    int split;
 };
-// needs BH, T, D, causal, windowed and the four windows of `a`
+bool mfma_tdp_split_supported(int D, int dtype_is_16bit);
+// needs BH, T, D, causal, windowed, split and the four windows of `a`
 size_t mfma_tdp_fwd_workspace(const MfmaFwdArgs& a);
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st);
@@ -119,6 +123,9 @@ struct MfmaBwdArgs {
     int windowed;  // some window can exclude a pair with j, k <= q: the banded kernels
     int k1_window, k2_window, kk_left, kk_right;
     int deterministic;  // 64-bit fixed-point accumulators: bitwise reproducible gradients
+    // split operands (D = 32, 64): Q (.) K2 and dO (.) V2 as hi + lo pairs; `o` holds the output followed by its
+    // rounding residual (what the forward wrote under the same flag), and Delta is formed from their sum
+    int split;
 };
 size_t mfma_tdp_bwd_workspace(int BH, int T, int D, bool deterministic);
 bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit);

@@ -481,7 +481,8 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
                                                        float* __restrict__ zero_d, float* __restrict__ zero_e, int T,
                                                        int Tp, int D, int zero_width,
                                                        unsigned* __restrict__ scale_parts,
-                                                       unsigned* __restrict__ poison) {
+                                                       unsigned* __restrict__ poison,
+                                                       const E* __restrict__ o_res) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * Tp;
     if (scale_parts) {
@@ -532,8 +533,14 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
         if (j < T) {
             const size_t off = base + (size_t)j * D + c * 8;
             const e8 a = *reinterpret_cast<const e8*>(o + off), b = *reinterpret_cast<const e8*>(d_o + off);
+            if (o_res) {  // split operands: the output to 16 mantissa bits (rounded value + rounding residual)
+                const e8 r = *reinterpret_cast<const e8*>(o_res + off);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) part += (float)a[e] * (float)b[e];
+                for (int e = 0; e < 8; ++e) part += ((float)a[e] + (float)r[e]) * (float)b[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) part += (float)a[e] * (float)b[e];
+            }
         }
         for (int off = cpr >> 1; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
         if (c == 0 && j < T) delta[(size_t)bh * T + j] = part;
@@ -636,7 +643,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
                        (E*)(ws + l.ut), (E*)(ws + l.k1t), (E*)(ws + l.k2t), (E*)(ws + l.v2t),
                        (float*)(ws + l.delta), dk1acc, duacc, dk2acc, dv2acc, dqacc, a.T, Tp, D,
                        a.deterministic ? 2 * D : D, a.deterministic ? (unsigned*)(ws + l.scale_parts) : nullptr,
-                       (unsigned*)(ws + l.poison));
+                       (unsigned*)(ws + l.poison),
+                       a.split ? (const E*)a.o + (size_t)a.BH * a.T * D : (const E*)nullptr);
 
     BwdParams<E> p;
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o;
@@ -658,6 +666,19 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         smem = bwdg_smem(32, 8, 32, true);
         kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true>;
         kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true>;
+        if (a.split) {
+            kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true, true>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true, true>;
+        }
+    } else if (a.split) {
+        // split operands: the general kernel (banded instantiation: full windows are windows of T)
+        if constexpr (D == 64) {
+            smem = bwdg_smem(64, 8, 64, true);
+            kern_dq = tdp_bwd_rows_general_kernel<E, 64, true, 8, 64, true, true>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 64, false, 8, 64, true, true>;
+        } else {
+            return hipErrorInvalidValue;
+        }
     } else if (a.windowed && D == 128 && knobs().bwd128_variant != 8) {
         // the 16-query kernel (tdp_bwd_rows_q16.hpp), banded instantiation
         if constexpr (D == 128) {

@@ -66,7 +66,11 @@ constexpr size_t bwdg_smem(int d, int nw, int ncol, bool with_dq) {
            + (ncol == 64 ? 2 * (2 * 64 * 16 * 2) : 0);          // Q and dO in accumulator layout (NCOL = 64)
 }
 
-template <typename E, int D, bool WITH_DQ, int NW, int NCOL, bool WIN>
+// SPLIT: the B operands of the score products, alpha log2e Q (.) K2[k] and dO (.) V2[k], are kept as hi + lo pairs
+// of 16-bit numbers (16 mantissa bits together; the streamed K1 / U operands are exact), two MFMAs per k-step: S
+// and dP then carry fp32 accumulation error only, and dS = P (dP - Delta) no longer cancels numbers that carry
+// 16-bit operand rounding.
+template <typename E, int D, bool WITH_DQ, int NW, int NCOL, bool WIN, bool SPLIT = false>
 __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -85,6 +89,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     static_assert((NW == 8 && NCOL == 64 && D >= 64) || (D == 128 && NW == 4 && NCOL == 128) ||
                   (D == 32 && NW == 8 && NCOL == 32), "workgroup shapes");
     static_assert(NBLK % NW == 0, "whole blocks per wave");
+    static_assert(!SPLIT || D <= 64, "split operands: the lo halves of a D = 128 round do not fit the register file");
 
     extern __shared__ __align__(16) char smem[];
     E* sStage = reinterpret_cast<E*>(smem);  // [NBUF][K1 rows 4096 | U rows 4096 | K1^T 2048 | U^T 2048]
@@ -264,6 +269,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
         }
 
         v8 bq[KS], bg[KS];
+        [[maybe_unused]] v8 bql[SPLIT ? KS : 1], bgl[SPLIT ? KS : 1];
         bool built = false;
         f32x16 accQ[DT], accT[DT];
 #pragma unroll
@@ -308,15 +314,28 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                         }
                     }
                     v8 a, b;
+                    [[maybe_unused]] v8 al, bl;
 #pragma unroll
                     for (int e = 0; e < 8; e += 2) {
-                        const v2 pa = M::pack((float)kv[e] * qf[e], (float)kv[e + 1] * qf[e + 1]);
-                        const v2 pb = M::pack((float)vv[e] * df[e], (float)vv[e + 1] * df[e + 1]);
+                        const float a0 = (float)kv[e] * qf[e], a1 = (float)kv[e + 1] * qf[e + 1];
+                        const float b0 = (float)vv[e] * df[e], b1 = (float)vv[e + 1] * df[e + 1];
+                        const v2 pa = M::pack(a0, a1);
+                        const v2 pb = M::pack(b0, b1);
                         a[e] = pa[0]; a[e + 1] = pa[1];
                         b[e] = pb[0]; b[e + 1] = pb[1];
+                        if constexpr (SPLIT) {
+                            const v2 la = M::pack(a0 - (float)pa[0], a1 - (float)pa[1]);
+                            const v2 lb = M::pack(b0 - (float)pb[0], b1 - (float)pb[1]);
+                            al[e] = la[0]; al[e + 1] = la[1];
+                            bl[e] = lb[0]; bl[e + 1] = lb[1];
+                        }
                     }
                     bq[ks] = a;
                     bg[ks] = b;
+                    if constexpr (SPLIT) {
+                        bql[ks] = al;
+                        bgl[ks] = bl;
+                    }
                 }
             }
 
@@ -375,6 +394,10 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             for (int ks = 0; ks < KB; ++ks) {
                 s = M::mma(ak[ks], bq[ks], s);
                 dp = M::mma(au[ks], bg[ks], dp);
+                if constexpr (SPLIT) {
+                    s = M::mma(ak[ks], bql[ks], s);
+                    dp = M::mma(au[ks], bgl[ks], dp);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (KS > 4) {
@@ -399,21 +422,37 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                 }
             __builtin_amdgcn_sched_barrier(0);
             v8 pa[2], da[2];
+            // SPLIT, in the launch that produces dQ: dS as a hi + lo pair too.  dQ[q] sums dS K1 (.) K2 over the (j, k)
+            // of ONE softmax row, terms of both signs that cancel when the row is close to one-hot, so the 8-bit
+            // rounding of a single 16-bit operand shows there (measured: 1.4 x the tolerance at scores spanning
+            // hundreds, 0.2 x with the pair).  The row gradients sum over many queries and P feeds sums of one
+            // sign: neither needs it (the launch without dQ stays at one operand).
+            constexpr bool SPLIT_DS = SPLIT && WITH_DQ;
+            [[maybe_unused]] v8 dal[SPLIT_DS ? 2 : 1];
             auto softmax_pair = [&](int r) {  // register pair r (0..7): P = exp2(S), dS = P dP, packed
                 const int h = r >> 2, e = 2 * (r & 3), i = h * 8 + e;
                 const float p0 = fast_exp2(s[i]), p1 = fast_exp2(s[i + 1]);
                 const v2 pp = M::pack(p0, p1);
-                const v2 dd = M::pack(p0 * dp[i], p1 * dp[i + 1]);
+                const float d0 = p0 * dp[i], d1 = p1 * dp[i + 1];
+                const v2 dd = M::pack(d0, d1);
                 pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
                 da[h][e] = dd[0]; da[h][e + 1] = dd[1];
+                if constexpr (SPLIT_DS) {
+                    const v2 dl = M::pack(d0 - (float)dd[0], d1 - (float)dd[1]);
+                    dal[h][e] = dl[0]; dal[h][e + 1] = dl[1];
+                }
             };
 #pragma unroll
             for (int r = 0; r < 4; ++r) softmax_pair(r);
             __builtin_amdgcn_sched_barrier(0);
             // gradient product r of half h (0 .. 2 DT - 1): even -> Tv += P U, odd -> Yq += dS K1
             auto grad = [&](int h, int r) {
-                if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[h], bt[r >> 1][h], accT[r >> 1]);
-                else accQ[r >> 1] = M::mma(da[h], bk[r >> 1][h], accQ[r >> 1]);
+                if ((r & 1) == 0) {
+                    accT[r >> 1] = M::mma(pa[h], bt[r >> 1][h], accT[r >> 1]);
+                } else {
+                    accQ[r >> 1] = M::mma(da[h], bk[r >> 1][h], accQ[r >> 1]);
+                    if constexpr (SPLIT_DS) accQ[r >> 1] = M::mma(dal[h], bk[r >> 1][h], accQ[r >> 1]);
+                }
             };
 #pragma unroll
             for (int r = 0; r < 4; ++r) {

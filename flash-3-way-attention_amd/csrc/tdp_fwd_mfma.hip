@@ -39,6 +39,7 @@ struct FwdParams {
     const E *q, *k1, *k2, *v2;
     const E* ut;  // [BH][D][Tp]  SiLU(V1) transposed, zero padded to Tp (multiple of 64)
     E* o;
+    E* o_res;  // SPLIT: the rounding residual of every output element, O(fp32) - O(16 bit), as a second tensor
     float* lse;
     int T, Tp, BH, nqt;
     float scale_log2;
@@ -55,6 +56,8 @@ struct FwdParams {
 
 constexpr float kLazyThreshold = 8.0f;
 
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+
 // Smallest row sum the FAST sweep (P = exp2(score), reference 0) accepts.  bf16 has the exponent range of fp32, so
 // only a vanished sum is refused.  fp16 loses mantissa bits below 2^-14 and flushes below 2^-24: a row whose sum is
 // under 2^-10 was summed from values in that range and is redone with a running maximum.
@@ -70,7 +73,15 @@ __device__ __forceinline__ constexpr float fast_row_sum_floor() {
 // MDIAG (NT = 1 only): the stages on the causal diagonal run the interleaved loop too, masked through the C
 // operand, instead of the general loop.  Pays on short sequences, where those stages are a large share of the
 // work; costs registers (a few more scratch reloads at D = 128), so long sequences keep the general loop.
-template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false>
+// SPLIT: the B operand of the score product, alpha log2e Q[q] (.) K2[k], is a product of two 16-bit numbers and a
+// scale: rounded to one 16-bit operand it loses half its bits, and scores that span hundreds then differ from the
+// exact ones by more than the softmax can absorb.  SPLIT keeps it as hi + lo (hi = the rounded product, lo = the
+// rounded remainder: 16 mantissa bits together) and issues two score MFMAs per k-step, K1 hi and K1 lo.  K1 itself
+// is exact (an input), so the scores carry fp32 accumulation error only.  The lo operands live in LDS (one
+// kilobyte per tile and k-step, private to the wave).  The output is stored with its rounding residual (o_res), so
+// the backward's Delta = rowsum(dO * O) does not inherit the 16-bit rounding of O.  (P as a hi + lo pair in the
+// value product was measured as well: no effect on any gradient at scores spanning hundreds, 40 % more time.)
+template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false, bool SPLIT = false>
 __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -95,6 +106,8 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     float* sQ = reinterpret_cast<float*>(sV2 + 2 * 32 * LDK);  // [BQ][LDQ] Q * alpha*log2(e), fp32
     float* sW = sQ + BQ * LDQ;                                  // [WAVES][32] per-wave scratch
     int* sFlag = reinterpret_cast<int*>(sW + WAVES * 32);
+    // SPLIT: lo operands of this wave's tiles, [NT][KS][64 lanes][8]
+    [[maybe_unused]] E* sLo = reinterpret_cast<E*>(sFlag + 4) + (size_t)wave_index() * (NT * KS * 512);
 
     // heavy-first, XCD-aware block order: consecutive block ids go to different XCDs, so give
     // every XCD its own set of heads (their K/V stay in that XCD's L2) and hand out the
@@ -289,15 +302,27 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                 const float4 qa = *reinterpret_cast<const float4*>(qp), qb = *reinterpret_cast<const float4*>(qp + 4);
                 const float qf[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
                 v8 r;
+                [[maybe_unused]] v8 rl;
 #pragma unroll
                 for (int e = 0; e < 8; e += 2) {
-                    const v2 pr = M::pack((float)kv[e] * qf[e], (float)kv[e + 1] * qf[e + 1]);
+                    const float x0 = (float)kv[e] * qf[e], x1 = (float)kv[e + 1] * qf[e + 1];
+                    const v2 pr = M::pack(x0, x1);
                     r[e] = pr[0];
                     r[e + 1] = pr[1];
+                    if constexpr (SPLIT) {
+                        const v2 pl = M::pack(x0 - (float)pr[0], x1 - (float)pr[1]);
+                        rl[e] = pl[0];
+                        rl[e + 1] = pl[1];
+                    }
                 }
                 bq[t][ks] = r;
+                if constexpr (SPLIT) *reinterpret_cast<v8*>(sLo + ((t * KS + ks) * 64 + lane) * 8) = rl;
             }
         }
+        // lo operand of tile t, k-step ks (the wave reads back what it wrote: program order is enough)
+        [[maybe_unused]] auto lo_of = [&](int t, int ks) {
+            return *reinterpret_cast<const v8*>(sLo + ((t * KS + ks) * 64 + lane) * 8);
+        };
 
         f32x16 acc[NT][DT];
         float mref[NT], lsum[NT];
@@ -359,8 +384,11 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
                         for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-                        for (int ks = 0; ks < KS; ++ks)
-                            s = M::mma(*reinterpret_cast<const v8*>(k1p + ks * 16), bq[t][ks], s);
+                        for (int ks = 0; ks < KS; ++ks) {
+                            const v8 kop = *reinterpret_cast<const v8*>(k1p + ks * 16);
+                            s = M::mma(kop, bq[t][ks], s);
+                            if constexpr (SPLIT) s = M::mma(kop, lo_of(t, ks), s);
+                        }
                         if constexpr (WIN) {
                             if (!inside) {
 #pragma unroll
@@ -507,9 +535,23 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                         pa[h][e + 1] = pr[1];
                     }
                 };
+                [[maybe_unused]] v8 lo[KS];
+                if constexpr (SPLIT) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) lo[ks] = lo_of(0, ks);
+                }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) s0 = M::mma(ka[ks], bq[0][ks], s0);
+                if constexpr (SPLIT) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) s0 = M::mma(ka[ks], lo[ks], s0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) lo[ks] = lo_of(1, ks);  // tile 1's, under the products above
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) s1 = M::mma(ka[ks], lo[ks], s1);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 // U^T operands are first needed two MFMA groups from here
 #pragma unroll
@@ -626,13 +668,17 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     load_k(0);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) sc[0] = M::mma(ka[ks], bq[0][ks], sc[0]);
+                    for (int ks = 0; ks < KS; ++ks) {
+                        sc[0] = M::mma(ka[ks], bq[0][ks], sc[0]);
+                        if constexpr (SPLIT) sc[0] = M::mma(ka[ks], lo_of(0, ks), sc[0]);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                     load_k(1);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks) {
                         sc[1] = M::mma(ka[ks], bq[0][ks], sc[1]);
+                        if constexpr (SPLIT) sc[1] = M::mma(ka[ks], lo_of(0, ks), sc[1]);
                         __builtin_amdgcn_sched_barrier(0);
                         if (ks == KS / 2 - 1) load_u(0, 0);
 #pragma unroll
@@ -766,7 +812,11 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const float o = (Orun[t][dt] + __shfl_xor(Orun[t][dt], 32, 64)) * inv;
-            if (q < T && g == 0) p.o[base + (size_t)q * D + dt * 32 + n] = (E)o;
+            if (q < T && g == 0) {
+                const E rounded = (E)o;
+                p.o[base + (size_t)q * D + dt * 32 + n] = rounded;
+                if constexpr (SPLIT) p.o_res[base + (size_t)q * D + dt * 32 + n] = (E)(o - (float)rounded);
+            }
         }
         if (q < T && lane == 0) p.lse[(size_t)bh * T + q] = (Mrun[t] + fast_log2(Lrun[t])) * kLn2;
     }
@@ -775,7 +825,8 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
 // Joins the parts a split forward left behind: one thread per (row, d).
 template <typename E>
 __global__ __launch_bounds__(256) void fwd_merge_kernel(const float* __restrict__ part, E* __restrict__ o,
-                                                        float* __restrict__ lse, int rows, int D, int splits) {
+                                                        E* __restrict__ o_res, float* __restrict__ lse, int rows,
+                                                        int D, int splits) {
     // 64-bit element index: rows * D can pass 2^31 (the forced-split override applies at any size)
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t row = idx / D;
@@ -792,7 +843,10 @@ __global__ __launch_bounds__(256) void fwd_merge_kernel(const float* __restrict_
         l += w * src[s * (D + 2) + D + 1];
         acc += w * src[s * (D + 2) + d];
     }
-    o[row * D + d] = (E)(acc / l);
+    const float out = acc / l;
+    const E rounded = (E)out;
+    o[row * D + d] = rounded;
+    if (o_res) o_res[row * D + d] = (E)(out - (float)rounded);  // split operands: see tdp_fwd_mfma_kernel
     if (d == 0) lse[row] = (m + fast_log2(l)) * kLn2;
 }
 
@@ -807,10 +861,11 @@ __global__ __launch_bounds__(256) void silu_transpose_kernel(const E* __restrict
     transpose_store<E>(ut + (size_t)bh * D * Tp, tile, j0, Tp, D);
 }
 
-template <int D, int NT, int WAVES, int JS>
+template <int D, int NT, int WAVES, int JS, bool SPLIT = false>
 constexpr size_t fwd_smem_bytes() {
     return sizeof(uint16_t) * (2 * JS * (D + 8) + 2 * D * (JS + 8) + 4 * 32 * (D + 8)) +
-           sizeof(float) * (WAVES * NT * (D + 4) + WAVES * 32) + 16;
+           sizeof(float) * (WAVES * NT * (D + 4) + WAVES * 32) + 16 +
+           (SPLIT ? sizeof(uint16_t) * WAVES * NT * (D / 16) * 512 : 0);
 }
 
 }  // namespace tritt
@@ -839,6 +894,7 @@ static size_t ut_bytes(int BH, int T, int D) {
 constexpr size_t kBandSmemLimit = 156 * 1024;
 static bool use_band_kernel(const MfmaFwdArgs& a) {
     if (!(a.windowed && a.causal)) return false;
+    if (a.split) return false;  // split operands: the streaming kernels only
     if (knobs().fwd_band < 0) return false;
     const int nr = band_rows(a.k1_window, a.k2_window);
     const size_t smem = a.D == 32 ? band_smem_bytes<32>(nr) : a.D == 64 ? band_smem_bytes<64>(nr) : band_smem_bytes<128>(nr);
@@ -852,7 +908,7 @@ static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
                        a.T, Tp, D);
     FwdParams<E> p;
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
-    p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse;
+    p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse; p.o_res = nullptr;
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + kBandQ - 1) / kBandQ;
     p.scale_log2 = a.alpha * kLog2e;
     p.causal = 1;
@@ -880,7 +936,7 @@ static int fwd_splits(const MfmaFwdArgs& a, int bq) {
     return max(1, min(kAutoFwdSplits, min(by_size, by_tiles)));
 }
 
-template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false>
+template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false, bool SPLIT = false>
 static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
@@ -890,21 +946,22 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     FwdParams<E> p;
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
     p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse;
+    p.o_res = SPLIT ? (E*)a.o + (size_t)a.BH * a.T * D : nullptr;
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + BQ - 1) / BQ;
     p.scale_log2 = a.alpha * kLog2e;
     p.causal = a.causal;
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
     p.splits = fwd_splits(a, BQ);
     p.part = reinterpret_cast<float*>(static_cast<char*>(a.ut) + ut_bytes(a.BH, a.T, D));
-    constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS>();
-    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG>;
+    constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS, SPLIT>();
+    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG, SPLIT>;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
     const int groups = (a.BH + 7) / 8;
     hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt * p.splits), dim3(64 * WAVES), smem, st, p);
     if (p.splits > 1) {
         const int rows = a.BH * a.T;
         hipLaunchKernelGGL(fwd_merge_kernel<E>, dim3((unsigned)(((size_t)rows * D + 255) / 256)), dim3(256), 0, st,
-                           p.part, (E*)a.o, a.lse, rows, D, p.splits);
+                           p.part, (E*)a.o, p.o_res, a.lse, rows, D, p.splits);
     }
     return hipGetLastError();
 }
@@ -916,11 +973,25 @@ size_t mfma_tdp_fwd_workspace(const MfmaFwdArgs& a) {
 }
 
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
+bool mfma_tdp_split_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64); }
 
 // D = 128: sequences up to this length run the diagonal stages in the interleaved loop (MDIAG)
 constexpr int kMaskedDiagonalUpTo = 768;
 
+template <typename E>
+static hipError_t launch_split(const MfmaFwdArgs& a, hipStream_t st) {
+    if (a.windowed) {
+        if (a.D == 32) return launch<E, 32, 1, 8, 2, 64, true, false, true>(a, st);
+        if (a.D == 64) return launch<E, 64, 2, 8, 2, 64, true, false, true>(a, st);
+    } else {
+        if (a.D == 32) return launch<E, 32, 1, 8, 2, 64, false, false, true>(a, st);
+        if (a.D == 64) return launch<E, 64, 2, 8, 2, 64, false, false, true>(a, st);
+    }
+    return hipErrorInvalidValue;
+}
+
 hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
+    if (a.split) return a.is_bf16 ? launch_split<__bf16>(a, st) : launch_split<_Float16>(a, st);
     if (use_band_kernel(a)) {
         if (a.is_bf16) {
             if (a.D == 32) return launch_band<__bf16, 32>(a, st);

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libtrittention_hip.so")
 CSRC_DIR = os.path.join(os.path.dirname(_HERE), "csrc")
 
 TRITT_F32, TRITT_BF16, TRITT_F16 = 0, 1, 2
-FLAG_AUTO, FLAG_FORCE_GENERIC, FLAG_FORCE_MFMA, FLAG_FLOAT_ATOMICS = 0, 1, 2, 4
+FLAG_AUTO, FLAG_FORCE_GENERIC, FLAG_FORCE_MFMA, FLAG_FLOAT_ATOMICS, FLAG_SPLIT_OPERANDS = 0, 1, 2, 4, 8
 
 _DTYPES = {torch.float32: TRITT_F32, torch.bfloat16: TRITT_BF16, torch.float16: TRITT_F16}
 

@@ -16,6 +16,14 @@ def _empty_like_bhtd(q):
     return torch.empty(q.shape, dtype=q.dtype, device=q.device)
 
 
+def _tdp_output(q, flags: int):
+    """What tritt_tdp_fwd writes through `o`: one [B,H,T,D] tensor, or under FLAG_SPLIT_OPERANDS two of them
+    stacked (the output and its rounding residual; the backward reads both)."""
+    if flags & _lib.FLAG_SPLIT_OPERANDS:
+        return torch.empty((2, *q.shape), dtype=q.dtype, device=q.device)
+    return _empty_like_bhtd(q)
+
+
 def tdp_fwd_impl(q, k1, k2, v1, v2, softmax_scale: float, causal: bool, k1_window: int, k2_window: int, kk_left: int,
                  kk_right: int, flags: int):
     _lib.require_gpu(q, "flash_trittention")
@@ -23,7 +31,7 @@ def tdp_fwd_impl(q, k1, k2, v1, v2, softmax_scale: float, causal: bool, k1_windo
     B, H, T, D = q.shape
     lib = _lib.lib()
     code = _lib.dtype_code(q.dtype)
-    o = _empty_like_bhtd(q)
+    o = _tdp_output(q, flags)
     lse = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
     with _lib.on_device(q.device):
         need = _lib.workspace_bytes("tritt_tdp_fwd_workspace_bytes", B, H, T, D, code, int(causal), k1_window, k2_window,
@@ -102,7 +110,7 @@ def tdp_fwd_op(q: _T, k1: _T, k2: _T, v1: _T, v2: _T, softmax_scale: float, caus
 
 @tdp_fwd_op.register_fake
 def _(q, k1, k2, v1, v2, softmax_scale, causal, k1_window, k2_window, kk_left, kk_right, flags):
-    return _empty_like_bhtd(q), q.new_empty(q.shape[:3], dtype=torch.float32)
+    return _tdp_output(q, flags), q.new_empty(q.shape[:3], dtype=torch.float32)
 
 
 @torch.library.custom_op("flash_trittention::tdp_bwd", mutates_args=())

@@ -56,13 +56,19 @@ class FlashTrittention(torch.autograd.Function):
         flags = _lib.FLAG_AUTO if compiling else getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
         if torch.are_deterministic_algorithms_enabled():
             flags &= ~_lib.FLAG_FLOAT_ATOMICS  # the default (fixed-point accumulation) is bitwise reproducible
-        if convert_to_float32 and not flags & _lib.FLAG_FORCE_MFMA:
-            # the reference forms its scores in fp32 under this flag (flash_trittention.py:408, bwd_dq.py:197); here
-            # 16-bit tensors then take the fp32 kernels: fp32 operands and products throughout, 16-bit results
-            flags |= _lib.FLAG_FORCE_GENERIC
+        if convert_to_float32 and not flags & (_lib.FLAG_FORCE_MFMA | _lib.FLAG_FORCE_GENERIC):
+            # the reference upcasts the operands of its score products under this flag (flash_trittention.py:408,
+            # bwd_dq.py:197,219).  16-bit tensors with D = 32 or 64 stay on the matrix cores with those operands
+            # kept to 16 mantissa bits (hi + lo pairs); other shapes take the fp32 kernels
+            if Q.dtype != torch.float32 and Q.shape[-1] in (32, 64):
+                flags |= _lib.FLAG_SPLIT_OPERANDS
+            else:
+                flags |= _lib.FLAG_FORCE_GENERIC
         call = torch.ops.flash_trittention.tdp_fwd if compiling else _ops.tdp_fwd_impl
         O, LSE = call(Q, K1, K2, V1, V2, float(softmax_scale), causal, k1_window, k2_window, kk_left, kk_right, flags)
-        ctx.save_for_backward(Q, K1, K2, V1, V2, O, LSE)
+        ctx.save_for_backward(Q, K1, K2, V1, V2, O, LSE)  # split operands: O is [2,B,H,T,D], output and residual
+        if flags & _lib.FLAG_SPLIT_OPERANDS:
+            O = O[0]
         ctx.softmax_scale = float(softmax_scale)
         ctx.windows = (k1_window, k2_window, kk_left, kk_right)
         ctx.causal = causal
@@ -96,9 +102,10 @@ def flash_trittention(q, k1, k2, v1, v2, softmax_scale=1 / 8, kk_left=1, kk_righ
 
     Window arguments: ``None`` (or any value >= seq_len) disables a window; note that the
     literal defaults are 1, a narrow band, exactly as in the reference.  Softmax and accumulation are
-    always fp32.  ``convert_to_float32=True`` also keeps the operands of the score products in fp32
-    (16-bit tensors then run the fp32 kernels: about ten times slower, but scores spanning hundreds
-    keep the full 16-bit tolerance, where the 16-bit operands of the default path do not).
+    always fp32.  ``convert_to_float32=True`` also keeps the operands of the score products beyond 16-bit
+    rounding: for 16-bit tensors with head_dim 32 or 64 as hi + lo pairs on the matrix cores (about 1.4 times
+    the default path's time), otherwise on the fp32 kernels.  Scores spanning hundreds then keep the full
+    16-bit tolerance, where the 16-bit operands of the default path do not.
     ``input_precision`` is accepted and ignored with a warning, as in the reference.
     """
     if input_precision is not None:

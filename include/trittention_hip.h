@@ -48,8 +48,19 @@ enum {
     TRITT_FLAG_AUTO = 0,
     TRITT_FLAG_FORCE_GENERIC = 1, /* use the fp32 VALU kernels even where an MFMA kernel exists */
     TRITT_FLAG_FORCE_MFMA = 2,    /* fail with TRITT_ERR_UNSUPPORTED instead of falling back    */
-    TRITT_FLAG_FLOAT_ATOMICS = 4  /* tritt_tdp_bwd, MFMA path: accumulate the shared gradients with fp32
+    TRITT_FLAG_FLOAT_ATOMICS = 4, /* tritt_tdp_bwd, MFMA path: accumulate the shared gradients with fp32
                                      atomics instead of 64-bit fixed point (see tritt_tdp_bwd)     */
+    TRITT_FLAG_SPLIT_OPERANDS = 8 /* tritt_tdp_fwd / tritt_tdp_bwd, 16-bit tensors, D = 32 or 64: what the
+                                     reference's convert_to_float32=True asks of its kernels
+                                     (triple_dot_product/flash_trittention.py:408, kernels/bwd_dq.py:197,219),
+                                     at matrix-core speed.  The operands Q (.) K2 and dO (.) V2 of the score
+                                     products are kept to 16 mantissa bits (a hi + lo pair of 16-bit numbers,
+                                     two MFMAs per k-step), so scores and dP carry fp32 accumulation error only.
+                                     `o` then points to TWO consecutive [B,H,T,D] tensors: the output, and the
+                                     rounding residual of every output element (fp32 value minus stored value;
+                                     written by tritt_tdp_fwd, read by tritt_tdp_bwd for Delta = rowsum(dO * O)).
+                                     Other configurations: TRITT_ERR_UNSUPPORTED (use TRITT_FLAG_FORCE_GENERIC,
+                                     the fp32 kernels, there).                                          */
 };
 
 /* Library version (major*10000 + minor*100 + patch) and a static, human

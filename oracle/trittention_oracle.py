@@ -90,6 +90,19 @@ def dps_mask(T: int, k_diff: int, q_lo: int = 0, q_hi: Optional[int] = None) -> 
     return (s > t) | (t > q) | (t - s > k_diff)
 
 
+def gated(v1, silu_dtype=None):
+    """U = SiLU(V1).  The naive modules apply SiLU in the precision they compute in (fp32 in every comparison
+    here).  The reference's kernel front-ends apply it in the TENSOR dtype before any kernel runs
+    (triple_dot_product/flash_trittention.py:62, dot_product_sum/trittention_triton.py:55), so with 16-bit tensors
+    their kernels see U rounded to 16 bit.  ``silu_dtype`` restates that rounding (straight-through for the
+    gradient, which the front-ends also take as dU * SiLU'(V1), flash_trittention.py:389-391): the comparison
+    target for tests that resolve differences below the 16-bit rounding of U itself."""
+    u = F.silu(v1)
+    if silu_dtype is not None:
+        u = u + (u.detach().to(silu_dtype).to(u.dtype) - u.detach())
+    return u
+
+
 def _softmax_pv(score, masked, alpha, u, v2):
     """score [..., q, j, k] (unscaled) -> (z [..., q, d], lse [..., q])."""
     if masked is not None:
@@ -103,7 +116,7 @@ def _softmax_pv(score, masked, alpha, u, v2):
 
 
 def tdp_forward_dense(q, k1, k2, v1, v2, alpha: float, causal: bool = True,
-                      k1_window=None, k2_window=None, kk_left=None, kk_right=None
+                      k1_window=None, k2_window=None, kk_left=None, kk_right=None, silu_dtype=None
                       ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Triple-dot-product forward, fully dense: returns (z, lse).
 
@@ -114,7 +127,7 @@ def tdp_forward_dense(q, k1, k2, v1, v2, alpha: float, causal: bool = True,
     T = q.shape[-2]
     score = torch.einsum("...qd,...jd,...kd->...qjk", q, k1, k2)
     masked = tdp_mask(T, k1_window, k2_window, kk_left, kk_right) if causal else None
-    return _softmax_pv(score, masked, alpha, F.silu(v1), v2)
+    return _softmax_pv(score, masked, alpha, gated(v1, silu_dtype), v2)
 
 
 def dps_forward_dense(q, k1, k2, v1, v2, alpha: float, causal: bool = True,

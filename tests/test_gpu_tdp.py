@@ -317,19 +317,31 @@ def test_mfma_forward_large_logits():
     assert (err > 5e-2).float().mean() < 0.01 and err.max() < 0.5, (err.max(), (err > 5e-2).float().mean())
 
 
+SPLIT = _lib.FLAG_SPLIT_OPERANDS
+
+
 @pytest.mark.parametrize("windows", [(None,) * 4, (64, 100, 20, 30)])
-def test_large_logits_with_convert_to_float32_hold_the_16_bit_bar(windows):
-    """convert_to_float32=True keeps the operands of the score products in fp32 (the fp32 kernels on the 16-bit
-    tensors): scores spanning hundreds, where the default path is held to a statistical bound, then meet the
-    ordinary 16-bit tolerance element by element, forward and all five gradients."""
+@pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (32, torch.bfloat16), (64, torch.float16), (128, torch.bfloat16)])
+def test_large_logits_with_convert_to_float32_hold_the_16_bit_bar(windows, D, dtype):
+    """convert_to_float32=True keeps the operands of the score products beyond 16-bit rounding, as the reference's
+    flag does (triple_dot_product/flash_trittention.py:408, kernels/bwd_dq.py:197,219): D = 32 / 64 as hi + lo
+    pairs on the 16-bit matrix-core kernels, D = 128 on the fp32 kernels.  Scores spanning hundreds, where the
+    default path is held to a statistical bound, then meet the ordinary 16-bit tolerance element by element,
+    forward and all five gradients.  The matrix-core kernels take SiLU(V1) rounded to the tensor dtype, as the
+    reference's kernels do (flash_trittention.py:62); with nearly one-hot softmax rows that rounding alone moves
+    dQ by several times the tolerance (every dP of a row shifts by 2^-9 |dP| independently, and K1 (.) K2 is 36
+    times larger here), so those cases are compared with the oracle on the same rounded SiLU(V1)."""
     from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
 
-    inputs = orc.make_inputs(1, 2, 160, 64, torch.bfloat16, seed=22)
-    inputs[1] = (inputs[1].float() * 6).bfloat16()
-    inputs[2] = (inputs[2].float() * 6).bfloat16()
-    z, _, grads = util.oracle_tdp(inputs, 1 / 8, True, windows)
+    print(f"case large logits, convert_to_float32: D={D} {dtype} {windows}", flush=True)
+    inputs = orc.make_inputs(1, 2, 160, D, dtype, seed=22)
+    scale = 6 if dtype == torch.bfloat16 else 4  # fp16: products of the scaled inputs stay inside half precision
+    inputs[1] = (inputs[1].float() * scale).to(dtype)
+    inputs[2] = (inputs[2].float() * scale).to(dtype)
+    alpha = 1 / math.sqrt(D)
+    z, _, grads = util.oracle_tdp(inputs, alpha, True, windows, silu_dtype=dtype if D != 128 else None)
     leaves = [t.cuda().requires_grad_(True) for t in inputs[:5]]
-    out = flash_trittention(*leaves, softmax_scale=1 / 8, k1_window=windows[0], k2_window=windows[1], kk_left=windows[2],
+    out = flash_trittention(*leaves, softmax_scale=alpha, k1_window=windows[0], k2_window=windows[1], kk_left=windows[2],
                             kk_right=windows[3], causal=True, convert_to_float32=True)
     out.backward(inputs[5].cuda())
     err = (out.detach().float().cpu() - z).abs()
@@ -337,6 +349,45 @@ def test_large_logits_with_convert_to_float32_hold_the_16_bit_bar(windows):
     util.assert_mostly_close("out", out.detach().float().cpu(), z, **LOWP)
     for name, leaf, want in zip(util.NAMES, leaves, grads):
         util.assert_mostly_close(name, leaf.grad.float().cpu(), want, **LOWP)
+
+
+@pytest.mark.parametrize("shape,windows", [((2, 4, 256, 64), (None,) * 4), ((1, 3, 203, 32), (None,) * 4),
+                                           ((1, 2, 449, 64), (100, 64, 33, 16)), ((2, 2, 130, 64), (3, 200, 0, 2)),
+                                           ((1, 5, 64, 32), (8, 8, 4, 4))])
+@pytest.mark.parametrize("causal", [True, False])
+def test_split_operands_through_the_c_abi(shape, windows, causal):
+    """TRITT_FLAG_SPLIT_OPERANDS on ordinary inputs: every result at the 16-bit bar against the oracle, the output
+    bitwise what the flag-less call stores where the two agree on the rounding (most elements), and the second
+    tensor behind `o` the rounding residual of the first."""
+    from flash_trittention import _ops
+
+    print(f"case split operands {shape} {windows} causal={causal}", flush=True)
+    B, H, T, D = shape
+    inputs = orc.make_inputs(B, H, T, D, torch.bfloat16, seed=T)
+    alpha = 1 / math.sqrt(D)
+    z, _, grads = util.oracle_tdp(inputs, alpha, causal, windows)
+    out, g = util.run_tdp(inputs, alpha, causal, windows, flags=SPLIT)
+    util.assert_mostly_close("out", out, z, **LOWP)
+    for name, a, b in zip(util.NAMES, g, grads):
+        util.assert_mostly_close(name, a, b, **LOWP)
+    dev = [t.cuda() for t in inputs[:5]]
+    w = [T if x is None else x for x in windows]
+    o2, lse = _ops.tdp_fwd_impl(*dev, alpha, causal, *w, SPLIT)
+    assert o2.shape == (2, B, H, T, D)
+    # the residual is what rounding to 16 bit removed: below half an ulp of the stored value, and adding it back
+    # moves the result towards the fp32 oracle on average
+    assert (o2[1].float().abs() <= o2[0].float().abs() * 2.0 ** -8 + 1e-30).all()
+    full = (o2[0].float() + o2[1].float()).cpu()
+    assert (full - z).abs().mean() < (o2[0].float().cpu() - z).abs().mean()
+
+
+def test_split_operands_refused_where_unsupported():
+    inputs = orc.make_inputs(1, 1, 64, 128, torch.bfloat16, seed=1)
+    with pytest.raises(RuntimeError, match="does not support"):
+        util.run_tdp(inputs, 0.1, True, backward=False, flags=SPLIT)
+    inputs = orc.make_inputs(1, 1, 64, 64, torch.float32, seed=1)
+    with pytest.raises(RuntimeError, match="does not support"):
+        util.run_tdp(inputs, 0.1, True, backward=False, flags=SPLIT)
 
 
 def test_mfma_forward_large_values_and_logits():

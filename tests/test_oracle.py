@@ -218,3 +218,23 @@ def test_make_inputs_is_seeded_and_ordered():
     assert len(a) == 6 and all(torch.equal(x, y) for x, y in zip(a, b))
     g = torch.Generator().manual_seed(3)
     assert torch.equal(a[0], torch.randn(1, 2, 4, 8, generator=g))
+
+
+def test_rounded_silu_is_the_dense_formula_on_rounded_gated_values():
+    """`silu_dtype` only replaces U = SiLU(V1) by its rounding (the forward equals the softmax-weighted sum with
+    that U passed in directly) and leaves the gradient path through SiLU'(V1) in place (straight-through: dV1 =
+    dU * SiLU'(V1) with dU taken at the rounded U)."""
+    q, k1, k2, v1, v2, do = (t[0, 0] for t in orc.make_inputs(1, 1, 20, 8, torch.float32, seed=3))
+    z, lse = orc.tdp_forward_dense(q, k1, k2, v1, v2, 0.3, True, silu_dtype=torch.bfloat16)
+    u = torch.nn.functional.silu(v1).bfloat16().float()
+    assert not torch.equal(u, torch.nn.functional.silu(v1))
+    score = torch.einsum("qd,jd,kd->qjk", q, k1, k2)
+    z2, lse2 = orc._softmax_pv(score, orc.tdp_mask(20), 0.3, u, v2)
+    assert torch.equal(z, z2) and torch.equal(lse, lse2)
+    # gradient: dV1 = dU * SiLU'(V1), dU from the formula evaluated at the rounded U
+    _, _, g = orc.tdp_forward_backward(q, k1, k2, v1, v2, do, 0.3, True, silu_dtype=torch.bfloat16)
+    ul = u.clone().requires_grad_(True)
+    z3, _ = orc._softmax_pv(score, orc.tdp_mask(20), 0.3, ul, v2)
+    z3.backward(do)
+    sg = torch.sigmoid(v1)
+    torch.testing.assert_close(g[3], ul.grad * sg * (1 + v1 * (1 - sg)), rtol=1e-6, atol=1e-7)

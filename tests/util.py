@@ -7,11 +7,14 @@ from oracle import trittention_oracle as orc
 NAMES = ("dq", "dk1", "dk2", "dv1", "dv2")
 
 
-def oracle_tdp(inputs, alpha, causal, windows=(None,) * 4, per_head=True):
+def oracle_tdp(inputs, alpha, causal, windows=(None,) * 4, per_head=True, silu_dtype=None):
     """Oracle in fp32 on the already-rounded inputs (what the reference's tests do:
-    tests/test_triple_dot_product.py:47).  Evaluated head by head to bound memory."""
+    tests/test_triple_dot_product.py:47).  Evaluated head by head to bound memory.  `silu_dtype`: SiLU(V1)
+    rounded to that dtype first, as the reference's kernel front-end does (oracle.gated)."""
     q, k1, k2, v1, v2, do = (t.float() for t in inputs)
     kw = dict(zip(("k1_window", "k2_window", "kk_left", "kk_right"), windows))
+    if silu_dtype is not None:
+        kw["silu_dtype"] = silu_dtype
     B, H, T, D = q.shape
     z = torch.empty_like(q)
     lse = torch.empty(B, H, T)
