@@ -285,6 +285,10 @@ int tdp_bwd_generic(Arena& ar, bool run, const void* q, const void* k1, const vo
 }
 
 // ---------------------------------------------------------------- dot-product-sum
+// fp32 path: the attention kernels on the fp32 matrix cores where they exist (D = 32, 64), else one lane per row on
+// the vector ALUs; TRITT_TUNE_F32_VALU forces the latter
+bool use_f32_mfma_dps(int D) { return !knobs().f32_valu && f32_mfma_dps_supported(D); }
+
 int dps_fwd_impl(Arena& ar, bool run, const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
                  void* o, float* lse, int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
                  hipStream_t st) {
@@ -301,7 +305,7 @@ int dps_fwd_impl(Arena& ar, bool run, const void* q, const void* k1, const void*
     a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
     a.o = o32; a.lse = lse;
     a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal; a.k_diff = k_diff;
-    hipError_t e = dps_fwd(a, st);
+    hipError_t e = use_f32_mfma_dps(D) ? f32_mfma_dps_fwd(a, st) : dps_fwd(a, st);
     if (e != hipSuccess) return (int)e;
     if (dtype != TRITT_F32) from_f32(o32, nullptr, o, n, dtype, st);
     return (int)hipGetLastError();
@@ -325,15 +329,28 @@ int dps_bwd_impl(Arena& ar, bool run, const void* q, const void* k1, const void*
     if (dtype != TRITT_F32) {
         dq32 = ar.take<float>(n); dk132 = ar.take<float>(n); dk232 = ar.take<float>(n); dv232 = ar.take<float>(n);
     }
+    // 16-bit tensors on the fp32 path: the output and the log-sum-exp are formed once more in fp32, as the triple-dot
+    // path does: Delta = rowsum(dO * O) from the stored 16-bit output carries that output's rounding, which nearly
+    // one-hot softmax rows (large scores) turn into gradient errors far above it
+    float* o32 = dtype != TRITT_F32 ? ar.take<float>(n) : nullptr;
+    float* lse32 = dtype != TRITT_F32 ? ar.take<float>(rows) : nullptr;
     if (!run) return TRITT_OK;
     fill_inputs(q, k1, k2, v1, v2, n, dtype, copies, u, st);
     if (dtype != TRITT_F32) to_f32<false>(d_o, do32, n, dtype, st);
-    rowdot(d_o, o, a.delta, (int)rows, D, dtype, st);
     a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
+    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal; a.k_diff = k_diff;
+    if (o32) {
+        a.o = o32; a.lse = lse32;
+        hipError_t ef = use_f32_mfma_dps(D) ? f32_mfma_dps_fwd(a, st) : dps_fwd(a, st);
+        if (ef != hipSuccess) return (int)ef;
+        rowdot(do32, o32, a.delta, (int)rows, D, TRITT_F32, st);
+        lse = lse32;
+    } else {
+        rowdot(d_o, o, a.delta, (int)rows, D, dtype, st);
+    }
     a.lse = const_cast<float*>(lse); a.d_o = do32;
     a.dq = dq32; a.dk1 = dk132; a.dk2 = dk232; a.du = du; a.dv2 = dv232;
-    a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal; a.k_diff = k_diff;
-    hipError_t e = dps_bwd(a, st);
+    hipError_t e = use_f32_mfma_dps(D) ? f32_mfma_dps_bwd(a, st) : dps_bwd(a, st);
     if (e != hipSuccess) return (int)e;
     from_f32(du, v1, dv1, n, dtype, st);
     if (dtype != TRITT_F32) {

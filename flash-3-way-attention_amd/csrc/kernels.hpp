@@ -87,6 +87,10 @@ struct DpsArgs {
 };
 hipError_t dps_fwd(const DpsArgs& a, hipStream_t st);
 hipError_t dps_bwd(const DpsArgs& a, hipStream_t st);
+// the same two calls with the attention kernels on the fp32 matrix cores (D = 32 or 64)
+bool f32_mfma_dps_supported(int D);
+hipError_t f32_mfma_dps_fwd(const DpsArgs& a, hipStream_t st);
+hipError_t f32_mfma_dps_bwd(const DpsArgs& a, hipStream_t st);
 
 // 16-bit MFMA triple-dot forward (any mask; D = 32, 64 or 128).
 struct MfmaFwdArgs {

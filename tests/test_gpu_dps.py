@@ -318,3 +318,42 @@ def test_forward_and_backward_replay_from_a_hip_graph(shape):
             assert torch.equal(a, b), rep
         z, lse, _ = util.oracle_dps(fresh, 1 / math.sqrt(D), True, k_diff, factorised=True)
         util.assert_close("out vs oracle", got[0].float().cpu(), z, **LOWP)
+
+
+@pytest.mark.parametrize("D", [32, 64])
+@pytest.mark.parametrize("causal,k_diff", [(True, 250), (True, 37), (True, 0), (False, 250)])
+def test_fp32_tensors_on_the_matrix_cores(D, causal, k_diff, tune):
+    """fp32 tensors run the three attention kernels on the fp32 MFMA (ragged length, two owner tiles per head and
+    more): forward, m and all five gradients at the fp32 bar against the oracle, and against the fp32 VALU
+    kernels of the same library (what the reference's fp32 test grid covers: tests/test_dot_product_sum.py:70-118)."""
+    from flash_trittention import _lib
+
+    print(f"case dps fp32 mfma D={D} causal={causal} k_diff={k_diff}", flush=True)
+    inputs = orc.make_inputs(2, 3, 250, D, torch.float32, seed=D + k_diff)
+    alpha = 1 / math.sqrt(D)
+    check_all(inputs, alpha, causal, k_diff, factorised=False)
+    out, m, g = util.run_dps(inputs, alpha, causal, k_diff)
+    tune(_lib.TUNE_F32_VALU, 1)
+    out_v, m_v, g_v = util.run_dps(inputs, alpha, causal, k_diff)
+    assert not torch.equal(out, out_v), "both runs took the same kernels"
+    util.assert_close("out vs VALU kernels", out, out_v, **FP32)
+    util.assert_close("m vs VALU kernels", m, m_v, rtol=1e-5, atol=1e-4)
+    for name, a, b in zip(util.NAMES, g, g_v):
+        util.assert_close(f"{name} vs VALU kernels", a, b, **FP32)
+
+
+def test_large_logits_with_convert_to_float32_hold_the_16_bit_bar():
+    """convert_to_float32=True on 16-bit tensors: fp32 operands throughout (the fp32 matrix-core kernels), as the
+    reference's flag asks of its kernels (dot_product_sum/trittention_triton.py:92-119).  Logits of a few hundred,
+    where the 16-bit MFMA path is held to a statistical bound, meet the 16-bit tolerance element by element."""
+    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
+
+    inputs = [t * (6.0 if i < 3 else 1.0) for i, t in enumerate(orc.make_inputs(1, 2, 128, 64, torch.bfloat16, seed=33))]
+    z, lse, grads = util.oracle_dps(inputs, 1 / 8, True, 128)
+    leaves = [t.cuda().requires_grad_(True) for t in inputs[:5]]
+    out, m = TrittentionTriton(causal=True, softmax_scale=1 / 8, k_diff=128, convert_to_float32=True)(*leaves)
+    out.backward(inputs[5].cuda())
+    util.assert_mostly_close("out", out.detach().float().cpu(), z, **LOWP)
+    util.assert_close("m", m.cpu(), lse, rtol=1e-4, atol=1e-3)
+    for name, leaf, want in zip(util.NAMES, leaves, grads):
+        util.assert_mostly_close(name, leaf.grad.float().cpu(), want, **LOWP)
