@@ -372,7 +372,10 @@ __device__ __forceinline__ float half_sum(float v) {  // over the 32 lanes of a 
 template <typename E, int D, int DOUT, bool WITH_DQ>
 __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_round) {
     constexpr int DTO = DOUT / 32, KS = D / 2, LD = D + 1, NW = kF32Waves;
-    constexpr bool FLY = D > 64;  // form the B operands of the score products as they are used
+    // form the B operands of the score products as they are used (two LDS reads and a multiply per MFMA) instead of
+    // holding D / 2 of each in registers where the accumulators leave no room for them: both at D = 128, those of
+    // dP alone at D = 64 in the launch that also carries the dQ accumulators
+    constexpr bool FLY = D > 64, FLY_G = FLY || (D == 64 && WITH_DQ);
     extern __shared__ __align__(16) float smem_f[];
     float* sK = smem_f;                 // [2][32][LD]
     float* sV = sK + 2 * 32 * LD;       // [2][32][LD]
@@ -464,13 +467,11 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
         }
         __syncthreads();
 
-        float bq[FLY ? 1 : KS], bg[FLY ? 1 : KS];
-        if constexpr (!FLY) {
+        float bq[FLY ? 1 : KS], bg[FLY_G ? 1 : KS];
 #pragma unroll
-            for (int s = 0; s < KS; ++s) {
-                bq[s] = sQ[n * LD + g * KS + s] * sKb[wave * D + g * KS + s];
-                bg[s] = sDO[n * LD + g * KS + s] * sVb[wave * D + g * KS + s];
-            }
+        for (int s = 0; s < KS; ++s) {
+            if constexpr (!FLY) bq[s] = sQ[n * LD + g * KS + s] * sKb[wave * D + g * KS + s];
+            if constexpr (!FLY_G) bg[s] = sDO[n * LD + g * KS + s] * sVb[wave * D + g * KS + s];
         }
         f32x16 accQ[DTO], accT[DTO];
 #pragma unroll
@@ -495,13 +496,21 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
                     s[i] = 0.f;
                     dp[i] = 0.f;
                 }
+                // The per-lane parts of the LDS addresses, opaque to the compiler from here on: every read below is
+                // then this base plus a compile-time offset (the instruction's immediate field).  Left to itself the
+                // compiler computes the hundreds of addresses of the unrolled loops ahead of the loops and keeps them
+                // in registers (D = 128: 150 of them spilled to scratch memory).
+                int row_base = n * LD + g * KS, own_base = wave * D + g * KS, out_base = 4 * g * LD + c0 + n;
+                asm volatile("" : "+v"(row_base), "+v"(out_base), "+v"(own_base));
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    const int col = g * KS + ks;
-                    const float oq = FLY ? sQ[n * LD + col] * sKb[wave * D + col] : bq[FLY ? 0 : ks];
-                    const float og = FLY ? sDO[n * LD + col] * sVb[wave * D + col] : bg[FLY ? 0 : ks];
-                    s = mma_f32(cK[n * LD + col], oq, s);
-                    dp = mma_f32(cV[n * LD + col], og, dp);
+                    const float oq = FLY ? sQ[row_base + ks] * sKb[own_base + ks] : bq[FLY ? 0 : ks];
+                    const float og = FLY_G ? sDO[row_base + ks] * sVb[own_base + ks] : bg[FLY_G ? 0 : ks];
+                    s = mma_f32(cK[row_base + ks], oq, s);
+                    dp = mma_f32(cV[row_base + ks], og, dp);
+                    // keep the operand reads of later k-steps from being hoisted over these (they would have to be
+                    // held in registers the accumulators need)
+                    if (FLY_G && (ks & 7) == 7) __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -515,8 +524,10 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
                 for (int dt = 0; dt < DTO; ++dt)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
-                        accT[dt] = mma_f32(cV[c_row(g, i) * LD + c0 + dt * 32 + n], s[i], accT[dt]);
-                        accQ[dt] = mma_f32(cK[c_row(g, i) * LD + c0 + dt * 32 + n], dp[i], accQ[dt]);
+                        // row c_row(g, i) = c_row(0, i) + 4 g
+                        accT[dt] = mma_f32(cV[out_base + c_row(0, i) * LD + dt * 32], s[i], accT[dt]);
+                        accQ[dt] = mma_f32(cK[out_base + c_row(0, i) * LD + dt * 32], dp[i], accQ[dt]);
+                        if (FLY_G && (i & 3) == 3) __builtin_amdgcn_sched_barrier(0);
                     }
             }
             if (more) {
@@ -525,15 +536,17 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
             }
         }
         if (row_ok) {
+            int q_base = n * LD + c0 + 4 * g, kb_base = wave * D + c0 + 4 * g;  // opaque bases, as in the loop above
+            asm volatile("" : "+v"(q_base), "+v"(kb_base));
 #pragma unroll
             for (int dt = 0; dt < DTO; ++dt)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int d = c0 + dt * 32 + c_row(g, i);
-                    if constexpr (WITH_DQ) accDQ[dt][i] += accQ[dt][i] * sKb[wave * D + d];
+                    const int d = c0 + dt * 32 + c_row(g, i), dc = dt * 32 + c_row(0, i);
+                    if constexpr (WITH_DQ) accDQ[dt][i] += accQ[dt][i] * sKb[kb_base + dc];
                     // sQ holds Q * alpha * log2(e): alpha is wanted, log2(e) is not
-                    const float rk = half_sum(accQ[dt][i] * sQ[n * LD + d]) * kLn2;
-                    const float rv = half_sum(accT[dt][i] * sDO[n * LD + d]);
+                    const float rk = half_sum(accQ[dt][i] * sQ[q_base + dc]) * kLn2;
+                    const float rv = half_sum(accT[dt][i] * sDO[q_base + dc]);
                     if (n == 0) {
                         const size_t idx = base + (size_t)b * D + d;
                         unsigned* prow = p.poison + (size_t)bh * T + b;
@@ -628,26 +641,28 @@ template <typename E, int D>
 hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, const E* k2, const E* v2, void* acc_k2,
                                 void* acc_v2, void* acc_k1, void* acc_u, const TdpMask& natural, bool want_q,
                                 bool want_k2, bool want_k1, hipStream_t st) {
-    constexpr int DOUT = D > 64 ? 64 : D;
+    // D = 128: the launch that also accumulates dQ produces 64 gradient columns per workgroup (both column halves
+    // form S and dP); without the dQ accumulators a workgroup holds all 128 columns and forms them once
+    constexpr int DOUT = D > 64 ? 64 : D, DOUT_NODQ = D;
     auto kern_dq = tdp_f32_bwd_kernel<E, D, DOUT, true>;
-    auto kern_nodq = tdp_f32_bwd_kernel<E, D, DOUT, false>;
+    auto kern_nodq = tdp_f32_bwd_kernel<E, D, DOUT_NODQ, false>;
     constexpr size_t smem = f32_bwd_smem<D>();
     static_assert(DOUT * 33 <= 4 * 32 * (D + 1), "dQ of the tile aliases the stage buffers");
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
     const int groups = (p.BH + 7) / 8;
-    const dim3 grid(8 * groups * p.nqt, D / DOUT);
+    const dim3 grid(8 * groups * p.nqt, D / DOUT), grid_nodq(8 * groups * p.nqt, D / DOUT_NODQ);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.ka = k1; p.va = u; p.kb = k2; p.vb = v2;
     p.acc_k = acc_k2; p.acc_v = acc_v2; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
     p.mask = natural;
     if (want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(512), smem, st, p);
-    else if (want_k2) hipLaunchKernelGGL(kern_nodq, grid, dim3(512), smem, st, p);
+    else if (want_k2) hipLaunchKernelGGL(kern_nodq, grid_nodq, dim3(512), smem, st, p);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU (the mask with the two key indices exchanged)
     p.ka = k2; p.va = v2; p.kb = k1; p.vb = u;
     p.acc_k = acc_k1; p.acc_v = acc_u; p.bit_k = kPoisonDK1; p.bit_v = kPoisonDU;
     p.mask = TdpMask{natural.causal, natural.wb, natural.wa, natural.rab, natural.lab};
-    if (want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(512), smem, st, p);
+    if (want_k1) hipLaunchKernelGGL(kern_nodq, grid_nodq, dim3(512), smem, st, p);
     return hipGetLastError();
 }
 

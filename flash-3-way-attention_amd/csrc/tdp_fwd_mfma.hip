@@ -273,6 +273,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     const int krow_off = key_of_row(n);  // K1 row (within a 32-key step) this lane feeds to the MFMA
 
     int gstage = 0;  // running stage counter (buffer = gstage & 1)
+    [[maybe_unused]] bool plain = true;  // every k-tile so far was merged with reference 0 (see the merge below)
     for (int kt = kt_lo; kt < nkt; ++kt) {
         const int kb = (kt - kt_lo) & 1;
         const int st_lo = first_stage(kt), st_hi = last_stage(kt);
@@ -713,6 +714,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
         };
 
         sweep(std::false_type{});
+        bool redone = false;
         {
             // did any valid virtual row of this workgroup leave the safe range?
             bool bad = false;
@@ -745,10 +747,46 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
                     }
                 }
                 sweep(std::true_type{});
+                redone = true;
             }
         }
 
         // ---- merge the 32 virtual rows (q, k) of each tile into the running O[q] -------------
+        // The common case first: this k-tile and every one before it kept the reference at 0 (FAST sweeps), so
+        // every weight is 1 and nothing is rescaled: O += sum_k V2[k] (.) Tv[(q, k)], L += sum_k l_k over the
+        // valid rows.  Only the diagonal k-tile holds rows past the causal bound; it clears them first.
+        if constexpr (!WIN) {
+            plain = plain && !redone;
+            if (plain) {
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const float lk = lsum[t] + __shfl_xor(lsum[t], 32, 64);
+                    const bool kval = (kt * 32 + n) <= jmax[t];
+                    float wl = kval ? lk : 0.f;
+#pragma unroll
+                    for (int off = 16; off > 0; off >>= 1) wl += __shfl_xor(wl, off, 64);
+                    Lrun[t] += wl;
+                    Mrun[t] = 0.f;
+                    if (!__all(kval)) {
+                        float wr[16];
+                        rows_of(kval ? 1.f : 0.f, wr);
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) acc[t][dt][i] = wr[i] == 0.f ? 0.f : acc[t][dt][i];
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        float part = 0.f;
+#pragma unroll
+                        for (int i = 0; i < 16; ++i)
+                            part += (float)sV2[(kb * 32 + c_row(g, i)) * LDK + dt * 32 + n] * acc[t][dt][i];
+                        Orun[t][dt] += part;
+                    }
+                }
+                continue;
+            }
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const float lk = lsum[t] + __shfl_xor(lsum[t], 32, 64);
