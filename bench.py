@@ -268,10 +268,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--brief", action="store_true", help="default mode: skip the other BASELINE configurations")
-    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "dps", "tdp", "published"], default="both",
+    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "seqlen", "dps", "tdp", "published"], default="both",
                     help="fwd: time only the forward (for profiling runs); copy: a plain 256 MiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against; "
                          "sweep: triple-dot forward at B=1 H=16 D=128 bf16 over T in 512..4096; "
+                         "seqlen: the reference's windowed sequence-length sweep (scripts/benchmark_seq_len_range.py:"
+                         "11-31,177: B=2 H=2 D=64, k1_window 24, k2_window 22, T = 256..2048 step 256, forward and "
+                         "backward, convert_to_float32=True), fp32 tensors as there and bf16; "
                          "dps: dot-product-sum forward+backward at --B --H --T --D; "
                          "tdp: triple-dot forward+backward at --B --H --T --D with --windows (secondary shapes: "
                          "D=128, windowed masks); "
@@ -310,6 +313,34 @@ def main():
         rows = sweep_rows(torch, flash_trittention, dev, args.steps)
         print(json.dumps({"metric": "triple-dot trittention fwd TFLOP/s vs T", "unit": "TFLOP/s",
                           "config": {"workload": "triple-dot fwd B=1 H=16 D=128 bf16 causal"}, "rows": rows}), flush=True)
+        return
+    if args.mode == "seqlen":
+        rows = []
+        for dtype in (torch.float32, torch.bfloat16):
+            for Ts in range(256, 2049, 256):
+                q, k1, k2, v1, v2, do = (t.to(dev) for t in make_inputs(2, 2, Ts, 64, dtype, seed=42))
+                leaves = [t.clone().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+                kw = dict(softmax_scale=1 / 8, k1_window=24, k2_window=22, kk_left=None, kk_right=None, causal=True,
+                          convert_to_float32=True)
+                hold = {}
+
+                def f():
+                    with torch.no_grad():
+                        return flash_trittention(q, k1, k2, v1, v2, **kw)
+
+                def b():
+                    hold["o"].backward(do, retain_graph=True)
+
+                ms_f = time_events(f, 20, 5, torch)
+                hold["o"] = flash_trittention(*leaves, **kw)
+                ms_b = time_events(b, 20, 5, torch)
+                nt = 4 * windowed_triples(Ts, 24, 22, Ts, Ts)
+                rows.append({"dtype": str(dtype).split(".")[-1], "T": Ts, "fwd_ms": ms_f, "bwd_ms": ms_b,
+                             "valid_triples": nt, "fwd_tflops": 4 * 64 * nt / ms_f / 1e9,
+                             "bwd_tflops": 12 * 64 * nt / ms_b / 1e9})
+        print(json.dumps({"metric": "triple-dot trittention fwd / bwd ms over T, windowed", "unit": "ms",
+                          "config": {"workload": "triple-dot fwd+bwd B=2 H=2 D=64 causal, k1_window=24 k2_window=22, "
+                                                 "convert_to_float32=True, T=256..2048"}, "rows": rows}), flush=True)
         return
     if args.mode == "published":
         # the reference's own forward table (h100/README.md:50-53, b200/README.md:53-56): milliseconds of its
