@@ -729,7 +729,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     // then all query tiles take the fp32 kernel (the work of such masks is small: T times the pair count).
     const bool first_in_f32 = a.causal != 0;
     const long long pairs = (long long)(a.k2_window + 1) * std::min(a.k1_window + 1, a.kk_left + a.kk_right + 1);
-    const bool all_in_f32 = first_in_f32 && a.windowed && pairs <= 1024;
+    const bool all_in_f32 = first_in_f32 && a.windowed && pairs <= 1024 && !a.split;
     if (first_in_f32) {
         FirstTileArgs f{};
         f.q = a.q; f.d_o = a.d_o; f.k1 = a.k1; f.u = u; f.k2 = a.k2; f.v2 = a.v2;
@@ -742,6 +742,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         f.k1_window = a.k1_window; f.k2_window = a.k2_window; f.kk_left = a.kk_left; f.kk_right = a.kk_right;
         f.want_q = want_q; f.want_k2 = want_k2; f.want_k1 = want_k1;
         f.tiles = all_in_f32 ? p.nqt : 1;
+        f.round_parts = (dqacc || !want_q) ? std::min(splits, f32_round_parts(a.BH, a.T)) : 1;
         if (hipError_t e = f32_mfma_tdp_bwd_first_tile(f, st); e != hipSuccess) return e;
     }
     const int tiles_here = all_in_f32 ? 0 : p.nqt - (first_in_f32 ? 1 : 0);

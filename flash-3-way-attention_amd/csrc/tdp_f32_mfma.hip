@@ -352,6 +352,9 @@ struct F32BwdParams {
     // when non-null, LSE and Delta of query tile 0 come from the partials the split STATS launch left here
     const float* stats_part;
     int split_rounds;      // tile 0 only: rounds dealt out to workgroups (see tdp_f32_tile0_kernel), else 0
+    // tdp_f32_bwd_kernel: workgroups per query tile (blockIdx.z); workgroup z walks rounds m_lo + z, m_lo + z + parts, ...
+    // More than one needs acc_q where dQ is produced (each workgroup holds a share of it)
+    int round_parts;
     // fixed-point accumulators (common.hpp); scale_parts null: the accumulators are float
     const unsigned* scale_parts;
     unsigned* poison;
@@ -368,9 +371,9 @@ __device__ __forceinline__ float half_sum(float v) {  // over the 32 lanes of a 
     return v;
 }
 
-// `only_round` >= 0: this workgroup walks that round of rows only
+// `only_round` >= 0: this workgroup walks that round of rows only; else every `parts`-th round from the `part`-th on
 template <typename E, int D, int DOUT, bool WITH_DQ>
-__device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_round) {
+__device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_round, int part = 0, int parts = 1) {
     constexpr int DTO = DOUT / 32, KS = D / 2, LD = D + 1, NW = kF32Waves;
     // form the B operands of the score products as they are used (two LDS reads and a multiply per MFMA) instead of
     // holding D / 2 of each in registers where the accumulators leave no room for them: both at D = 128, those of
@@ -406,6 +409,13 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
 
     const int q0 = qt * 32, q1 = min(T - 1, q0 + 31);
     const int q = q0 + n;
+    const Range rows = row_range(mask, q0, q1, T);
+    int m_lo = rows.lo / NW + part, m_hi = rows.hi / NW;
+    if (only_round >= 0) {
+        m_lo = max(m_lo, only_round);
+        m_hi = min(m_hi, only_round);
+    }
+    if (parts > 1 && m_lo > m_hi) return;  // fewer rounds than workgroups: nothing to add (uniform, before any barrier)
     for (int idx = tid; idx < 32 * D; idx += 512) {
         const int r = idx / D, d = idx % D;
         const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
@@ -432,13 +442,6 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
         }
     }
 
-    const Range rows = row_range(mask, q0, q1, T);
-    int m_lo = rows.lo / NW, m_hi = rows.hi / NW;
-    if (only_round >= 0) {
-        m_lo = max(m_lo, only_round);
-        m_hi = min(m_hi, only_round);
-    }
-
     f32x16 accDQ[DTO];
 #pragma unroll
     for (int dt = 0; dt < DTO; ++dt)
@@ -446,7 +449,7 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
         for (int i = 0; i < 16; ++i) accDQ[dt][i] = 0.f;
 
     StageE<E, D> regs;
-    for (int m = m_lo; m <= m_hi; ++m) {
+    for (int m = m_lo; m <= m_hi; m += parts) {
         const int b = m * NW + wave;
         const Range ra = streamed_range(mask, q0, q1, min(m * NW, T - 1), T);
         const Range rb = streamed_range(mask, q0, q1, min(m * NW + NW - 1, T - 1), T);
@@ -586,7 +589,7 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
 
 template <typename E, int D, int DOUT, bool WITH_DQ>
 __global__ __launch_bounds__(512) void tdp_f32_bwd_kernel(F32BwdParams<E> p) {
-    f32_bwd_body<E, D, DOUT, WITH_DQ>(p, -1);
+    f32_bwd_body<E, D, DOUT, WITH_DQ>(p, -1, blockIdx.z, gridDim.z);
 }
 
 // Query tile 0 of a 16-bit backward, both launches' roles and all rounds at once: blockIdx.z = role * rounds + round
@@ -615,6 +618,16 @@ __global__ __launch_bounds__(256) void f32_scale_kernel(const float* __restrict_
     const size_t lo = min(pieces, blockIdx.x * per_part), hi = min(pieces, lo + per_part);
     const unsigned m = block_absmax_bits<float>(d_o + blockIdx.y * per_slice + lo * 4, hi - lo, red);
     if (threadIdx.x == 0) parts[blockIdx.y * kScaleParts + blockIdx.x] = m;
+}
+// fixed point -> fp32, one tensor (dQ / alpha accumulated over the workgroups of a tile)
+__global__ __launch_bounds__(256) void f32_finish_q_kernel(const long long* __restrict__ acc, float* __restrict__ dq, size_t n,
+                                                           int T, int D, const unsigned* __restrict__ scale_parts,
+                                                           const unsigned* __restrict__ poison, float alpha) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const size_t row = i / D;
+        const double inv = fixed_scale_inverse(fixed_scale_field<false>(scale_parts, (int)(row / T), kF32FixedBias));
+        dq[i] = (poison[row] & kPoisonDQ) ? __builtin_nanf("") : (float)((double)acc[i] * inv) * alpha;
+    }
 }
 // fixed point -> fp32
 __global__ __launch_bounds__(256) void f32_finish_kernel(const long long* __restrict__ acc, float* __restrict__ dk_rows,
@@ -651,7 +664,9 @@ hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, cons
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
     const int groups = (p.BH + 7) / 8;
-    const dim3 grid(8 * groups * p.nqt, D / DOUT), grid_nodq(8 * groups * p.nqt, D / DOUT_NODQ);
+    // small grids: the rounds of a tile dealt out to several workgroups (the launch with dQ only when dQ has an accumulator)
+    const int parts = std::max(1, p.round_parts);
+    const dim3 grid(8 * groups * p.nqt, D / DOUT, p.acc_q ? parts : 1), grid_nodq(8 * groups * p.nqt, D / DOUT_NODQ, parts);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.ka = k1; p.va = u; p.kb = k2; p.vb = v2;
     p.acc_k = acc_k2; p.acc_v = acc_v2; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
@@ -672,10 +687,14 @@ hipError_t launch_f32_bwd(const GenericTdpArgs& a, long long* acc, hipStream_t s
     const bool want_q = a.dq != nullptr, want_k2 = a.dk2 && a.dv2, want_k1 = a.dk1 && a.du;
     F32BwdParams<float> p{};
     p.q = a.q; p.d_o = a.d_o; p.lse = a.lse_in; p.delta = a.delta;
-    p.dq = a.dq; p.acc_q = nullptr; p.acc_q_rows = 0; p.stats_part = nullptr; p.split_rounds = 0;
-    // scratch: four accumulators, the rows' poison words, the slices' scale partials
-    const size_t rows = (size_t)a.BH * a.T, zero_n = 4 * n + (rows + 3) / 4 * 2;  // 16-byte aligned parts
-    unsigned* poison = reinterpret_cast<unsigned*>(acc + 4 * n);
+    p.round_parts = f32_round_parts(a.BH, a.T);
+    const bool q_shared = want_q && p.round_parts > 1;
+    p.dq = a.dq; p.acc_q = q_shared ? acc + 4 * n : nullptr; p.acc_q_rows = 0; p.stats_part = nullptr; p.split_rounds = 0;
+    // scratch: four accumulators (five when the rounds of a tile are dealt out: dQ then has one too), the rows'
+    // poison words, the slices' scale partials
+    const size_t nacc = (p.round_parts > 1 ? 5 : 4) * n;
+    const size_t rows = (size_t)a.BH * a.T, zero_n = nacc + (rows + 3) / 4 * 2;  // 16-byte aligned parts
+    unsigned* poison = reinterpret_cast<unsigned*>(acc + nacc);
     unsigned* parts = reinterpret_cast<unsigned*>(acc + zero_n);
     p.scale_parts = parts; p.poison = poison; p.scale_bias = kF32FixedBias;
     p.T = a.T; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
@@ -691,6 +710,9 @@ hipError_t launch_f32_bwd(const GenericTdpArgs& a, long long* acc, hipStream_t s
         return e;
     size_t gf = (n + 255) / 256;
     if (gf > 4096) gf = 4096;
+    if (q_shared)
+        hipLaunchKernelGGL(f32_finish_q_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc + 4 * n, a.dq, n, a.T, D, parts,
+                           poison, a.alpha);
     if (want_k2)
         hipLaunchKernelGGL(f32_finish_kernel, dim3((unsigned)gf), dim3(256), 0, st, acc, a.dk2, a.dv2, n, a.T, D, parts,
                            poison, kPoisonDK2, kPoisonDV2);
@@ -726,6 +748,14 @@ hipError_t launch_f32_fwd(const GenericTdpArgs& a, hipStream_t st) {
 }  // namespace
 
 bool f32_mfma_tdp_supported(int D) { return D == 32 || D == 64 || D == 128; }
+
+// Measured at D = 64 with narrow windows (seven rounds of two or three stages per tile): a round costs about 25 us and
+// a workgroup about 50 us before its first one, so dealing rounds out pays while the tiles alone leave more than half
+// of the compute units idle (32 tiles: 245 -> 75 us per launch), and not beyond (128 tiles: 245 -> 260 us).
+int f32_round_parts(int BH, int T) {
+    const int tiles = BH * ((T + 31) / 32);
+    return tiles >= 128 ? 1 : std::min(16, (256 + tiles - 1) / tiles);
+}
 
 // The first query tiles of a 16-bit backward, in fp32 (see the comment above tdp_f32_bwd_kernel).
 template <typename E, int D>
@@ -769,7 +799,7 @@ static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
     }
     F32BwdParams<E> r0{};
     r0.q = (const E*)a.q; r0.d_o = (const E*)a.d_o; r0.lse = nullptr; r0.delta = nullptr;
-    r0.stats_part = a.delta_f32; r0.split_rounds = rounds;
+    r0.stats_part = a.delta_f32; r0.split_rounds = rounds; r0.round_parts = 1;
     r0.dq = (E*)a.dq; r0.acc_q = a.acc_q ? a.acc_q : a.dq0_acc; r0.acc_q_rows = a.acc_q ? 0 : 32;
     r0.scale_parts = a.scale_parts; r0.poison = a.poison; r0.scale_bias = a.scale_bias;
     r0.T = a.T; r0.BH = a.BH; r0.nqt = 1; r0.alpha = a.alpha;
@@ -801,6 +831,7 @@ static hipError_t first_tile_typed(const FirstTileArgs& a, hipStream_t st) {
     F32BwdParams<E> p{};
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o; p.lse = a.lse_f32; p.delta = a.delta_f32;
     p.dq = (E*)a.dq; p.acc_q = a.acc_q; p.acc_q_rows = 0; p.stats_part = nullptr; p.split_rounds = 0;
+    p.round_parts = a.round_parts;
     p.scale_parts = a.scale_parts; p.poison = a.poison; p.scale_bias = a.scale_bias;
     p.T = a.T; p.BH = a.BH; p.nqt = a.tiles;
     p.alpha = a.alpha;
@@ -827,7 +858,8 @@ hipError_t f32_mfma_tdp_fwd(const GenericTdpArgs& a, hipStream_t st) {
 }
 
 size_t f32_mfma_tdp_bwd_scratch_elems(int BH, int T, int D) {
-    return 4 * (size_t)BH * T * D + ((size_t)BH * T + 3) / 4 * 2 + (size_t)BH * kScaleParts / 2;
+    return (f32_round_parts(BH, T) > 1 ? 5 : 4) * (size_t)BH * T * D + ((size_t)BH * T + 3) / 4 * 2 +
+           (size_t)BH * kScaleParts / 2;
 }
 
 hipError_t f32_mfma_tdp_bwd(const GenericTdpArgs& a, long long* scratch, hipStream_t st) {

@@ -320,7 +320,7 @@ def test_mfma_forward_large_logits():
 SPLIT = _lib.FLAG_SPLIT_OPERANDS
 
 
-@pytest.mark.parametrize("windows", [(None,) * 4, (64, 100, 20, 30)])
+@pytest.mark.parametrize("windows", [(None,) * 4, (64, 100, 20, 30), (24, 22, None, None), (3, 200, 0, 2)])
 @pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (32, torch.bfloat16), (64, torch.float16), (128, torch.bfloat16)])
 def test_large_logits_with_convert_to_float32_hold_the_16_bit_bar(windows, D, dtype):
     """convert_to_float32=True keeps the operands of the score products beyond 16-bit rounding, as the reference's
