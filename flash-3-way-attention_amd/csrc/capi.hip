@@ -193,9 +193,10 @@ int clampw(int w, int T) { return w > T ? T : w; }
 
 // The fp32 path has two sets of kernels: on the matrix cores (v_mfma_f32_32x32x2_f32; a workgroup per 32 queries)
 // and on the vector ALUs (a wave per query: far more workgroups, the better shape for problems of a few tiles).
-bool use_f32_mfma(int BH, int T) {
+bool use_f32_mfma(int BH, int T, bool backward = false) {
     if (knobs().f32_valu) return false;
-    return (long long)BH * ((T + 31) / 32) >= 64;
+    // the backward deals the rounds of a tile out to workgroups when the tiles alone leave the chip idle
+    return (long long)BH * ((T + 31) / 32) >= (backward ? 8 : 64);
 }
 
 // ---------------------------------------------------------------- triple-dot, fp32 VALU path
@@ -258,10 +259,10 @@ int tdp_bwd_generic(Arena& ar, bool run, const void* q, const void* k1, const vo
     a.q = in.q; a.k1 = in.k1; a.k2 = in.k2; a.u = in.u; a.v2 = in.v2;
     a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha;
     a.causal = causal; a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
-    const bool mfma32 = fixed && use_f32_mfma(B * H, T);
+    const bool mfma32 = fixed && use_f32_mfma(B * H, T, true);
     if (o32) {
         a.o = o32; a.lse = lse32;
-        hipError_t ef = mfma32 ? f32_mfma_tdp_fwd(a, st) : generic_tdp_fwd(a, st);
+        hipError_t ef = (fixed && use_f32_mfma(B * H, T)) ? f32_mfma_tdp_fwd(a, st) : generic_tdp_fwd(a, st);
         if (ef != hipSuccess) return (int)ef;
         rowdot(do32, o32, delta, B * H * T, D, TRITT_F32, st);
         lse = lse32;
@@ -402,6 +403,88 @@ bool any_misaligned(std::initializer_list<const void*> ps) {
         if (reinterpret_cast<uintptr_t>(p) & 15) return true;
     return false;
 }
+
+// ---------------------------------------------------------------- strided views of the inputs
+// A view is dense when it is the [B,H,T,D] layout itself (strides of dimensions of extent 1 never matter).
+bool layout_dense(const tritt_layout* l, int B, int H, int T, int D) {
+    if (!l) return true;
+    return (T == 1 || l->stride_t == D) && (H == 1 || l->stride_h == (long long)T * D) &&
+           (B == 1 || l->stride_b == (long long)H * T * D);
+}
+// 16-byte pieces must stay aligned: every stride a multiple of 16 bytes, none negative
+int check_layout(const tritt_layout* l, int dtype) {
+    if (!l) return TRITT_OK;
+    const long long unit = 16 / (long long)elem_size(dtype);
+    if (l->stride_b < 0 || l->stride_h < 0 || l->stride_t < 0) return TRITT_ERR_INVALID;
+    if (l->stride_b % unit || l->stride_h % unit || l->stride_t % unit) return TRITT_ERR_INVALID;
+    return TRITT_OK;
+}
+bool same_layout(const tritt_layout& a, const tritt_layout& b) {
+    return a.stride_b == b.stride_b && a.stride_h == b.stride_h && a.stride_t == b.stride_t;
+}
+
+// Dense copies of up to six strided [B,H,T,D] views, one launch: blockIdx.y picks the view, a thread moves 16 bytes.
+constexpr int kMaxViews = 6;
+struct PackArgs {
+    const char* src[kMaxViews];
+    char* dst[kMaxViews];
+    long long sb[kMaxViews], sh[kMaxViews], st[kMaxViews];  // bytes
+    int H, T, pieces;                                       // pieces: 16-byte pieces per row
+};
+__global__ __launch_bounds__(256) void pack_kernel(PackArgs a, long long total) {
+    const int v = blockIdx.y;
+    const char* __restrict__ src = a.src[v];
+    char* __restrict__ dst = a.dst[v];
+    const long long sb = a.sb[v], sh = a.sh[v], st = a.st[v];
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
+        const int c = (int)(i % a.pieces);
+        const long long row = i / a.pieces;
+        const int t = (int)(row % a.T);
+        const long long bh = row / a.T;
+        const long long b = bh / a.H, h = bh % a.H;
+        *reinterpret_cast<uint4*>(dst + i * 16) = *reinterpret_cast<const uint4*>(src + b * sb + h * sh + t * st + c * 16);
+    }
+}
+
+// The plan of a strided call: which views are packed into the tail of the workspace, and what the dense entry point
+// is then handed.  `base` null: measuring only.
+struct Views {
+    const void* ptr[kMaxViews];
+    PackArgs pack;
+    int jobs = 0;
+    size_t bytes = 0;  // of the packed copies
+};
+void plan_view(Views& v, int slot, const void* src, const tritt_layout* l, bool keep, char* base, size_t n_bytes, int es) {
+    v.ptr[slot] = src;
+    if (keep) return;
+    char* dst = base ? base + v.bytes : nullptr;
+    v.bytes += (n_bytes + 255) & ~size_t(255);
+    v.pack.src[v.jobs] = static_cast<const char*>(src);
+    v.pack.dst[v.jobs] = dst;
+    v.pack.sb[v.jobs] = l->stride_b * es; v.pack.sh[v.jobs] = l->stride_h * es; v.pack.st[v.jobs] = l->stride_t * es;
+    ++v.jobs;
+    v.ptr[slot] = dst;
+}
+void run_pack(Views& v, int B, int H, int T, int D, int dtype, hipStream_t st) {
+    if (!v.jobs) return;
+    v.pack.H = H; v.pack.T = T; v.pack.pieces = D * (int)elem_size(dtype) / 16;
+    const long long total = (long long)B * H * T * v.pack.pieces;
+    long long g = (total + 255) / 256;
+    if (g > 4096) g = 4096;
+    hipLaunchKernelGGL(pack_kernel, dim3((unsigned)g, v.jobs), dim3(256), 0, st, v.pack, total);
+}
+// every view of `src[count]` that is not dense gets a packed copy (layouts null: all dense)
+int plan_all(Views& v, int first_slot, const void* const* src, const tritt_layout* layouts, int count, char* base, int B,
+             int H, int T, int D, int dtype) {
+    const size_t n_bytes = (size_t)B * H * T * D * elem_size(dtype);
+    for (int i = 0; i < count; ++i) {
+        const tritt_layout* l = layouts ? layouts + i : nullptr;
+        if (int rc = check_layout(l, dtype); rc != TRITT_OK) return rc;
+        plan_view(v, first_slot + i, src[i], l, layout_dense(l, B, H, T, D), base, n_bytes, (int)elem_size(dtype));
+    }
+    return TRITT_OK;
+}
+size_t round256(size_t x) { return (x + 255) & ~size_t(255); }
 
 // Library-owned scratch of tritt_tdp_fwd_static_scratch: one copy per GPU the code object is loaded on, held
 // until the process ends.  The name is a host-side stand-in; the device address comes from hipGetSymbolAddress.
@@ -649,6 +732,179 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
     Arena ar(workspace);
     return dps_bwd_impl(ar, true, q, k1, k2, v1, v2, o, lse, d_o, dq, dk1, dk2, dv1, dv2, B, H, T, D, dtype, alpha,
                         causal, clampw(k_diff, T), (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------- strided entry points
+// The triple-dot forward on the 16-bit matrix-core path reads strided views in place: V1 always (the SiLU / transpose
+// pass takes its layout), the other four when they share one layout with a row stride the kernels' 32-bit field holds.
+static bool fwd_reads_in_place(const tritt_layout* l, int dtype, int T) {
+    if (!l) return true;
+    for (int i : {1, 2, 4})
+        if (!same_layout(l[0], l[i])) return false;
+    for (int i = 0; i < 5; ++i)
+        // the kernels form row offsets in 32 bits; a row stride of 0 (a broadcast view) would read as "dense" in the
+        // launch arguments
+        if (check_layout(l + i, dtype) != TRITT_OK || (long long)T * l[i].stride_t > 0x7fffffffLL ||
+            (T > 1 && l[i].stride_t == 0))
+            return false;
+    return true;
+}
+
+size_t tritt_tdp_fwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window,
+                                             int k2_window, int kk_left, int kk_right, unsigned flags,
+                                             const tritt_layout* in_layouts) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    const size_t plain =
+        round256(tritt_tdp_fwd_workspace_bytes(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags));
+    if (use_mfma_fwd(T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags) &&
+        fwd_reads_in_place(in_layouts, dtype, T))
+        return plain;
+    Views v;
+    const void* none[5] = {};
+    if (plan_all(v, 0, none, in_layouts, 5, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
+    return plain + v.bytes;
+}
+
+int tritt_tdp_fwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, void* o, float* lse, int B, int H, int T, int D, int dtype,
+                          float alpha, int causal, int k1_window, int k2_window, int kk_left, int kk_right,
+                          void* workspace, size_t workspace_bytes, unsigned flags, void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o})) return TRITT_ERR_INVALID;
+    if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
+    for (int i = 0; in_layouts && i < 5; ++i)
+        if ((rc = check_layout(in_layouts + i, dtype)) != TRITT_OK) return rc;
+    const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
+    const size_t plain = round256(tritt_tdp_fwd_workspace_bytes(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags));
+    const bool mfma = use_mfma_fwd(T, D, dtype, causal, w1, w2, kl, kr, flags);
+    if (mfma && in_layouts && fwd_reads_in_place(in_layouts, dtype, T)) {
+        if ((flags & TRITT_FLAG_SPLIT_OPERANDS) && !use_split(D, dtype, flags)) return TRITT_ERR_UNSUPPORTED;
+        if (plain && (!workspace || workspace_bytes < plain)) return TRITT_ERR_WORKSPACE;
+        MfmaFwdArgs a = mfma_fwd_shape(B, H, T, D, dtype, causal, w1, w2, kl, kr, flags);
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.lse = lse; a.ut = workspace;
+        a.alpha = alpha;
+        a.H = H;
+        // a dense view goes as dense (strides of extent-1 dimensions may hold anything)
+        if (!layout_dense(in_layouts, B, H, T, D)) {
+            a.in_sb = in_layouts[0].stride_b; a.in_sh = in_layouts[0].stride_h; a.in_st = in_layouts[0].stride_t;
+            if (T == 1) a.in_st = D;  // never used as a step; 0 would read as "dense"
+        }
+        if (!layout_dense(in_layouts + 3, B, H, T, D)) {
+            a.v1_sb = in_layouts[3].stride_b; a.v1_sh = in_layouts[3].stride_h; a.v1_st = in_layouts[3].stride_t;
+            if (T == 1) a.v1_st = D;
+        }
+        return (int)mfma_tdp_fwd(a, (hipStream_t)stream);
+    }
+    Views v;
+    const void* src[5] = {q, k1, k2, v1, v2};
+    rc = plan_all(v, 0, src, in_layouts, 5, workspace ? (char*)workspace + plain : nullptr, B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if ((plain + v.bytes) && (!workspace || workspace_bytes < plain + v.bytes)) return TRITT_ERR_WORKSPACE;
+    run_pack(v, B, H, T, D, dtype, (hipStream_t)stream);
+    return tritt_tdp_fwd(v.ptr[0], v.ptr[1], v.ptr[2], v.ptr[3], v.ptr[4], o, lse, B, H, T, D, dtype, alpha, causal,
+                         k1_window, k2_window, kk_left, kk_right, workspace, plain, flags, stream);
+}
+size_t tritt_dps_fwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags,
+                                             const tritt_layout* in_layouts) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    Views v;
+    const void* none[5] = {};
+    if (plan_all(v, 0, none, in_layouts, 5, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
+    return round256(tritt_dps_fwd_workspace_bytes(B, H, T, D, dtype, flags)) + v.bytes;
+}
+
+int tritt_dps_fwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, void* o, float* lse, int B, int H, int T, int D, int dtype,
+                          float alpha, int causal, int k_diff, void* workspace, size_t workspace_bytes, unsigned flags,
+                          void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o})) return TRITT_ERR_INVALID;
+    const size_t plain = round256(tritt_dps_fwd_workspace_bytes(B, H, T, D, dtype, flags));
+    Views v;
+    const void* src[5] = {q, k1, k2, v1, v2};
+    rc = plan_all(v, 0, src, in_layouts, 5, workspace ? (char*)workspace + plain : nullptr, B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (!workspace || workspace_bytes < plain + v.bytes) return TRITT_ERR_WORKSPACE;
+    run_pack(v, B, H, T, D, dtype, (hipStream_t)stream);
+    return tritt_dps_fwd(v.ptr[0], v.ptr[1], v.ptr[2], v.ptr[3], v.ptr[4], o, lse, B, H, T, D, dtype, alpha, causal, k_diff,
+                         workspace, plain, flags, stream);
+}
+
+size_t tritt_dps_bwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags,
+                                             const tritt_layout* in_layouts, const tritt_layout* d_o_layout) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    Views v;
+    const void* none[5] = {};
+    if (plan_all(v, 0, none, in_layouts, 5, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (plan_all(v, 5, none, d_o_layout, 1, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
+    return round256(tritt_dps_bwd_workspace_bytes(B, H, T, D, dtype, flags)) + v.bytes;
+}
+
+int tritt_dps_bwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, const void* o, const float* lse, const void* d_o,
+                          const tritt_layout* d_o_layout, void* dq, void* dk1, void* dk2, void* dv1, void* dv2, int B,
+                          int H, int T, int D, int dtype, float alpha, int causal, int k_diff, void* workspace,
+                          size_t workspace_bytes, unsigned flags, void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse, d_o})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o, d_o})) return TRITT_ERR_INVALID;
+    const size_t plain = round256(tritt_dps_bwd_workspace_bytes(B, H, T, D, dtype, flags));
+    Views v;
+    const void* src[5] = {q, k1, k2, v1, v2};
+    char* tail = workspace ? (char*)workspace + plain : nullptr;
+    rc = plan_all(v, 0, src, in_layouts, 5, tail, B, H, T, D, dtype);
+    if (rc == TRITT_OK) rc = plan_all(v, 5, &d_o, d_o_layout, 1, tail, B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (!workspace || workspace_bytes < plain + v.bytes) return TRITT_ERR_WORKSPACE;
+    run_pack(v, B, H, T, D, dtype, (hipStream_t)stream);
+    return tritt_dps_bwd(v.ptr[0], v.ptr[1], v.ptr[2], v.ptr[3], v.ptr[4], o, lse, v.ptr[5], dq, dk1, dk2, dv1, dv2, B, H, T,
+                         D, dtype, alpha, causal, k_diff, workspace, plain, flags, stream);
+}
+
+size_t tritt_tdp_bwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window,
+                                             int k2_window, int kk_left, int kk_right, unsigned flags,
+                                             const tritt_layout* in_layouts, const tritt_layout* d_o_layout) {
+    if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    Views v;
+    const void* none[5] = {};
+    if (plan_all(v, 0, none, in_layouts, 5, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (plan_all(v, 5, none, d_o_layout, 1, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
+    return round256(tritt_tdp_bwd_workspace_bytes(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags)) +
+           v.bytes;
+}
+
+int tritt_tdp_bwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, const void* o, const float* lse, const void* d_o,
+                          const tritt_layout* d_o_layout, void* dq, void* dk1, void* dk2, void* dv1, void* dv2, int B,
+                          int H, int T, int D, int dtype, float alpha, int causal, int k1_window, int k2_window,
+                          int kk_left, int kk_right, void* workspace, size_t workspace_bytes, unsigned flags,
+                          void* stream) {
+    if (empty_problem(B, H, T)) return check_common(1, 1, 1, D, dtype);
+    int rc = check_common(B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (any_null({q, k1, k2, v1, v2, o, lse, d_o})) return TRITT_ERR_INVALID;
+    if (any_misaligned({q, k1, k2, v1, v2, o, d_o})) return TRITT_ERR_INVALID;
+    if (!dq && !dk1 && !dk2 && !dv1 && !dv2) return TRITT_OK;
+    const size_t plain =
+        round256(tritt_tdp_bwd_workspace_bytes(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags));
+    Views v;
+    const void* src[5] = {q, k1, k2, v1, v2};
+    char* tail = workspace ? (char*)workspace + plain : nullptr;
+    rc = plan_all(v, 0, src, in_layouts, 5, tail, B, H, T, D, dtype);
+    if (rc == TRITT_OK) rc = plan_all(v, 5, &d_o, d_o_layout, 1, tail, B, H, T, D, dtype);
+    if (rc != TRITT_OK) return rc;
+    if (!workspace || workspace_bytes < plain + v.bytes) return TRITT_ERR_WORKSPACE;
+    run_pack(v, B, H, T, D, dtype, (hipStream_t)stream);
+    return tritt_tdp_bwd(v.ptr[0], v.ptr[1], v.ptr[2], v.ptr[3], v.ptr[4], o, lse, v.ptr[5], dq, dk1, dk2, dv1, dv2, B, H, T,
+                         D, dtype, alpha, causal, k1_window, k2_window, kk_left, kk_right, workspace, plain, flags, stream);
 }
 
 }  // extern "C"

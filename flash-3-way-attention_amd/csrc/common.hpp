@@ -63,7 +63,7 @@ __device__ __forceinline__ float wave_max(float v) {
 // SILU applies x -> SiLU(x) on the way and, with `rows` non-null, also stores the result row-major.
 template <typename E, bool SILU>
 __device__ __forceinline__ void transpose_load(const E* __restrict__ src, E* __restrict__ rows, E* tile, int j0, int T,
-                                               int D) {
+                                               int D, unsigned src_stride = 0 /* elements between rows of src; 0: D */) {
     typedef __attribute__((ext_vector_type(8))) E e8;
     const int ld = D + 2, cpr = D / 8;
     for (int idx = threadIdx.x; idx < 64 * cpr; idx += 256) {
@@ -72,7 +72,7 @@ __device__ __forceinline__ void transpose_load(const E* __restrict__ src, E* __r
 #pragma unroll
         for (int e = 0; e < 8; ++e) x[e] = (E)0.f;
         if (j < T) {
-            x = *reinterpret_cast<const e8*>(src + (size_t)j * D + c * 8);
+            x = *reinterpret_cast<const e8*>(src + (size_t)j * (src_stride ? src_stride : (unsigned)D) + c * 8);
             if (SILU) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) x[e] = (E)silu_f((float)x[e]);

@@ -68,8 +68,13 @@ struct FirstTileArgs {
     int causal, k1_window, k2_window, kk_left, kk_right;
     bool want_q, want_k2, want_k1;
     int tiles;
+    int round_parts;  // tiles > 1: workgroups per query tile (its rounds of eight rows dealt out); above 1 needs acc_q when dQ is wanted
 };
 hipError_t f32_mfma_tdp_bwd_first_tile(const FirstTileArgs& a, hipStream_t st);
+// Workgroups per query tile of the fp32 matrix-core backward over all tiles: one workgroup walks a tile's rounds (of
+// eight rows) one after another, so a grid that leaves most compute units idle (short sequences, few heads) is
+// dealt out by rounds as well.
+int f32_round_parts(int BH, int T);
 
 // fp32 operands of the dot-product-sum kernels (two chained attention passes).
 struct DpsArgs {
@@ -107,6 +112,10 @@ struct MfmaFwdArgs {
     // split operands (D = 32, 64): the Q (.) K2 operand of the score products as a hi + lo pair of 16-bit numbers;
     // `o` then holds two [BH][T][D] tensors, the output and its rounding residual
     int split;
+    // Strided inputs: element (b, h, t, d) of Q, K1, K2 and V2 at b in_sb + h in_sh + t in_st + d elements, of V1 at the
+    // v1_* strides; H = heads (BH = batch * H).  in_st == 0 / v1_st == 0: dense [BH][T][D].  Row strides below 2^32.
+    long long in_sb, in_sh, in_st, v1_sb, v1_sh, v1_st;
+    int H;
 };
 bool mfma_tdp_split_supported(int D, int dtype_is_16bit);
 // needs BH, T, D, causal, windowed, split and the four windows of `a`

@@ -58,22 +58,24 @@ __global__ __launch_bounds__(512, 2) void tdp_fwd_band_kernel(FwdParams<E> p, in
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
-    const size_t base = (size_t)bh * T * D;
-    const E* __restrict__ Q = p.q + base;
+    const size_t base = (size_t)bh * T * D;  // of the outputs
+    const size_t in_base = (size_t)(bh / p.H) * p.in_sb + (size_t)(bh % p.H) * p.in_sh;
+    const unsigned in_st = p.in_st;
+    const E* __restrict__ Q = p.q + in_base;
     const int wa = p.wa, wb = p.wb, lab = p.lab, rab = p.rab;
     const int q0 = qt * kBandQ;
     const int rlo = max(0, q0 - max(wa, wb)) & ~31;  // first resident key row
 
     // ---- load the band ---------------------------------------------------------------------------
     {
-        const E* __restrict__ K1 = p.k1 + base;
-        const E* __restrict__ K2 = p.k2 + base;
-        const E* __restrict__ V2 = p.v2 + base;
+        const E* __restrict__ K1 = p.k1 + in_base;
+        const E* __restrict__ K2 = p.k2 + in_base;
+        const E* __restrict__ V2 = p.v2 + in_base;
         const E* __restrict__ UT = p.ut + (size_t)bh * D * p.Tp;
         const int row_chunks = NR * (D / 8);
         for (int c = tid; c < row_chunks; c += 512) {
             const int r = c / (D / 8), ch = c % (D / 8);
-            const size_t src = (size_t)min(rlo + r, T - 1) * D + ch * 8;
+            const size_t src = (size_t)((unsigned)min(rlo + r, T - 1) * in_st) + ch * 8;
             const uint4 a = *reinterpret_cast<const uint4*>(K1 + src);
             const uint4 b = *reinterpret_cast<const uint4*>(K2 + src);
             const uint4 v = *reinterpret_cast<const uint4*>(V2 + src);
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(512, 2) void tdp_fwd_band_kernel(FwdParams<E> p, in
     }
     for (int idx = tid; idx < kBandQ * D; idx += 512) {
         const int r = idx / D, d = idx % D;
-        sQ[idx] = (float)Q[(size_t)min(q0 + r, T - 1) * D + d] * p.scale_log2;
+        sQ[idx] = (float)Q[(size_t)((unsigned)min(q0 + r, T - 1) * in_st) + d] * p.scale_log2;
     }
     // ---- band mask table: slot -> offset m = (jb - k0) / 32 ----------------------------------------
     const int mlo = -((lab + 31) / 32), mhi = (rab + 31) / 32;

@@ -38,6 +38,11 @@ template <typename E>
 struct FwdParams {
     const E *q, *k1, *k2, *v2;
     const E* ut;  // [BH][D][Tp]  SiLU(V1) transposed, zero padded to Tp (multiple of 64)
+    // Q, K1, K2, V2 are views of one layout: element (b, h, t, d) at b in_sb + h in_sh + t in_st + d.  The outputs, U^T
+    // and the parts are dense.
+    long long in_sb, in_sh;
+    unsigned in_st;
+    int H;
     E* o;
     E* o_res;  // SPLIT: the rounding residual of every output element, O(fp32) - O(16 bit), as a second tensor
     float* lse;
@@ -124,11 +129,13 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it scalar
     const int T = p.T;
-    const size_t base = (size_t)bh * T * D;
-    const E* __restrict__ Q = p.q + base;
-    const E* __restrict__ K1 = p.k1 + base;
-    const E* __restrict__ K2 = p.k2 + base;
-    const E* __restrict__ V2 = p.v2 + base;
+    const size_t base = (size_t)bh * T * D;  // of the outputs
+    const size_t in_base = (size_t)(bh / p.H) * p.in_sb + (size_t)(bh % p.H) * p.in_sh;
+    const unsigned in_st = p.in_st;  // row stride of the inputs, elements; (T - 1) in_st + D fits 32 bits
+    const E* __restrict__ Q = p.q + in_base;
+    const E* __restrict__ K1 = p.k1 + in_base;
+    const E* __restrict__ K2 = p.k2 + in_base;
+    const E* __restrict__ V2 = p.v2 + in_base;
     const E* __restrict__ UT = p.ut + (size_t)bh * D * p.Tp;
     float* sWw = sW + wave * 32;
 
@@ -170,7 +177,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     uint4 ra0, ra1, rb0, rb1, rkv0, rkv1;
     auto k1_chunk = [&](int item, int jb) {
         const int r = item / (D / 8), ch = item % (D / 8);
-        return reinterpret_cast<const uint4*>(K1 + (size_t)min(jb + r, T - 1) * D + ch * 8);
+        return reinterpret_cast<const uint4*>(K1 + (size_t)((unsigned)min(jb + r, T - 1) * in_st) + ch * 8);
     };
     auto ut_chunk = [&](int i2, int jb) {
         const int d = i2 / (JS / 8), cj = i2 % (JS / 8);
@@ -217,7 +224,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     auto kt_src = [&](int item, int kt) {
         const int which = item / (4 * D), rem = item % (4 * D);
         const int r = rem / (D / 8), ch = rem % (D / 8);
-        return reinterpret_cast<const uint4*>((which ? V2 : K2) + (size_t)min(kt * 32 + r, T - 1) * D + ch * 8);
+        return reinterpret_cast<const uint4*>((which ? V2 : K2) + (size_t)((unsigned)min(kt * 32 + r, T - 1) * in_st) + ch * 8);
     };
     auto kt_dst = [&](int item, int buf) {
         const int which = item / (4 * D), rem = item % (4 * D);
@@ -252,7 +259,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     // ---- prologue: Q tile, first k-tile, first stage ------------------------------------------
     for (int idx = tid; idx < BQ * D; idx += NTH) {
         const int r = idx / D, d = idx % D;
-        sQ[r * LDQ + d] = (float)Q[(size_t)min(q0 + r, T - 1) * D + d] * p.scale_log2;
+        sQ[r * LDQ + d] = (float)Q[(size_t)((unsigned)min(q0 + r, T - 1) * in_st) + d] * p.scale_log2;
     }
     if (tid < 2) sFlag[tid] = 0;  // two flags, used by alternate k-tiles
     issue_ktile(kt_lo);
@@ -891,10 +898,11 @@ __global__ __launch_bounds__(256) void fwd_merge_kernel(const float* __restrict_
 // U^T[bh][d][j] = SiLU(V1[bh][j][d]) for j < T, 0 for T <= j < Tp
 template <typename E>
 __global__ __launch_bounds__(256) void silu_transpose_kernel(const E* __restrict__ v1, E* __restrict__ ut, int T,
-                                                             int Tp, int D) {
+                                                             int Tp, int D, int H, long long sb, long long sh,
+                                                             unsigned st) {
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     __shared__ E tile[64 * (128 + 2)];
-    transpose_load<E, true>(v1 + (size_t)bh * T * D, nullptr, tile, j0, T, D);
+    transpose_load<E, true>(v1 + (size_t)(bh / H) * sb + (size_t)(bh % H) * sh, nullptr, tile, j0, T, D, st);
     __syncthreads();
     transpose_store<E>(ut + (size_t)bh * D * Tp, tile, j0, Tp, D);
 }
@@ -939,14 +947,28 @@ static bool use_band_kernel(const MfmaFwdArgs& a) {
     return smem <= kBandSmemLimit;
 }
 
+// The layout the kernels are handed: the caller's strides, or those of a dense [BH][T][D] tensor (in_st == 0)
+struct InLayout {
+    long long sb, sh;
+    unsigned st;
+    int H;
+};
+static InLayout input_layout(const MfmaFwdArgs& a, bool of_v1) {
+    const long long st = of_v1 ? a.v1_st : a.in_st;
+    if (st == 0) return {(long long)a.T * a.D, 0, (unsigned)a.D, 1};  // dense: batch and head are one index
+    return of_v1 ? InLayout{a.v1_sb, a.v1_sh, (unsigned)a.v1_st, a.H} : InLayout{a.in_sb, a.in_sh, (unsigned)a.in_st, a.H};
+}
+
 template <typename E, int D>
 static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
+    const InLayout lin = input_layout(a, false), lv1 = input_layout(a, true);
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
-                       a.T, Tp, D);
+                       a.T, Tp, D, lin.H, lv1.sb, lv1.sh, lv1.st);
     FwdParams<E> p;
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
     p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse; p.o_res = nullptr;
+    p.in_sb = lin.sb; p.in_sh = lin.sh; p.in_st = lin.st; p.H = lin.H;
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + kBandQ - 1) / kBandQ;
     p.scale_log2 = a.alpha * kLog2e;
     p.causal = 1;
@@ -977,13 +999,15 @@ static int fwd_splits(const MfmaFwdArgs& a, int bq) {
 template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false, bool SPLIT = false>
 static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
+    const InLayout lin = input_layout(a, false), lv1 = input_layout(a, true);
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
-                       a.T, Tp, D);
+                       a.T, Tp, D, lin.H, lv1.sb, lv1.sh, lv1.st);
     constexpr int BQ = WAVES * NT;
     if (BQ != fwd_tile_queries(D, a.windowed)) return hipErrorInvalidValue;  // the workspace was sized for another shape
     FwdParams<E> p;
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
     p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse;
+    p.in_sb = lin.sb; p.in_sh = lin.sh; p.in_st = lin.st; p.H = lin.H;
     p.o_res = SPLIT ? (E*)a.o + (size_t)a.BH * a.T * D : nullptr;
     p.T = a.T; p.Tp = Tp; p.BH = a.BH; p.nqt = (a.T + BQ - 1) / BQ;
     p.scale_log2 = a.alpha * kLog2e;

@@ -185,6 +185,62 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
                   int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
                   void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
 
+/* ---- strided inputs ------------------------------------------------------------------------
+ * The entry points above take dense [B,H,T,D] tensors.  The reference accepts views of any strides and copies them
+ * (triple_dot_product/flash_trittention.py:64-68,153; dot_product_sum/trittention_triton.py:43-47;
+ * tests/test_dot_product_sum.py:121-134); a projection layer usually hands over [B,T,H,D] (or a slice of a fused
+ * [B,T,5,H,D]) transposed.  The *_strided entry points take such views as they are: a tritt_layout gives the
+ * element strides of a view whose last dimension is dense (element (b,h,t,d) at
+ * ptr + b*stride_b + h*stride_h + t*stride_t + d).  `in_layouts` points to five of them, for q, k1, k2, v1, v2 in this
+ * order (NULL: all dense); `d_o_layout` to the one of dO (NULL: dense).  Strides are non-negative multiples of 16
+ * bytes (8 elements of a 16-bit type, 4 of fp32), the row stride below 2^31 elements, pointers 16-byte aligned as
+ * before; else TRITT_ERR_INVALID.  Outputs (o, lse, the gradients) and the saved `o` are dense.
+ *   tritt_tdp_fwd_strided on the 16-bit matrix-core path (see tritt_tdp_fwd) reads the views in place: V1 through
+ *     the SiLU/transpose pass it makes anyway, Q, K1, K2 and V2 inside the main kernel when the four share one layout.
+ *   Everywhere else (the backward calls, dot-product-sum, fp32 tensors, four differing layouts) the views that are
+ *     not dense are first gathered into the tail of the workspace by one launch for all of them, and the dense
+ *     code runs on the copies: one read and one write of each such tensor (B=4 H=8 T=1024 D=64: 12 us for six
+ *     tensors, against 11 ms of triple-dot backward), no allocation, no per-tensor launches.
+ * The *_strided_workspace_bytes queries take the same layouts and return the dense call's size plus the room of those
+ * copies; everything else is as in the dense call of the same name. */
+typedef struct tritt_layout {
+    long long stride_b, stride_h, stride_t;
+} tritt_layout;
+
+size_t tritt_tdp_fwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
+                                             int k1_window, int k2_window, int kk_left, int kk_right,
+                                             unsigned flags, const tritt_layout* in_layouts);
+int tritt_tdp_fwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, void* o, float* lse,
+                          int B, int H, int T, int D, int dtype, float alpha, int causal,
+                          int k1_window, int k2_window, int kk_left, int kk_right,
+                          void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+size_t tritt_tdp_bwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, int causal,
+                                             int k1_window, int k2_window, int kk_left, int kk_right,
+                                             unsigned flags, const tritt_layout* in_layouts,
+                                             const tritt_layout* d_o_layout);
+int tritt_tdp_bwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, const void* o, const float* lse,
+                          const void* d_o, const tritt_layout* d_o_layout,
+                          void* dq, void* dk1, void* dk2, void* dv1, void* dv2,
+                          int B, int H, int T, int D, int dtype, float alpha, int causal,
+                          int k1_window, int k2_window, int kk_left, int kk_right,
+                          void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+size_t tritt_dps_fwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags,
+                                             const tritt_layout* in_layouts);
+int tritt_dps_fwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, void* o, float* lse,
+                          int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
+                          void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+size_t tritt_dps_bwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags,
+                                             const tritt_layout* in_layouts, const tritt_layout* d_o_layout);
+int tritt_dps_bwd_strided(const void* q, const void* k1, const void* k2, const void* v1, const void* v2,
+                          const tritt_layout* in_layouts, const void* o, const float* lse,
+                          const void* d_o, const tritt_layout* d_o_layout,
+                          void* dq, void* dk1, void* dk2, void* dv1, void* dv2,
+                          int B, int H, int T, int D, int dtype, float alpha, int causal, int k_diff,
+                          void* workspace, size_t workspace_bytes, unsigned flags, void* stream);
+
 /* Calibration for benchmarks (no counterpart in the reference).  Launches `blocks` workgroups of
  * eight waves that each issue iters * 4 independent 32x32x16 bf16 MFMAs and nothing else:
  * blocks * 8 * iters * 4 * 32768 flop.  Timed by the caller, it gives the rate the matrix pipes
