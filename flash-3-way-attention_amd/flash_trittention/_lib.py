@@ -21,6 +21,14 @@ _DTYPES = {torch.float32: TRITT_F32, torch.bfloat16: TRITT_BF16, torch.float16: 
 
 _vp, _i, _f, _sz, _u = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_uint
 
+
+class Layout(ctypes.Structure):
+    """tritt_layout: element strides of a [B,H,T,D] view whose last dimension is dense."""
+    _fields_ = [("stride_b", ctypes.c_longlong), ("stride_h", ctypes.c_longlong), ("stride_t", ctypes.c_longlong)]
+
+
+_lp = ctypes.POINTER(Layout)
+
 _PROTOS = {
     "tritt_version": (_i, []),
     "tritt_status_string": (ctypes.c_char_p, [_i]),
@@ -36,6 +44,16 @@ _PROTOS = {
     "tritt_dps_fwd": (_i, [_vp] * 7 + [_i] * 5 + [_f] + [_i] * 2 + [_vp, _sz, _u, _vp]),
     "tritt_dps_bwd_workspace_bytes": (_sz, [_i] * 5 + [_u]),
     "tritt_dps_bwd": (_i, [_vp] * 13 + [_i] * 5 + [_f] + [_i] * 2 + [_vp, _sz, _u, _vp]),
+    "tritt_tdp_fwd_strided_workspace_bytes": (_sz, [_i] * 10 + [_u, _lp]),
+    "tritt_tdp_fwd_strided": (_i, [_vp] * 5 + [_lp] + [_vp] * 2 + [_i] * 5 + [_f] + [_i] * 5 + [_vp, _sz, _u, _vp]),
+    "tritt_tdp_bwd_strided_workspace_bytes": (_sz, [_i] * 10 + [_u, _lp, _lp]),
+    "tritt_tdp_bwd_strided": (_i, [_vp] * 5 + [_lp] + [_vp] * 3 + [_lp] + [_vp] * 5 + [_i] * 5 + [_f] + [_i] * 5
+                              + [_vp, _sz, _u, _vp]),
+    "tritt_dps_fwd_strided_workspace_bytes": (_sz, [_i] * 5 + [_u, _lp]),
+    "tritt_dps_fwd_strided": (_i, [_vp] * 5 + [_lp] + [_vp] * 2 + [_i] * 5 + [_f] + [_i] * 2 + [_vp, _sz, _u, _vp]),
+    "tritt_dps_bwd_strided_workspace_bytes": (_sz, [_i] * 5 + [_u, _lp, _lp]),
+    "tritt_dps_bwd_strided": (_i, [_vp] * 5 + [_lp] + [_vp] * 3 + [_lp] + [_vp] * 5 + [_i] * 5 + [_f] + [_i] * 2
+                              + [_vp, _sz, _u, _vp]),
 }
 
 _lib = None
@@ -136,6 +154,38 @@ def dense(t):
     return t
 
 
+def viewable(t) -> bool:
+    """Whether the library can read `t` (a [B,H,T,D] view) where it lies: dense last dimension, every other stride
+    a non-negative multiple of 16 bytes, 16-byte aligned start (tritt_layout's contract)."""
+    unit = 16 // t.element_size()
+    B, H, T, D = t.shape
+    if (D > 1 and t.stride(3) != 1) or t.data_ptr() % 16:
+        return False
+    return all(n == 1 or (s >= 0 and s % unit == 0) for n, s in zip((B, H, T), t.stride()[:3]))
+
+
+def view(t):
+    """`t` as the library can take it: the tensor itself when `viewable`, else a dense copy (what the reference
+    does with every input: triple_dot_product/flash_trittention.py:64-68)."""
+    return t if viewable(t) else dense(t)
+
+
+def layouts(tensors):
+    """A tritt_layout array for `tensors`, or None when every one of them is dense (the plain entry points serve)."""
+    if all(t.is_contiguous() for t in tensors):
+        return None
+    arr = (Layout * len(tensors))()
+    for slot, t in zip(arr, tensors):
+        # dimensions of extent 1 may carry any stride: the library ignores them, ctypes needs them in range
+        slot.stride_b, slot.stride_h, slot.stride_t = (s if n > 1 else 0 for n, s in zip(t.shape[:3], t.stride()[:3]))
+    return arr
+
+
+def layouts_key(arr):
+    """Hashable form of a layout array (workspace sizes are remembered per argument tuple)."""
+    return None if arr is None else tuple((l.stride_b, l.stride_h, l.stride_t) for l in arr)
+
+
 def ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
@@ -174,8 +224,9 @@ _workspace_sizes = {}
 
 def workspace_bytes(query: str, *args) -> int:
     """A `*_workspace_bytes` query of the library, remembered per argument tuple (the answer depends on nothing
-    else, except the tuning knobs: `tuning` and the tests' knob changes clear the memory)."""
-    key = (query, args)
+    else, except the tuning knobs: `tuning` and the tests' knob changes clear the memory).  Layout arrays in `args`
+    enter the key by value."""
+    key = (query, tuple(layouts_key(a) if isinstance(a, ctypes.Array) else a for a in args))
     size = _workspace_sizes.get(key)
     if size is None:
         size = _workspace_sizes[key] = getattr(lib(), query)(*args)

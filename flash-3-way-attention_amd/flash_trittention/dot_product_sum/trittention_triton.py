@@ -40,9 +40,11 @@ class TrittentionTritonFunction(torch.autograd.Function):
         if D not in (8, 16, 32, 64, 128):
             raise ValueError(f"head_dim must be one of 8, 16, 32, 64, 128, got {D}")
         _lib.dtype_code(q.dtype)
-        q, k1, k2, v1, v2 = (t.contiguous() for t in (q, k1, k2, v1, v2))
         k_diff = clamp_window(k_diff, T, "k_diff")
         compiling = _ops.compiling()
+        # views the library can read where they lie stay as they are (and are what the backward gets); the rest is
+        # copied, as the reference copies every input (trittention_triton.py:43-47)
+        q, k1, k2, v1, v2 = (t.contiguous() if compiling else _lib.view(t) for t in (q, k1, k2, v1, v2))
         flags = _lib.FLAG_AUTO if compiling else getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
         if convert_to_float32 and not flags & _lib.FLAG_FORCE_MFMA:
             flags |= _lib.FLAG_FORCE_GENERIC  # fp32 operands throughout (trittention_triton.py:92-98 of the reference)
@@ -62,7 +64,8 @@ class TrittentionTritonFunction(torch.autograd.Function):
         assert grad_output.shape == o.shape, f"Shape mismatch: O={o.shape}, dO={grad_output.shape}"
         assert o.device == grad_output.device, "O and dO must be on the same device"
         assert o.dtype == grad_output.dtype, "O and dO must have the same dtype"
-        grad_output = grad_output.contiguous()
+        if _ops.compiling():
+            grad_output = grad_output.contiguous()
         call = torch.ops.flash_trittention.dps_bwd if _ops.compiling() else _ops.dps_bwd_impl
         dq, dk1, dk2, dv1, dv2 = call(q, k1, k2, v1, v2, o, m, grad_output, ctx.softmax_scale, ctx.causal, ctx.k_diff,
                                       ctx.flags)

@@ -49,10 +49,13 @@ class FlashTrittention(torch.autograd.Function):
                 convert_to_float32):
         _validate(Q, (("K1", K1), ("K2", K2), ("V1", V1), ("V2", V2)))
         T = Q.shape[2]
-        Q, K1, K2, V1, V2 = (t.contiguous() for t in (Q, K1, K2, V1, V2))
         k1_window, k2_window, kk_left, kk_right = process_masking_variables(T, k1_window, k2_window, kk_left, kk_right)
         causal = bool(causal)
         compiling = _ops.compiling()  # tracing: the implementation flags are the class default
+        # views the library can read where they lie ([B,T,H,D] transposed, slices of a fused projection) stay as they
+        # are, and are what the backward gets; the rest is copied, as the reference copies every input
+        # (flash_trittention.py:64-68)
+        Q, K1, K2, V1, V2 = (t.contiguous() if compiling else _lib.view(t) for t in (Q, K1, K2, V1, V2))
         flags = _lib.FLAG_AUTO if compiling else getattr(getattr(ctx, "_forward_cls", None), "IMPL_FLAGS", _lib.FLAG_AUTO)
         if torch.are_deterministic_algorithms_enabled():
             flags &= ~_lib.FLAG_FLOAT_ATOMICS  # the default (fixed-point accumulation) is bitwise reproducible
@@ -80,7 +83,8 @@ class FlashTrittention(torch.autograd.Function):
         Q, K1, K2, V1, V2, O, LSE = ctx.saved_tensors
         if dO.dtype != Q.dtype:
             dO = dO.to(Q.dtype)
-        dO = dO.contiguous()
+        if _ops.compiling():
+            dO = dO.contiguous()
         k1_window, k2_window, kk_left, kk_right = ctx.windows
         # only the gradients autograd asks for: the library skips the others (and the kernel launch that serves
         # nothing else)

@@ -1,0 +1,213 @@
+"""Strided [B,H,T,D] views at the C ABI (tritt_*_strided): a projection layer's [B,T,H,D] output transposed, slices of
+one fused [B,T,5,H,D] tensor, mixed layouts.  The reference accepts such views and copies them
+(triple_dot_product/flash_trittention.py:64-68; its test: tests/test_dot_product_sum.py:121-134); here the triple-dot
+forward reads them where they lie and the other calls gather them inside the library's workspace.
+
+Every case is held to two bars: the oracle at the dtype's tolerance, and the dense call on `.contiguous()` copies of
+the same views bit for bit (the same kernels see the same numbers)."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from oracle import trittention_oracle as orc
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+LOWP = dict(rtol=5e-2, atol=2e-2)
+FP32 = dict(rtol=2e-3, atol=2e-4)
+
+
+def fused_views(B, H, T, D, dtype, seed):
+    """q, k1, k2, v1, v2 as slices of one [B,T,5,H,D] tensor, each seen as [B,H,T,D] (strides 5HDT, D, 5HD, 1)."""
+    g = torch.Generator().manual_seed(seed)
+    fused = torch.randn(B, T, 5, H, D, generator=g).to(dtype).cuda()
+    return [fused[:, :, i].transpose(1, 2) for i in range(5)], fused
+
+
+def bthd_view(B, H, T, D, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(B, T, H, D, generator=g).to(dtype).cuda().transpose(1, 2)
+
+
+def dense_inputs(views, d_o):
+    return [t.detach().contiguous().cpu() for t in (*views, d_o)]
+
+
+@pytest.mark.parametrize("shape,dtype,windows", [
+    ((2, 4, 256, 64), torch.bfloat16, (None,) * 4),
+    ((1, 3, 203, 32), torch.bfloat16, (None,) * 4),
+    ((1, 2, 160, 128), torch.float16, (None,) * 4),
+    ((2, 2, 300, 64), torch.bfloat16, (100, 64, 33, 16)),   # windowed streaming kernel
+    ((2, 2, 300, 64), torch.bfloat16, (24, 22, None, None)),  # band-resident kernel
+    ((1, 2, 96, 32), torch.float32, (None,) * 4),           # fp32 tensors: gathered, then the dense kernels
+    ((1, 2, 64, 16), torch.bfloat16, (None,) * 4),          # no matrix-core kernel at D = 16: gathered
+])
+def test_triple_dot_on_slices_of_a_fused_projection(shape, dtype, windows):
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    print(f"case strided triple-dot {shape} {dtype} {windows}", flush=True)
+    B, H, T, D = shape
+    views, _ = fused_views(B, H, T, D, dtype, seed=T)
+    assert not any(v.is_contiguous() for v in views)
+    d_o = bthd_view(B, H, T, D, dtype, seed=T + 1)
+    alpha = 1 / math.sqrt(D)
+    kw = dict(softmax_scale=alpha, k1_window=windows[0], k2_window=windows[1], kk_left=windows[2], kk_right=windows[3],
+              causal=True)
+
+    def run(tensors, grad):
+        leaves = [t.detach().requires_grad_(True) for t in tensors]
+        out = flash_trittention(*leaves, **kw)
+        out.backward(grad)
+        return out.detach(), [t.grad for t in leaves]
+
+    out_s, g_s = run(views, d_o)
+    out_d, g_d = run([v.contiguous() for v in views], d_o.contiguous())
+    torch.cuda.synchronize()
+    assert out_s.is_contiguous() and all(g.shape == (B, H, T, D) for g in g_s)
+    assert torch.equal(out_s, out_d)
+    for name, a, b in zip(util.NAMES, g_s, g_d):
+        assert torch.equal(a, b), name
+
+    inputs = dense_inputs(views, d_o)
+    z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
+    tol = FP32 if dtype == torch.float32 else LOWP
+    util.assert_mostly_close("out", out_s.float().cpu(), z, **tol)
+    for name, a, b in zip(util.NAMES, g_s, grads):
+        util.assert_mostly_close(name, a.float().cpu(), b, **tol)
+
+
+@pytest.mark.parametrize("shape,dtype", [((2, 4, 192, 64), torch.bfloat16), ((1, 2, 100, 32), torch.float16),
+                                         ((2, 2, 64, 32), torch.float32), ((1, 2, 130, 128), torch.bfloat16)])
+def test_dot_product_sum_on_transposed_projections(shape, dtype):
+    """All five inputs and dO as [B,T,H,D] tensors transposed (the layout tests/test_dot_product_sum.py:121-134 of the
+    reference feeds for K1 and K2)."""
+    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
+
+    print(f"case strided dot-product-sum {shape} {dtype}", flush=True)
+    B, H, T, D = shape
+    views = [bthd_view(B, H, T, D, dtype, seed=10 * T + i) for i in range(5)]
+    d_o = bthd_view(B, H, T, D, dtype, seed=10 * T + 5)
+    module = TrittentionTriton(causal=True, softmax_scale=1 / 8, k_diff=T // 2)
+
+    def run(tensors, grad):
+        leaves = [t.detach().requires_grad_(True) for t in tensors]
+        out, m = module(*leaves)
+        out.backward(grad)
+        return out.detach(), m.detach(), [t.grad for t in leaves]
+
+    out_s, m_s, g_s = run(views, d_o)
+    out_d, m_d, g_d = run([v.contiguous() for v in views], d_o.contiguous())
+    torch.cuda.synchronize()
+    assert torch.equal(out_s, out_d) and torch.equal(m_s, m_d)
+    for name, a, b in zip(util.NAMES, g_s, g_d):
+        assert torch.equal(a, b), name
+    z, _, grads = util.oracle_dps(dense_inputs(views, d_o), 1 / 8, True, T // 2)
+    tol = FP32 if dtype == torch.float32 else LOWP
+    util.assert_mostly_close("out", out_s.float().cpu(), z, **tol)
+    for name, a, b in zip(util.NAMES, g_s, grads):
+        util.assert_mostly_close(name, a.float().cpu(), b, **tol)
+
+
+def test_triple_dot_forward_reads_the_views_in_place():
+    """The 16-bit matrix-core forward takes five slices of a fused tensor without a copy: its workspace is the dense
+    call's, and the peak of device memory over the call is the outputs plus that workspace."""
+    from flash_trittention import _lib, _ops
+
+    B, H, T, D = 2, 8, 512, 64
+    views, fused = fused_views(B, H, T, D, torch.bfloat16, seed=3)
+    lay = _lib.layouts(views)
+    assert lay is not None and all(_lib.viewable(v) for v in views)
+    args = (B, H, T, D, _lib.TRITT_BF16, 1, T, T, T, T, 0)
+    plain = _lib.lib().tritt_tdp_fwd_workspace_bytes(*args)
+    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, lay) == (plain + 255) // 256 * 256
+    # four equal layouts and a dense V1 still need no copy; K2 on a layout of its own makes all five be gathered
+    mixed = [views[0], views[1], views[2], views[3].contiguous(), views[4]]
+    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(mixed)) == (plain + 255) // 256 * 256
+    odd = [views[0], views[1], bthd_view(B, H, T, D, torch.bfloat16, 4), views[3], views[4]]
+    n_bytes = B * H * T * D * 2
+    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(odd)) == \
+        (plain + 255) // 256 * 256 + 5 * n_bytes
+
+    _ops.tdp_fwd_impl(*views, 1 / 8, True, T, T, T, T, 0)  # first call: kernel attributes, allocator pools
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    o, lse = _ops.tdp_fwd_impl(*views, 1 / 8, True, T, T, T, T, 0)
+    torch.cuda.synchronize()
+    grown = torch.cuda.max_memory_allocated() - before
+    outputs = o.numel() * 2 + lse.numel() * 4
+    assert grown <= outputs + plain + 4096, (grown, outputs, plain)  # one input copy would add n_bytes = 1 MiB
+    assert grown < outputs + plain + n_bytes // 2
+    o_d, lse_d = _ops.tdp_fwd_impl(*(v.contiguous() for v in views), 1 / 8, True, T, T, T, T, 0)
+    assert torch.equal(o, o_d) and torch.equal(lse, lse_d)
+    del fused
+
+
+def test_split_operands_and_static_layout_cases():
+    """convert_to_float32 (split operands) on strided views; extent-1 dimensions with arbitrary strides; a broadcast
+    (stride 0) head dimension."""
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    B, H, T, D = 1, 2, 128, 64
+    views, _ = fused_views(B, H, T, D, torch.bfloat16, seed=9)
+    a = flash_trittention(*views, softmax_scale=1 / 8, k1_window=None, k2_window=None, kk_left=None, kk_right=None,
+                          causal=True, convert_to_float32=True)
+    b = flash_trittention(*(v.contiguous() for v in views), softmax_scale=1 / 8, k1_window=None, k2_window=None,
+                          kk_left=None, kk_right=None, causal=True, convert_to_float32=True)
+    assert torch.equal(a, b)
+    # one head broadcast to two: stride_h = 0
+    base = [torch.randn(1, 1, T, D, generator=torch.Generator().manual_seed(i)).bfloat16().cuda() for i in range(5)]
+    wide = [t.expand(1, 2, T, D) for t in base]
+    a = flash_trittention(*wide, softmax_scale=1 / 8, k1_window=None, k2_window=None, kk_left=None, kk_right=None)
+    b = flash_trittention(*(t.contiguous() for t in wide), softmax_scale=1 / 8, k1_window=None, k2_window=None,
+                          kk_left=None, kk_right=None)
+    assert torch.equal(a, b) and torch.equal(a[:, 0], a[:, 1])
+
+
+def test_layouts_the_library_refuses():
+    """Strides that would break the 16-byte pieces are an error at the C ABI (the Python front copies such views
+    first, as the reference copies every view)."""
+    from flash_trittention import _lib
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+
+    B, H, T, D = 1, 2, 64, 32
+    g = torch.Generator().manual_seed(0)
+    big = torch.randn(B, H, T, D + 4, generator=g).bfloat16().cuda()
+    odd = big[..., :D]  # row stride 36 elements: not a multiple of 16 bytes
+    assert not _lib.viewable(odd)
+    dense = [torch.randn(B, H, T, D, generator=g).bfloat16().cuda() for _ in range(4)]
+    out = flash_trittention(odd, *dense)
+    assert torch.equal(out, flash_trittention(odd.contiguous(), *dense))
+
+    lay = (_lib.Layout * 5)()
+    for slot in lay:
+        slot.stride_b, slot.stride_h, slot.stride_t = H * T * D, T * D, D
+    lay[0].stride_t = D + 4
+    o = torch.empty(B, H, T, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, T, dtype=torch.float32, device="cuda")
+    ws = torch.empty(1 << 22, dtype=torch.uint8, device="cuda")
+    ptrs = [_lib.ptr(t) for t in (odd, *dense)]
+    st = _lib.lib().tritt_tdp_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125, 1,
+                                          T, T, T, T, _lib.ptr(ws), ws.numel(), 0, _lib.stream_ptr(o.device))
+    assert st == -1  # TRITT_ERR_INVALID
+    lay[0].stride_t = -D
+    st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125, 1,
+                                          T, _lib.ptr(ws), ws.numel(), 0, _lib.stream_ptr(o.device))
+    assert st == -1
+    # too small a workspace for the gathered copies
+    lay[0].stride_t = 2 * D
+    need = _lib.lib().tritt_dps_fwd_strided_workspace_bytes(B, H, T, D, _lib.TRITT_BF16, 0, lay)
+    plain = _lib.lib().tritt_dps_fwd_workspace_bytes(B, H, T, D, _lib.TRITT_BF16, 0)
+    assert need == (plain + 255) // 256 * 256 + B * H * T * D * 2
+    wide = torch.randn(B, H, T, 2 * D, generator=g).bfloat16().cuda()
+    ptrs[0] = _lib.ptr(wide)
+    st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125, 1,
+                                          T, _lib.ptr(ws), need - 1, 0, _lib.stream_ptr(o.device))
+    assert st == -3  # TRITT_ERR_WORKSPACE
+    st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125, 1,
+                                          T, _lib.ptr(ws), need, 0, _lib.stream_ptr(o.device))
+    assert st == 0
+    torch.cuda.synchronize()
