@@ -24,6 +24,7 @@ for _p in (ROOT, os.path.join(ROOT, "flash-3-way-attention_amd")):
         sys.path.insert(0, _p)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3   # dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0
 NOMINAL_CLOCK_MHZ = 2400.0  # the clock behind the published peak
 # HBM bytes per launch, NOT measured live: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script at the
@@ -198,14 +199,17 @@ def sweep_rows(torch, flash_trittention, dev, steps):
     return rows
 
 
-def dps_times(torch, dev, B, H, T, D, steps, warmup):
-    """BASELINE config 4: dot-product-sum forward and backward (events around the Python calls)."""
+def dps_times(torch, dev, B, H, T, D, steps, warmup, dtype=None, k_diff=None):
+    """Dot-product-sum forward and backward (events around the Python calls): BASELINE config 4 by default; `dtype`
+    and `k_diff` for the reference's own large configurations (scripts/benchmark_dot_product_sum.py:400-510)."""
     from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
 
+    dtype = dtype or torch.bfloat16
+    k_diff = T if k_diff is None else min(k_diff, T)
     alpha = 1 / math.sqrt(D)
-    ins = [t.to(dev) for t in make_inputs(B, H, T, D, torch.bfloat16, seed=0)]
+    ins = [t.to(dev) for t in make_inputs(B, H, T, D, dtype, seed=0)]
     lv = [t.clone().requires_grad_(True) for t in ins[:5]]
-    mod = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=T)
+    mod = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=k_diff)
     hold = {}
 
     def f():
@@ -216,20 +220,29 @@ def dps_times(torch, dev, B, H, T, D, steps, warmup):
 
     ms_f = time_events(f, steps, max(warmup, 3), torch)
     ms_b = time_events(b, steps, max(warmup, 3), torch)  # the first backward pays one-time set-up
-    n3 = B * H * T * (T + 1) * (T + 2) // 6   # valid (q,s,t) triples of the reference's formulation
-    n2 = B * H * T * (T + 1) // 2              # (row, column) pairs of the factorised one
-    bytes_f, bytes_b = 6 * B * H * T * D * 2 + 4 * B * H * T, 12 * B * H * T * D * 2 + 8 * B * H * T
-    return {"fwd_ms": ms_f, "bwd_ms": ms_b,
-            "executed_fwd_tflops": 8 * D * n2 / ms_f / 1e9, "executed_bwd_tflops": 20 * D * n2 / ms_b / 1e9,
-            "reference_formulation_fwd_tflops_equiv": 4 * D * n3 / ms_f / 1e9,
-            "algorithmic_bytes_fwd": bytes_f, "algorithmic_bytes_bwd": bytes_b,
-            "io_gbs_fwd": bytes_f / ms_f / 1e6, "io_gbs_bwd": bytes_b / ms_b / 1e6,
-            # the factorised path is bound by HBM (8.6 / 21.5 GFLOP on 25 / 50 MB): fraction of the 8 TB/s floor
-            "roofline_fwd": {"bound": "hbm", "achieved": bytes_f / ms_f / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": bytes_f / ms_f / 1e6 / PEAK_HBM_GBS},
-            "roofline_bwd": {"bound": "hbm", "achieved": bytes_b / ms_b / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": bytes_b / ms_b / 1e6 / PEAK_HBM_GBS},
-            "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} bf16 causal"}}
+    n3 = B * H * T * (T + 1) * (T + 2) // 6   # valid (q,s,t) triples of the reference's formulation, k_diff = T
+    # (row, column) pairs of the factorised form: the inner attention (t, s) with t - s <= k_diff, the outer (q, t)
+    n_in = B * H * sum(min(t + 1, k_diff + 1) for t in range(T))
+    n_out = B * H * T * (T + 1) // 2
+    elem = 4 if dtype == torch.float32 else 2
+    peak = PEAK_F32_TFLOPS if dtype == torch.float32 else PEAK_BF16_TFLOPS
+    bytes_f, bytes_b = 6 * B * H * T * D * elem + 4 * B * H * T, 12 * B * H * T * D * elem + 8 * B * H * T
+    tf_f, tf_b = 4 * D * (n_in + n_out) / ms_f / 1e9, 10 * D * (n_in + n_out) / ms_b / 1e9
+    row = {"fwd_ms": ms_f, "bwd_ms": ms_b,
+           "executed_fwd_tflops": tf_f, "executed_bwd_tflops": tf_b,
+           "mfma_frac_fwd": tf_f / peak, "mfma_frac_bwd": tf_b / peak,
+           "algorithmic_bytes_fwd": bytes_f, "algorithmic_bytes_bwd": bytes_b,
+           "io_gbs_fwd": bytes_f / ms_f / 1e6, "io_gbs_bwd": bytes_b / ms_b / 1e6,
+           # the factorised path is bound by HBM (8.6 / 21.5 GFLOP on 25 / 50 MB): fraction of the 8 TB/s floor
+           "roofline_fwd": {"bound": "hbm", "achieved": bytes_f / ms_f / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                            "frac": bytes_f / ms_f / 1e6 / PEAK_HBM_GBS},
+           "roofline_bwd": {"bound": "hbm", "achieved": bytes_b / ms_b / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                            "frac": bytes_b / ms_b / 1e6 / PEAK_HBM_GBS},
+           "config": {"workload": f"dot-product-sum fwd+bwd B={B} H={H} T={T} D={D} {str(dtype).split('.')[-1]} causal "
+                                  f"k_diff={k_diff}"}}
+    if k_diff >= T:
+        row["reference_formulation_fwd_tflops_equiv"] = 4 * D * n3 / ms_f / 1e9
+    return row
 
 
 def tdp_times(torch, flash_trittention, dev, B, H, T, D, dtype, steps, warmup, backward=True, convert=False):
@@ -268,7 +281,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--brief", action="store_true", help="default mode: skip the other BASELINE configurations")
-    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "seqlen", "dps", "tdp", "published"], default="both",
+    ap.add_argument("--mode", choices=["both", "fwd", "copy", "sweep", "seqlen", "dps", "dpsrange", "tdp", "published"], default="both",
                     help="fwd: time only the forward (for profiling runs); copy: a plain 256 MiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated against; "
                          "sweep: triple-dot forward at B=1 H=16 D=128 bf16 over T in 512..4096; "
@@ -276,6 +289,9 @@ def main():
                          "11-31,177: B=2 H=2 D=64, k1_window 24, k2_window 22, T = 256..2048 step 256, forward and "
                          "backward, convert_to_float32=True), fp32 tensors as there and bf16; "
                          "dps: dot-product-sum forward+backward at --B --H --T --D; "
+                         "dpsrange: the large configurations of the reference's dot-product-sum benchmark "
+                         "(scripts/benchmark_dot_product_sum.py:400-510: B=1 H=8 D=64, T = 1024..8192, k_diff 128 / 1024 / "
+                         "2048, fp32 and bf16); "
                          "tdp: triple-dot forward+backward at --B --H --T --D with --windows (secondary shapes: "
                          "D=128, windowed masks); "
                          "published: the forward cases the reference publishes timings for (B=2 H=8 D=64 fp16 causal: "
@@ -364,6 +380,18 @@ def main():
                          "speedup_vs_best_published": min(h100_ms, b200_ms) / ms})
         print(json.dumps({"metric": "triple-dot trittention fwd ms on the reference's published cases", "unit": "ms",
                           "config": {"workload": "triple-dot fwd B=2 H=8 D=64 fp16 causal"}, "rows": rows}), flush=True)
+        return
+    if args.mode == "dpsrange":
+        rows = []
+        for dtype in (torch.float32, torch.bfloat16):
+            for Ts, kd in ((1024, None), (2048, 1024), (2048, 128), (4096, 2048), (4096, 128), (8192, 2048), (8192, 128)):
+                r = dps_times(torch, dev, 1, 8, Ts, 64, 10, 3, dtype=dtype, k_diff=kd)
+                rows.append({"dtype": str(dtype).split(".")[-1], "T": Ts, "k_diff": kd or Ts,
+                             **{k: r[k] for k in ("fwd_ms", "bwd_ms", "executed_fwd_tflops", "executed_bwd_tflops",
+                                                  "mfma_frac_fwd", "mfma_frac_bwd", "io_gbs_fwd", "io_gbs_bwd")}})
+        print(json.dumps({"metric": "dot-product-sum trittention fwd / bwd ms", "unit": "ms",
+                          "config": {"workload": "dot-product-sum fwd+bwd B=1 H=8 D=64 causal, T=1024..8192"},
+                          "rows": rows}), flush=True)
         return
     if args.mode == "dps":
         r = dps_times(torch, dev, B, H, T, D, args.steps, args.warmup)

@@ -76,8 +76,9 @@ __device__ __forceinline__ constexpr float fast_row_sum_floor() {
 // through the general (per tile, element-wise masked) loop, and the CAREFUL sweep tolerates rows whose
 // first valid key comes late.
 // MDIAG (NT = 1 only): the stages on the causal diagonal run the interleaved loop too, masked through the C
-// operand, instead of the general loop.  Pays on short sequences, where those stages are a large share of the
-// work; costs registers (a few more scratch reloads at D = 128), so long sequences keep the general loop.
+// operand, instead of the general loop.  Not instantiated: at D = 128 it needs 40 bytes of scratch per lane and
+// measures no faster where the diagonal is the largest share of the work (B=1 H=16 bf16: T=512 0.492 ms against
+// 0.489 ms with the general loop, T=768 1.334 against 1.323).
 // SPLIT: the B operand of the score product, alpha log2e Q[q] (.) K2[k], is a product of two 16-bit numbers and a
 // scale: rounded to one 16-bit operand it loses half its bits, and scores that span hundreds then differ from the
 // exact ones by more than the softmax can absorb.  SPLIT keeps it as hi + lo (hi = the rounded product, lo = the
@@ -1037,9 +1038,6 @@ size_t mfma_tdp_fwd_workspace(const MfmaFwdArgs& a) {
 bool mfma_tdp_fwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
 bool mfma_tdp_split_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64); }
 
-// D = 128: sequences up to this length run the diagonal stages in the interleaved loop (MDIAG)
-constexpr int kMaskedDiagonalUpTo = 768;
-
 template <typename E>
 static hipError_t launch_split(const MfmaFwdArgs& a, hipStream_t st) {
     if (a.windowed) {
@@ -1083,15 +1081,11 @@ hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st) {
     if (a.is_bf16) {
         if (a.D == 32) return launch<__bf16, 32, 1, 8, 2, 64>(a, st);
         if (a.D == 64) return launch<__bf16, 64, 2, 8, 2, 64>(a, st);
-        if (a.D == 128)
-            return a.T <= kMaskedDiagonalUpTo ? launch<__bf16, 128, 1, 8, 2, 64, false, true>(a, st)
-                                               : launch<__bf16, 128, 1, 8, 2, 64>(a, st);
+        if (a.D == 128) return launch<__bf16, 128, 1, 8, 2, 64>(a, st);
     } else {
         if (a.D == 32) return launch<_Float16, 32, 1, 8, 2, 64>(a, st);
         if (a.D == 64) return launch<_Float16, 64, 2, 8, 2, 64>(a, st);
-        if (a.D == 128)
-            return a.T <= kMaskedDiagonalUpTo ? launch<_Float16, 128, 1, 8, 2, 64, false, true>(a, st)
-                                               : launch<_Float16, 128, 1, 8, 2, 64>(a, st);
+        if (a.D == 128) return launch<_Float16, 128, 1, 8, 2, 64>(a, st);
     }
     return hipErrorInvalidValue;
 }
