@@ -96,6 +96,31 @@ __device__ __forceinline__ void transpose_store(E* __restrict__ dst, const E* ti
     }
 }
 
+// ---- XCD-aware order of a one-dimensional grid over (batch*head slice, tile) pairs -------------------------------
+// Consecutive workgroup ids go to different XCDs (eight of them, each with its own L2), so workgroup id b works for
+// XCD b % 8 and slot b / 8 of that XCD's list.  Whole groups of eight slices give every XCD its own slices (their keys
+// and values stay in that XCD's L2), tiles in launch order 0 .. ntiles - 1 (callers map order 0 to their heaviest tile).
+// The B*H % 8 slices left over would keep only some XCDs busy (B*H = 4: half the chip), so their (slice, tile) pairs are
+// dealt out over all eight XCDs instead, ahead of the whole groups (their light tiles then overlap the groups' heavy
+// ones; the end of the grid is light tiles either way).  xcd_slots = list length per XCD = grid size / 8.
+__host__ __device__ inline int xcd_slots(int BH, int ntiles) {
+    return (BH >> 3) * ntiles + (((BH & 7) * ntiles + 7) >> 3);
+}
+// false: a padding workgroup (the left-over pairs do not fill the last slot of every XCD)
+__device__ __forceinline__ bool xcd_tile(int BH, int ntiles, int slot, int xcd, int& bh, int& order) {
+    const int gf = BH >> 3, r = BH & 7, rem_slots = (r * ntiles + 7) >> 3;
+    if (slot < rem_slots) {
+        const int idx = slot * 8 + xcd;
+        bh = gf * 8 + idx % r;
+        order = idx / r;
+        return idx < r * ntiles;
+    }
+    slot -= rem_slots;
+    bh = (slot % gf) * 8 + xcd;
+    order = slot / gf;
+    return true;
+}
+
 // ---- 64-bit fixed-point gradient accumulators (backward kernels whose workgroups add shares of one gradient
 // element to a common sum; integer addition is associative, so the sums do not depend on the order of arrival).
 // The scale is a power of two chosen per (batch, head) slice from the largest finite |dO| of that slice,

@@ -40,16 +40,14 @@ __device__ __forceinline__ int row_of_key(int k) {
     const int i = 8 * (k >> 4) + (k & 7), g = (k >> 3) & 1;
     return ((i >> 2) << 3) | (g << 2) | (i & 3);
 }
-// XCD-aware block order of a 1-D grid of 8 * ceil(BH / 8) * ntiles workgroups: consecutive block ids go to
-// different XCDs, so every XCD gets its own (batch, head) slices and their packed operands stay in that
-// XCD's L2.  `tile` counts 0 .. ntiles-1 in launch order.  False: a padding block (BH not a multiple of 8).
-__device__ __forceinline__ bool block_to_tile(int BH, int& bh, int& tile) {
-    const int groups = (BH + 7) / 8;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    bh = (slot % groups) * 8 + xcd;
-    tile = slot / groups;
-    return bh < BH;
+// XCD-aware block order of a 1-D grid of 8 * xcd_slots(BH, ntiles) workgroups (common.hpp): every XCD gets its own
+// (batch, head) slices and their packed operands stay in that XCD's L2.  `tile` counts 0 .. ntiles-1 in launch order.
+// False: a padding block.
+__device__ __forceinline__ bool block_to_tile(int BH, int ntiles, int& bh, int& tile) {
+    return xcd_tile(BH, ntiles, blockIdx.x >> 3, blockIdx.x & 7, bh, tile);
 }
+// owner tiles a launch of the attention kernels hands out (paired: a long and a short one per workgroup)
+__device__ __forceinline__ int launch_tiles(int pair, int nt) { return pair ? (nt + 1) / 2 : nt; }
 
 // Under a full causal mask the owner tiles of a launch are a triangle: the longest walks nt streamed tiles, the
 // shortest one, and with one tile per workgroup the launch lasts as long as its longest tile while most SIMDs
@@ -144,7 +142,7 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     float* sL = sM + kW * 32;                        // [kW][32]
 
     int bh, tile0;
-    if (!block_to_tile(p.BH, bh, tile0)) return;
+    if (!block_to_tile(p.BH, launch_tiles(p.pair, p.Tp / 32), bh, tile0)) return;
     const int nparts = owner_tiles(p.pair, p.Tp / 32, tile0);
     for (int op = 0; op < nparts; ++op) {
     if (op) __syncthreads();  // the merge tiles of the first owner tile have been read
@@ -371,7 +369,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
     float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
 
     int bh, tile0;
-    if (!block_to_tile(p.BH, bh, tile0)) return;
+    if (!block_to_tile(p.BH, launch_tiles(p.pair, p.Tp / 32), bh, tile0)) return;
     const int nparts = owner_tiles(p.pair, p.Tp / 32, tile0);
     for (int op = 0; op < nparts; ++op) {
     if (op) __syncthreads();  // the merge tiles of the first owner tile have been read
@@ -515,7 +513,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> 
     float* sR = sB + kW * 32;                        // [2 kW][32]   delta1 partials
 
     int bh, tile0;
-    if (!block_to_tile(p.BH, bh, tile0)) return;
+    if (!block_to_tile(p.BH, launch_tiles(p.pair, p.Tp / 32), bh, tile0)) return;
     const int nparts = owner_tiles(p.pair, p.Tp / 32, tile0);
     for (int op = 0; op < nparts; ++op) {
     if (op) __syncthreads();  // the merge tiles of the first owner tile have been read
@@ -757,7 +755,7 @@ template <typename E, int D>
 __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
     using v8 = typename Mma<E>::v8;
     int bh, tile_id;
-    if (!block_to_tile(p.BH, bh, tile_id)) return;
+    if (!block_to_tile(p.BH, p.Tp / 32, bh, tile_id)) return;
     const int j0 = tile_id * 32, T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp;
     // One 16-byte piece (8 consecutive d of one row) per thread and step: it is one piece of P1 as it stands.
@@ -890,7 +888,7 @@ bool pair_tiles(const MfmaDpsArgs& a, int k_diff, int workgroups, bool backward)
 }
 dim3 attn_grid(const MfmaDpsArgs& a, int Tp, bool pair) {
     const int nt = Tp / 32;
-    return dim3(8 * ((a.BH + 7) / 8) * (pair ? (nt + 1) / 2 : nt));
+    return dim3(8 * xcd_slots(a.BH, pair ? (nt + 1) / 2 : nt));
 }
 
 template <typename E, int D, int kW>
@@ -898,7 +896,7 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, for_bwd);
     char* ws = static_cast<char*>(a.workspace);
-    const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
+    const dim3 grid(8 * xcd_slots(a.BH, Tp / 32));
     const bool pair_in = pair_tiles(a, a.k_diff, grid.x, for_bwd), pair_out = pair_tiles(a, a.T, grid.x, for_bwd);
     auto kern = attn_fwd_mfma_kernel<E, D, kW>;
     hipError_t e = allow_smem(kern, fwd_smem<D, kW>());
@@ -937,7 +935,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, true);
     char* ws = static_cast<char*>(a.workspace);
-    const dim3 grid(8 * ((a.BH + 7) / 8) * (Tp / 32));
+    const dim3 grid(8 * xcd_slots(a.BH, Tp / 32));
     const bool pair_in = pair_tiles(a, a.k_diff, grid.x, true), pair_out = pair_tiles(a, a.T, grid.x, true);
     auto krow = attn_bwd_row_mfma_kernel<E, D, kW>;
     auto kcol_link = attn_bwd_col_mfma_kernel<E, D, kW, true>;

@@ -46,6 +46,7 @@ struct BwdParams {
     unsigned* poison;             // [BH][T]
     unsigned bit_k, bit_v;        // poison bits of acc_k / acc_v
     int T, Tp, BH, nqt;
+    int grid_tiles;  // query tiles the grid covers (nqt - 1 .. nqt - grid_tiles: tile 0 may be left to the fp32 kernel)
     float alpha;
     int causal;
     // windowed kernels only, in terms of the streamed index a and the row index b: (q, a, b) takes part
@@ -123,14 +124,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     E* sQe = reinterpret_cast<E*>(sOb + BQ * LDQ + (NW / 2) * (BQ * D));
     E* sOe = sQe + DT * 64 * 16;
 
-    const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7;
     int slot = blockIdx.x >> 3;
     const int split = slot % p.splits;  // which share of the tile's rounds this workgroup walks (small grids)
     slot /= p.splits;
-    const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
-    if (bh >= p.BH) return;
+    int bh, order;
+    if (!xcd_tile(p.BH, p.grid_tiles, slot, xcd, bh, order)) return;
+    const int qt = p.nqt - 1 - order;  // heaviest query tiles first
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -746,8 +746,8 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         if (hipError_t e = f32_mfma_tdp_bwd_first_tile(f, st); e != hipSuccess) return e;
     }
     const int tiles_here = all_in_f32 ? 0 : p.nqt - (first_in_f32 ? 1 : 0);
-    const int groups = (a.BH + 7) / 8;
-    const dim3 grid(8 * groups * std::max(tiles_here, 1) * col_parts * p.splits);
+    p.grid_tiles = std::max(tiles_here, 1);  // the tiles the grid covers: nqt - 1 .. nqt - grid_tiles
+    const dim3 grid(8 * xcd_slots(a.BH, p.grid_tiles) * col_parts * p.splits);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;

@@ -109,7 +109,6 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     E* sQe = reinterpret_cast<E*>(sDQall + (WITH_DQ ? (NW / 2) * (BQ * DH) : 0));  // [DT][64][16] (EPI_TILES)
     E* sOe = sQe + DT * 64 * 16;
 
-    const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7;
     int slot = blockIdx.x >> 3;
     int c0 = 0;  // first gradient column of this workgroup
@@ -119,9 +118,9 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     }
     const int split = slot % p.splits;  // which share of the tile's rows (rounds) this workgroup walks
     slot /= p.splits;
-    const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
-    if (bh >= p.BH) return;
+    int bh, order;
+    if (!xcd_tile(p.BH, p.grid_tiles, slot, xcd, bh, order)) return;
+    const int qt = p.nqt - 1 - order;  // heaviest query tiles first
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -84,14 +84,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     E* sQb = sVr + 2 * RPR * D;              // [BQ][LDK]
     E* sOb = sQb + BQ * LDK;
 
-    const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7;
     int slot = blockIdx.x >> 3;
     const int split = slot % p.splits;  // which share of the tile's rounds this workgroup walks
     slot /= p.splits;
-    const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
-    if (bh >= p.BH) return;
+    int bh, order;
+    if (!xcd_tile(p.BH, p.grid_tiles, slot, xcd, bh, order)) return;
+    const int qt = p.nqt - 1 - order;  // heaviest query tiles first
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, grp = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

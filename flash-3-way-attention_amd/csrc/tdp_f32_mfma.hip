@@ -124,11 +124,9 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
     float* sL = sM + NW * 32;           // [NW][32]
     float* sO = sK;                     // [D][33]     end of kernel: merged output (aliases the stages)
 
-    const int groups = (p.BH + 7) / 8;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;  // heaviest query tiles first
-    if (bh >= p.BH) return;
+    int bh, order;
+    if (!xcd_tile(p.BH, p.nqt, blockIdx.x >> 3, blockIdx.x & 7, bh, order)) return;
+    const int qt = p.nqt - 1 - order;  // heaviest query tiles first
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -388,12 +386,10 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
     float* sVb = sKb + NW * D;          // [NW][D]
     float* sO = sK;                     // [DOUT][33]   end of kernel: dQ of the tile (aliases the stages)
 
-    const int groups = (p.BH + 7) / 8;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;
+    int bh, order;
+    if (!xcd_tile(p.BH, p.nqt, blockIdx.x >> 3, blockIdx.x & 7, bh, order)) return;
+    const int qt = p.nqt - 1 - order;
     const int c0 = blockIdx.y * DOUT;  // first gradient column of this workgroup
-    if (bh >= p.BH) return;
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -663,10 +659,9 @@ hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, cons
     static_assert(DOUT * 33 <= 4 * 32 * (D + 1), "dQ of the tile aliases the stage buffers");
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
-    const int groups = (p.BH + 7) / 8;
     // small grids: the rounds of a tile dealt out to several workgroups (the launch with dQ only when dQ has an accumulator)
     const int parts = std::max(1, p.round_parts);
-    const dim3 grid(8 * groups * p.nqt, D / DOUT, p.acc_q ? parts : 1), grid_nodq(8 * groups * p.nqt, D / DOUT_NODQ, parts);
+    const dim3 grid(8 * xcd_slots(p.BH, p.nqt), D / DOUT, p.acc_q ? parts : 1), grid_nodq(8 * xcd_slots(p.BH, p.nqt), D / DOUT_NODQ, parts);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.ka = k1; p.va = u; p.kb = k2; p.vb = v2;
     p.acc_k = acc_k2; p.acc_v = acc_v2; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
@@ -740,8 +735,7 @@ hipError_t launch_f32_fwd(const GenericTdpArgs& a, hipStream_t st) {
     constexpr size_t smem = f32_fwd_smem<D>();
     static_assert(D * 33 <= 4 * 32 * (D + 1), "the merged output aliases the stage buffers");
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
-    const int groups = (a.BH + 7) / 8;
-    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p);
+    hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, p.nqt)), dim3(512), smem, st, p);
     return hipGetLastError();
 }
 
@@ -770,7 +764,7 @@ static hipError_t launch_stats(const FirstTileArgs& a, hipStream_t st) {
     auto kern = tdp_f32_fwd_kernel<E, D, true>;
     constexpr size_t smem = f32_fwd_smem<D>();
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(8 * ((a.BH + 7) / 8) * p.nqt), dim3(512), smem, st, p);
+    hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, p.nqt)), dim3(512), smem, st, p);
     return hipGetLastError();
 }
 
@@ -795,7 +789,7 @@ static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
         auto kern = tdp_f32_fwd_kernel<E, D, true>;
         constexpr size_t smem = f32_fwd_smem<D>();
         if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3(8 * groups, rounds), dim3(512), smem, st, p);
+        hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, 1), rounds), dim3(512), smem, st, p);
     }
     F32BwdParams<E> r0{};
     r0.q = (const E*)a.q; r0.d_o = (const E*)a.d_o; r0.lse = nullptr; r0.delta = nullptr;
@@ -813,7 +807,7 @@ static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
     auto kern = tdp_f32_tile0_kernel<E, D, DOUT>;
     constexpr size_t smem = f32_bwd_smem<D>();
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(8 * groups, D / DOUT, 2 * rounds), dim3(512), smem, st, r0, r1, roles);
+    hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, 1), D / DOUT, 2 * rounds), dim3(512), smem, st, r0, r1, roles);
     return hipGetLastError();
 }
 

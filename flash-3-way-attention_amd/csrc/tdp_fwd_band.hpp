@@ -49,11 +49,9 @@ __global__ __launch_bounds__(512, 2) void tdp_fwd_band_kernel(FwdParams<E> p, in
     float* sW = sQ + kBandQ * D;                                // [8][32] per-wave scratch
     float* sTab = sW + 8 * 32;  // [5 slots][4][64 lanes][4]  band masks in the MFMA C layout; slot 4: zeros
 
-    const int groups = (p.BH + 7) / 8;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;
-    if (bh >= p.BH) return;
+    int bh, order;
+    if (!xcd_tile(p.BH, p.nqt, blockIdx.x >> 3, blockIdx.x & 7, bh, order)) return;
+    const int qt = p.nqt - 1 - order;
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

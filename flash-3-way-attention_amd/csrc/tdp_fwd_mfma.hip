@@ -118,14 +118,13 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     // heavy-first, XCD-aware block order: consecutive block ids go to different XCDs, so give
     // every XCD its own set of heads (their K/V stay in that XCD's L2) and hand out the
     // longest query tiles first.
-    const int groups = (p.BH + 7) / 8;
     const int xcd = blockIdx.x & 7;
     int slot = blockIdx.x >> 3;
     const int split = slot % p.splits;
     slot /= p.splits;
-    const int bh = (slot % groups) * 8 + xcd;
-    const int qt = p.nqt - 1 - slot / groups;
-    if (bh >= p.BH) return;
+    int bh, order;
+    if (!xcd_tile(p.BH, p.nqt, slot, xcd, bh, order)) return;
+    const int qt = p.nqt - 1 - order;
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it scalar
@@ -981,8 +980,7 @@ static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
     auto kern = tdp_fwd_band_kernel<E, D>;
     hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem);
     if (e != hipSuccess) return e;
-    const int groups = (a.BH + 7) / 8;
-    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt), dim3(512), smem, st, p, nr);
+    hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, p.nqt)), dim3(512), smem, st, p, nr);
     return hipGetLastError();
 }
 
@@ -1019,8 +1017,7 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS, SPLIT>();
     auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG, SPLIT>;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
-    const int groups = (a.BH + 7) / 8;
-    hipLaunchKernelGGL(kern, dim3(8 * groups * p.nqt * p.splits), dim3(64 * WAVES), smem, st, p);
+    hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, p.nqt) * p.splits), dim3(64 * WAVES), smem, st, p);
     if (p.splits > 1) {
         const int rows = a.BH * a.T;
         hipLaunchKernelGGL(fwd_merge_kernel<E>, dim3((unsigned)(((size_t)rows * D + 255) / 256)), dim3(256), 0, st,
