@@ -434,8 +434,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         if constexpr (WITH_DQ) {
             if (k <= jend && (wave & 1) == 0) add_dq();
         }
-        // all waves are done with this round's K2/V2 rows; the next round's have landed
-        barrier_keep_loads<LW + 4>();
+        // all waves are done with this round's K2/V2 rows; the next round's have landed: they are older than the newest
+        // stage's loads, the only ones allowed to stay in flight (a tile of a single stage issues both in its one step)
+        barrier_keep_loads<LW>();
         if constexpr (WITH_DQ) {
             if (k <= jend && (wave & 1) == 1) add_dq();
         }
