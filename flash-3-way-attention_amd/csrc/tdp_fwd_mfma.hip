@@ -964,7 +964,7 @@ static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
     const InLayout lin = input_layout(a, false), lv1 = input_layout(a, true);
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
-                       a.T, Tp, D, lin.H, lv1.sb, lv1.sh, lv1.st);
+                       a.T, Tp, D, lv1.H, lv1.sb, lv1.sh, lv1.st);
     FwdParams<E> p;
     p.q = (const E*)a.q; p.k1 = (const E*)a.k1; p.k2 = (const E*)a.k2; p.v2 = (const E*)a.v2;
     p.ut = (const E*)a.ut; p.o = (E*)a.o; p.lse = a.lse; p.o_res = nullptr;
@@ -1000,7 +1000,7 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + kTpad - 1) / kTpad * kTpad;
     const InLayout lin = input_layout(a, false), lv1 = input_layout(a, true);
     hipLaunchKernelGGL(silu_transpose_kernel<E>, dim3(Tp / 64, a.BH), dim3(256), 0, st, (const E*)a.v1, (E*)a.ut,
-                       a.T, Tp, D, lin.H, lv1.sb, lv1.sh, lv1.st);
+                       a.T, Tp, D, lv1.H, lv1.sb, lv1.sh, lv1.st);
     constexpr int BQ = WAVES * NT;
     if (BQ != fwd_tile_queries(D, a.windowed)) return hipErrorInvalidValue;  // the workspace was sized for another shape
     FwdParams<E> p;

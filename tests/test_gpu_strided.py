@@ -143,6 +143,14 @@ def test_triple_dot_forward_reads_the_views_in_place():
     assert grown < outputs + plain + n_bytes // 2
     o_d, lse_d = _ops.tdp_fwd_impl(*(v.contiguous() for v in views), 1 / 8, True, T, T, T, T, 0)
     assert torch.equal(o, o_d) and torch.equal(lse, lse_d)
+    # V1 on a layout of its own, either way round (its pass takes its own strides and head count)
+    o_m, lse_m = _ops.tdp_fwd_impl(*mixed, 1 / 8, True, T, T, T, T, 0)
+    assert torch.equal(o_m, o_d) and torch.equal(lse_m, lse_d)
+    only_v1 = [v.contiguous() for v in views]
+    only_v1[3] = views[3]
+    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(only_v1)) == (plain + 255) // 256 * 256
+    o_v, lse_v = _ops.tdp_fwd_impl(*only_v1, 1 / 8, True, T, T, T, T, 0)
+    assert torch.equal(o_v, o_d) and torch.equal(lse_v, lse_d)
     del fused
 
 
