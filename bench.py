@@ -31,11 +31,13 @@ NOMINAL_CLOCK_MHZ = 2400.0  # the clock behind the published peak
 # default workload only, scaled by a plain 256 MiB copy (summary and commands:
 # profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt).  Reported only when the workload is the default one.
 TRAFFIC_SOURCE = "profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt (rocprofv3 --pmc, default workload only)"
-TRAFFIC_FWD = 25.6e6        # 20.3 MiB fetched + 4.1 MiB written
-# average of the two launches: ~530 MiB written by 64-bit atomics each, 36 / 78 MiB fetched (some runs: up to 440 MiB in the first
+# 27.4 MiB fetched + 15.0 MiB written: the algorithmic 20 + 4 MiB, and 28 bytes per lane that the kernel's prologue
+# spills (a million lanes: ~11 MiB written once; spill-free builds of the kernel measured 2 % slower)
+TRAFFIC_FWD = 44.4e6
+# average of the two launches: ~530 MiB written by 64-bit atomics each, 34 / 40 MiB fetched (some runs: up to 440 MiB in the first
 # launch, when its accumulators fall out of their XCD's L2; the bytes are L2 <-> fabric traffic, which the 256 MB Infinity
 # Cache absorbs)
-TRAFFIC_BWD_ROWS = 614e6
+TRAFFIC_BWD_ROWS = 593e6
 
 
 def triples(B, H, T, causal=True):
@@ -297,7 +299,7 @@ def main():
                          "published: the forward cases the reference publishes timings for (B=2 H=8 D=64 fp16 causal: "
                          "T=256/512/1024 full windows, T=2048 windows 128,128,32,32), its best H100 / B200 figures beside ours")
     ap.add_argument("--windows", default="", help="k1_window,k2_window,kk_left,kk_right for --mode tdp (empty: full)")
-    ap.add_argument("--dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="tensor type for --mode tdp")
+    ap.add_argument("--dtype", choices=["bf16", "fp16", "fp32"], default="bf16", help="tensor type for --mode tdp and --mode dps")
     ap.add_argument("--convert", action="store_true", help="--mode tdp: pass convert_to_float32=True")
     ap.add_argument("--B", type=int, default=4)
     ap.add_argument("--H", type=int, default=8)
@@ -394,7 +396,8 @@ def main():
                           "rows": rows}), flush=True)
         return
     if args.mode == "dps":
-        r = dps_times(torch, dev, B, H, T, D, args.steps, args.warmup)
+        ddtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype]
+        r = dps_times(torch, dev, B, H, T, D, args.steps, args.warmup, dtype=ddtype)
         print(json.dumps({"metric": "dot-product-sum trittention fwd / bwd ms", "unit": "ms", **r}), flush=True)
         return
     tdtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[args.dtype if args.mode == "tdp" else "bf16"]
