@@ -36,26 +36,30 @@ def dense_inputs(views, d_o):
     return [t.detach().contiguous().cpu() for t in (*views, d_o)]
 
 
-@pytest.mark.parametrize("shape,dtype,windows", [
-    ((2, 4, 256, 64), torch.bfloat16, (None,) * 4),
-    ((1, 3, 203, 32), torch.bfloat16, (None,) * 4),
-    ((1, 2, 160, 128), torch.float16, (None,) * 4),
-    ((2, 2, 300, 64), torch.bfloat16, (100, 64, 33, 16)),   # windowed streaming kernel
-    ((2, 2, 300, 64), torch.bfloat16, (24, 22, None, None)),  # band-resident kernel
-    ((1, 2, 96, 32), torch.float32, (None,) * 4),           # fp32 tensors: gathered, then the dense kernels
-    ((1, 2, 64, 16), torch.bfloat16, (None,) * 4),          # no matrix-core kernel at D = 16: gathered
+@pytest.mark.parametrize("shape,dtype,windows,causal", [
+    ((2, 4, 256, 64), torch.bfloat16, (None,) * 4, True),
+    ((1, 3, 203, 32), torch.bfloat16, (None,) * 4, True),
+    ((1, 2, 160, 128), torch.float16, (None,) * 4, True),
+    ((2, 2, 300, 64), torch.bfloat16, (100, 64, 33, 16), True),   # windowed streaming kernel
+    ((2, 2, 300, 64), torch.bfloat16, (24, 22, None, None), True),  # band-resident kernel
+    ((1, 2, 96, 32), torch.float32, (None,) * 4, True),           # fp32 tensors: gathered, then the dense kernels
+    ((1, 2, 64, 16), torch.bfloat16, (None,) * 4, True),          # no matrix-core kernel at D = 16: gathered
+    ((2, 6, 64, 64), torch.bfloat16, (None,) * 4, False),         # no mask; twelve slices: one whole group of eight and four over
+    ((1, 5, 257, 128), torch.float16, (None,) * 4, False),
+    ((1, 3, 64, 128), torch.bfloat16, (40, 24, 300, 0), True),    # band-resident kernel at D = 128
+    ((1, 1, 100, 128), torch.float16, (None,) * 4, True),         # one batch, one head: both strides of extent-1 dimensions
 ])
-def test_triple_dot_on_slices_of_a_fused_projection(shape, dtype, windows):
+def test_triple_dot_on_slices_of_a_fused_projection(shape, dtype, windows, causal):
     from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
 
-    print(f"case strided triple-dot {shape} {dtype} {windows}", flush=True)
+    print(f"case strided triple-dot {shape} {dtype} {windows} causal={causal}", flush=True)
     B, H, T, D = shape
     views, _ = fused_views(B, H, T, D, dtype, seed=T)
     assert not any(v.is_contiguous() for v in views)
     d_o = bthd_view(B, H, T, D, dtype, seed=T + 1)
     alpha = 1 / math.sqrt(D)
     kw = dict(softmax_scale=alpha, k1_window=windows[0], k2_window=windows[1], kk_left=windows[2], kk_right=windows[3],
-              causal=True)
+              causal=causal)
 
     def run(tensors, grad):
         leaves = [t.detach().requires_grad_(True) for t in tensors]
@@ -72,25 +76,26 @@ def test_triple_dot_on_slices_of_a_fused_projection(shape, dtype, windows):
         assert torch.equal(a, b), name
 
     inputs = dense_inputs(views, d_o)
-    z, _, grads = util.oracle_tdp(inputs, alpha, True, windows)
+    z, _, grads = util.oracle_tdp(inputs, alpha, causal, windows)
     tol = FP32 if dtype == torch.float32 else LOWP
     util.assert_mostly_close("out", out_s.float().cpu(), z, **tol)
     for name, a, b in zip(util.NAMES, g_s, grads):
         util.assert_mostly_close(name, a.float().cpu(), b, **tol)
 
 
-@pytest.mark.parametrize("shape,dtype", [((2, 4, 192, 64), torch.bfloat16), ((1, 2, 100, 32), torch.float16),
-                                         ((2, 2, 64, 32), torch.float32), ((1, 2, 130, 128), torch.bfloat16)])
-def test_dot_product_sum_on_transposed_projections(shape, dtype):
+@pytest.mark.parametrize("shape,dtype,causal", [((2, 4, 192, 64), torch.bfloat16, True), ((1, 2, 100, 32), torch.float16, True),
+                                                ((2, 2, 64, 32), torch.float32, True), ((1, 2, 130, 128), torch.bfloat16, True),
+                                                ((2, 6, 257, 64), torch.float16, False), ((1, 1, 257, 64), torch.float16, True)])
+def test_dot_product_sum_on_transposed_projections(shape, dtype, causal):
     """All five inputs and dO as [B,T,H,D] tensors transposed (the layout tests/test_dot_product_sum.py:121-134 of the
     reference feeds for K1 and K2)."""
     from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
 
-    print(f"case strided dot-product-sum {shape} {dtype}", flush=True)
+    print(f"case strided dot-product-sum {shape} {dtype} causal={causal}", flush=True)
     B, H, T, D = shape
     views = [bthd_view(B, H, T, D, dtype, seed=10 * T + i) for i in range(5)]
     d_o = bthd_view(B, H, T, D, dtype, seed=10 * T + 5)
-    module = TrittentionTriton(causal=True, softmax_scale=1 / 8, k_diff=T // 2)
+    module = TrittentionTriton(causal=causal, softmax_scale=1 / 8, k_diff=T // 2)
 
     def run(tensors, grad):
         leaves = [t.detach().requires_grad_(True) for t in tensors]
@@ -104,7 +109,7 @@ def test_dot_product_sum_on_transposed_projections(shape, dtype):
     assert torch.equal(out_s, out_d) and torch.equal(m_s, m_d)
     for name, a, b in zip(util.NAMES, g_s, g_d):
         assert torch.equal(a, b), name
-    z, _, grads = util.oracle_dps(dense_inputs(views, d_o), 1 / 8, True, T // 2)
+    z, _, grads = util.oracle_dps(dense_inputs(views, d_o), 1 / 8, causal, T // 2)
     tol = FP32 if dtype == torch.float32 else LOWP
     util.assert_mostly_close("out", out_s.float().cpu(), z, **tol)
     for name, a, b in zip(util.NAMES, g_s, grads):
