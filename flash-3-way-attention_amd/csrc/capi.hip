@@ -33,7 +33,7 @@ Knobs knobs() {
     return Knobs{g_knobs[TRITT_TUNE_FWD_SPLITS].load(), g_knobs[TRITT_TUNE_FWD_BAND].load(),
                  g_knobs[TRITT_TUNE_BWD_SPLITS].load(), g_knobs[TRITT_TUNE_BWD128_WAVES].load(),
                  g_knobs[TRITT_TUNE_F32_VALU].load(), g_knobs[TRITT_TUNE_DPS_WAVES].load(),
-                 g_knobs[TRITT_TUNE_DPS_PAIR].load()};
+                 g_knobs[TRITT_TUNE_DPS_PAIR].load(), g_knobs[TRITT_TUNE_DPS_SHARED].load()};
 }
 
 hipError_t ensure_dynamic_smem(const void* kernel, size_t bytes) {

@@ -35,6 +35,15 @@ __device__ __forceinline__ void direct_load_16(const void* gbase, unsigned byte_
                  : "memory");
 }
 
+// the same with 4 bytes per lane: one instruction fills 256 consecutive bytes
+__device__ __forceinline__ void direct_load_4(const void* gbase, unsigned byte_off, void* lds_dst) {
+    const unsigned lds = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :
+                 : "s"(lds), "v"(byte_off), "s"(gbase)
+                 : "memory");
+}
+
 // make a wave-uniform pointer provably scalar (keeps it in SGPRs instead of spilled VGPR pairs)
 template <typename T>
 __device__ __forceinline__ const T* uniform_ptr(const T* p) {

@@ -28,6 +28,7 @@
 // element has one owner: no atomics, bitwise reproducible.
 #include "kernels.hpp"
 #include "mfma.hpp"
+#include "direct_lds.hpp"
 
 namespace tritt {
 namespace {
@@ -328,6 +329,8 @@ __global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     }
     }  // owner tiles of this workgroup
 }
+
+#include "dps_fwd_shared.hpp"
 
 // ------------------------------------------------------------------------------ backward, rows
 template <typename E>
@@ -919,14 +922,33 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     p.outm_p2 = (E*)(ws + l.wp2);
     p.lse = (float*)(ws + l.lse1); p.lse_stride = Tp; p.lse_scale = 1.0f;
     p.BH = a.BH; p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff; p.pair = pair_in;
-    hipLaunchKernelGGL(kern, attn_grid(a, Tp, pair_in), dim3(64 * kW), (fwd_smem<D, kW>()), st, p);
+    // Large grids take the kernel whose workgroups own 128 rows and share the streamed tiles through LDS
+    // (dps_fwd_shared.hpp).  One wave per 32 rows walks all streamed tiles of its rows, so the kernel needs four of
+    // its workgroups per CU to keep the SIMDs busy; measured forward, bf16 D = 64, one owner tile per workgroup ->
+    // shared tiles: B=8 H=16 T=2048 398 -> 282 us, B=4 H=8 T=4096 305 -> 262 us, but B=1 H=8 T=8192 (512 workgroups)
+    // 277 -> 391 us and B=4 H=8 T=1024 (256) 45 -> 70 us.
+    constexpr int kSW = 4, kNS = 4;  // its waves and ring slots
+    using Shared = FwdSharedShape<D, kSW, kNS>;
+    auto kern_in = attn_fwd_shared_kernel<E, D, kSW, kNS, false>;
+    auto kern_out = attn_fwd_shared_kernel<E, D, kSW, kNS, true>;
+    const int owners = (Tp / 32 + kSW - 1) / kSW;
+    const bool shared = knobs().dps_shared ? knobs().dps_shared > 0 : (long long)a.BH * owners >= 1024;
+    const dim3 grid_shared(8 * xcd_slots(a.BH, owners));
+    if (shared) {
+        if (e = allow_smem(kern_in, Shared::smem); e != hipSuccess) return e;
+        if (e = allow_smem(kern_out, Shared::smem); e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern_in, grid_shared, dim3(64 * kSW), Shared::smem, st, p);
+    } else {
+        hipLaunchKernelGGL(kern, attn_grid(a, Tp, pair_in), dim3(64 * kW), (fwd_smem<D, kW>()), st, p);
+    }
     if (for_bwd) return hipGetLastError();
     // outer: rows Q[q], keys K2 with bias lse1, values W; O and LSE (natural log)
     AttnFwdP<E> o{};
     o.x = (const E*)a.q; o.kp = (const E*)(ws + l.k2p1); o.vp2 = (const E*)(ws + l.wp2); o.bias = (const float*)(ws + l.lse1);
     o.out = (E*)a.o_out; o.lse = a.lse_out; o.lse_stride = a.T; o.lse_scale = kLn2;
     o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T; o.pair = pair_out;
-    hipLaunchKernelGGL(kern, attn_grid(a, Tp, pair_out), dim3(64 * kW), (fwd_smem<D, kW>()), st, o);
+    if (shared) hipLaunchKernelGGL(kern_out, grid_shared, dim3(64 * kSW), Shared::smem, st, o);
+    else hipLaunchKernelGGL(kern, attn_grid(a, Tp, pair_out), dim3(64 * kW), (fwd_smem<D, kW>()), st, o);
     return hipGetLastError();
 }
 

@@ -85,7 +85,8 @@ def exported_symbols():
     return list(_PROTOS)
 
 
-TUNE_FWD_SPLITS, TUNE_FWD_BAND, TUNE_BWD_SPLITS, TUNE_BWD128_WAVES, TUNE_F32_VALU, TUNE_DPS_WAVES, TUNE_DPS_PAIR = range(7)
+(TUNE_FWD_SPLITS, TUNE_FWD_BAND, TUNE_BWD_SPLITS, TUNE_BWD128_WAVES, TUNE_F32_VALU, TUNE_DPS_WAVES, TUNE_DPS_PAIR,
+ TUNE_DPS_SHARED) = range(8)
 
 
 def set_tuning(knob: int, value: int) -> int:

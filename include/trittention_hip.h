@@ -84,9 +84,12 @@ const char* tritt_status_string(int status);
  *                           fp32 MFMA kernels at D = 32, 64 and 128)
  *   TRITT_TUNE_DPS_WAVES    waves per workgroup of the dot-product-sum MFMA kernels at D = 64: 2 | 4
  *   TRITT_TUNE_DPS_PAIR     dot-product-sum MFMA kernels: 1 = a workgroup always takes two owner tiles (a long and a
- *                           short one), -1 = never */
+ *                           short one), -1 = never
+ *   TRITT_TUNE_DPS_SHARED   dot-product-sum forward passes: 1 = always the kernel whose workgroups own 128 rows and share
+ *                           the streamed tiles through LDS, -1 = never (0: from 1024 such workgroups on) */
 enum { TRITT_TUNE_FWD_SPLITS = 0, TRITT_TUNE_FWD_BAND = 1, TRITT_TUNE_BWD_SPLITS = 2, TRITT_TUNE_BWD128_WAVES = 3,
-       TRITT_TUNE_F32_VALU = 4, TRITT_TUNE_DPS_WAVES = 5, TRITT_TUNE_DPS_PAIR = 6, TRITT_TUNE_COUNT_ = 7 };
+       TRITT_TUNE_F32_VALU = 4, TRITT_TUNE_DPS_WAVES = 5, TRITT_TUNE_DPS_PAIR = 6, TRITT_TUNE_DPS_SHARED = 7,
+       TRITT_TUNE_COUNT_ = 8 };
 int tritt_set_tuning(int knob, int value, int* previous);
 
 /* ---- triple-dot-product:  s[q,j,k] = alpha * sum_d Q[q,d] K1[j,d] K2[k,d] ----------------

@@ -192,6 +192,53 @@ def test_paired_owner_tiles_change_nothing(T, D, k_diff, causal, waves, tune):
         util.assert_close(name, x, y, **LOWP)
 
 
+@pytest.mark.parametrize("B,H,T,D,k_diff,causal,dtype", [
+    (2, 3, 203, 64, 203, True, torch.bfloat16), (1, 2, 449, 64, 100, True, torch.float16),
+    (1, 3, 160, 128, 160, True, torch.bfloat16), (2, 2, 130, 32, 40, True, torch.bfloat16),
+    (1, 2, 257, 64, 257, False, torch.bfloat16), (1, 1, 33, 64, 5, True, torch.float16),
+    (1, 2, 128, 64, 0, True, torch.bfloat16), (1, 1, 1, 64, 1, True, torch.bfloat16)])
+def test_shared_tile_forward_kernel(B, H, T, D, k_diff, causal, dtype, tune):
+    """The forward kernel whose workgroups own 128 rows and read the streamed tiles from an LDS ring (the one large
+    grids take), forced on: output, LSE and, through the inner pass the backward runs again, all gradients against
+    the oracle; ragged lengths, bands narrower than a tile, no mask, one row, the three head dimensions."""
+    from flash_trittention import _lib
+
+    print(f"case dps shared-tile forward B={B} H={H} T={T} D={D} k_diff={k_diff} causal={causal} {dtype}", flush=True)
+    inputs = orc.make_inputs(B, H, T, D, dtype, seed=T + D + k_diff)
+    alpha = 1 / math.sqrt(D)
+    tune(_lib.TUNE_DPS_SHARED, 1)
+    out, m, grads = util.run_dps(inputs, alpha, causal, k_diff, flags=_lib.FLAG_FORCE_MFMA)
+    tune(_lib.TUNE_DPS_SHARED, -1)
+    other = util.run_dps(inputs, alpha, causal, k_diff, flags=_lib.FLAG_FORCE_MFMA)
+    z, lse, ref = util.oracle_dps(inputs, alpha, causal, k_diff)
+    util.assert_close("out", out, z, **LOWP)
+    util.assert_close("m", m, lse, rtol=1e-3, atol=2e-2)
+    for name, a, b in zip(util.NAMES, grads, ref):
+        util.assert_close(name, a, b, **LOWP)
+    # the two forward kernels round the same sums in a different order: a few 16-bit ulps apart
+    util.assert_close("out vs the per-tile kernel", out, other[0].float().cpu(), rtol=2e-2, atol=1e-2)
+
+
+def test_large_grids_take_the_shared_tile_forward(tune):
+    """B=16 H=16 T=500 D=64 (1024 workgroups of 128 rows): the default dispatch is the shared-tile kernel, bitwise what
+    the knob forces, and it matches the oracle on the heads checked."""
+    from flash_trittention import _lib
+
+    B, H, T, D = 16, 16, 500, 64
+    inputs = orc.make_inputs(B, H, T, D, torch.bfloat16, seed=77)
+    default = util.run_dps(inputs, 1 / 8, True, T, backward=False)
+    tune(_lib.TUNE_DPS_SHARED, 1)
+    forced = util.run_dps(inputs, 1 / 8, True, T, backward=False)
+    tune(_lib.TUNE_DPS_SHARED, -1)
+    never = util.run_dps(inputs, 1 / 8, True, T, backward=False)
+    assert torch.equal(default[0], forced[0]) and torch.equal(default[1], forced[1])
+    assert not torch.equal(default[0], never[0])
+    for b, h in ((0, 0), (7, 9), (15, 15)):
+        z, lse, _ = util.oracle_dps([t[b:b + 1, h:h + 1] for t in inputs], 1 / 8, True, T)
+        util.assert_close("out", default[0][b:b + 1, h:h + 1], z, **LOWP)
+        util.assert_close("m", default[1][b:b + 1, h:h + 1], lse, rtol=1e-3, atol=2e-2)
+
+
 def test_rejects_mismatched_shapes():
     from flash_trittention import TrittentionTriton
 
