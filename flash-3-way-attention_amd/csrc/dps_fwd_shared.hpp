@@ -25,7 +25,7 @@ struct FwdSharedShape {
 // BIAS: keys carry a bias (the outer pass); otherwise no bias is fetched (the inner pass).
 // With a multiplier (p.mul) every 16-bit output is the product out * mul, so `out` is for passes without one.
 template <typename E, int D, int kW, int kNS, bool BIAS>
-__global__ __launch_bounds__(64 * kW) void attn_fwd_shared_kernel(AttnFwdP<E> p) {
+__global__ __launch_bounds__(64 * kW, 2) void attn_fwd_shared_kernel(AttnFwdP<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using S = FwdSharedShape<D, kW, kNS>;

@@ -131,9 +131,12 @@ struct AttnFwdP {
     int pair;           // a workgroup takes two owner tiles, a long and a short one (see owner_tiles)
 };
 
-// kW: waves per workgroup (they split the streamed tiles of one owner tile)
+// kW: waves per workgroup (they split the streamed tiles of one owner tile).
+// Two waves per SIMD are asked for wherever the kernel fits 256 registers: a workgroup of 128 or 256 threads alone
+// would let the compiler plan for 512, and it then keeps every MFMA result in accumulation registers and copies the
+// accumulators to and from vector registers around the rescaling, every tile (80 of 240 vector instructions).
 template <typename E, int D, int kW>
-__global__ __launch_bounds__(64 * kW) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
+__global__ __launch_bounds__(64 * kW, 2) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
@@ -364,7 +367,7 @@ struct AttnBwdP {
 };
 
 template <typename E, int D, int kW>
-__global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> p) {
+__global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_kernel(AttnBwdP<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
@@ -506,7 +509,7 @@ __global__ __launch_bounds__(64 * kW) void attn_bwd_row_mfma_kernel(AttnBwdP<E> 
 
 // --------------------------------------------------------------------------- backward, columns
 template <typename E, int D, int kW, bool LINK>
-__global__ __launch_bounds__(64 * kW) void attn_bwd_col_mfma_kernel(AttnBwdP<E> p) {
+__global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_kernel(AttnBwdP<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
@@ -800,12 +803,15 @@ __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
             __syncthreads();
         }
     };
-    emit(p.v1, p.up1, p.up2, true);
-    emit(p.k1, p.k1p1, p.k1p2, false);
-    emit(p.k2, p.k2p1, p.k2p2, false);
-    if (p.q) emit(p.q, p.qp1, p.qp2, false);
-    if (p.d_o) emit(p.d_o, p.dop1, p.dop2, false);
-    if (p.delta) {
+    // blockIdx.y deals the tensors out (3 in the forward, 5 and the row vectors in the backward): a workgroup per
+    // tile walking them one after the other was five dependent round trips through LDS
+    const int job = blockIdx.y;
+    if (job == 0) emit(p.v1, p.up1, p.up2, true);
+    if (job == 1) emit(p.k1, p.k1p1, p.k1p2, false);
+    if (job == 2) emit(p.k2, p.k2p1, p.k2p2, false);
+    if (job == 3 && p.q) emit(p.q, p.qp1, p.qp2, false);
+    if (job == 4 && p.d_o) emit(p.d_o, p.dop1, p.dop2, false);
+    if (job == 5 && p.delta) {
         // Delta[j] = dO[j] . O[j]: the D / 8 lanes that hold a row's 16-byte pieces sit next to each other
         constexpr int cpr = D / 8;
         for (int idx = threadIdx.x; idx < 32 * cpr; idx += 256) {
@@ -911,7 +917,7 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
         pp.v1 = (const E*)a.v1; pp.k1 = (const E*)a.k1; pp.k2 = (const E*)a.k2;
         pp.up2 = (E*)(ws + l.up2); pp.k1p1 = (E*)(ws + l.k1p1); pp.k2p1 = (E*)(ws + l.k2p1);
         pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp;
-        hipLaunchKernelGGL((dps_prep_kernel<E, D>), grid, dim3(256), 0, st, pp);
+        hipLaunchKernelGGL((dps_prep_kernel<E, D>), dim3(grid.x, 3), dim3(256), 0, st, pp);
     }
     // inner: rows K2[t], keys K1, values U; R (fp32, backward only), W = R * V2 and W^T, lse1 (log2)
     AttnFwdP<E> p{};
@@ -977,7 +983,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     pp.qp2 = (E*)(ws + l.qp2); pp.dop2 = (E*)(ws + l.dop2);
     pp.lse2 = (float*)(ws + l.lse2); pp.delta = (float*)(ws + l.delta);
     pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp;
-    hipLaunchKernelGGL((dps_prep_kernel<E, D>), grid, dim3(256), 0, st, pp);
+    hipLaunchKernelGGL((dps_prep_kernel<E, D>), dim3(grid.x, 6), dim3(256), 0, st, pp);
     // recompute the inner pass: R, W, W^T, lse1
     e = run_fwd<E, D, kW>(a, st, true);
     if (e != hipSuccess) return e;
