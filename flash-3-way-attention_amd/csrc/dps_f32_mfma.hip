@@ -143,7 +143,7 @@ __device__ __forceinline__ int owner_tile(int causal) { return causal ? gridDim.
 //   out[r] = softmax_a(scale X[r].K[a] + bias[a]) @ V ;  lse_out[r] = lse_scale * log2-sum-exp2
 //   out_mul[r] = out[r] * mul[r]   (when mul != nullptr)
 template <int D>
-__global__ __launch_bounds__(128) void attn_fwd_f32m_kernel(
+__global__ __launch_bounds__(128, 2) void attn_fwd_f32m_kernel(
     const float* __restrict__ X, const float* __restrict__ K, const float* __restrict__ V,
     const float* __restrict__ bias, const float* __restrict__ mul, float* __restrict__ out,
     float* __restrict__ out_mul, float* __restrict__ lse_out, float lse_scale, int T, float scale_log2, int causal,
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(128) void attn_fwd_f32m_kernel(
 //   P = exp2(scale X[r].K[a] + bias[a] - lse2[r]);  dS = P (G[r].V[a] - delta[r]);
 //   dX[r] = alpha * sum_a dS K[a]  (+ addend[r])
 template <int D>
-__global__ __launch_bounds__(128) void attn_bwd_row_f32m_kernel(
+__global__ __launch_bounds__(128, 2) void attn_bwd_row_f32m_kernel(
     const float* __restrict__ X, const float* __restrict__ G, const float* __restrict__ K,
     const float* __restrict__ V, const float* __restrict__ bias, const float* __restrict__ lse, float lse_to_log2,
     const float* __restrict__ delta, const float* __restrict__ addend, float* __restrict__ dX, int T, float alpha,
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(128) void attn_bwd_row_f32m_kernel(
 // Attention backward, owner = key-like row a (the MFMA column); the query-like rows r are staged:
 //   dK[a] = alpha * sum_r dS X[r];  dV[a] = sum_r P G[r];  dbias[a] = sum_r dS
 template <int D>
-__global__ __launch_bounds__(128) void attn_bwd_col_f32m_kernel(
+__global__ __launch_bounds__(128, (D <= 32 ? 2 : 1)) void attn_bwd_col_f32m_kernel(
     const float* __restrict__ X, const float* __restrict__ G, const float* __restrict__ K,
     const float* __restrict__ V, const float* __restrict__ bias, const float* __restrict__ lse, float lse_to_log2,
     const float* __restrict__ delta, float* __restrict__ dK, float* __restrict__ dV, float* __restrict__ dbias, int T,
