@@ -807,9 +807,23 @@ int tritt_tdp_fwd_strided(const void* q, const void* k1, const void* k2, const v
     return tritt_tdp_fwd(v.ptr[0], v.ptr[1], v.ptr[2], v.ptr[3], v.ptr[4], o, lse, B, H, T, D, dtype, alpha, causal,
                          k1_window, k2_window, kk_left, kk_right, workspace, plain, flags, stream);
 }
+// The dot-product-sum kernels on the 16-bit matrix-core path read every strided view where it lies (the packing pass
+// and the owner-tile loads take the caller's strides); the fp32 path gets packed copies.
+static RowLayout row_layout(const tritt_layout* l, int H, int T, int D) {
+    if (!l) return RowLayout{(long long)H * T * D, (long long)T * D, D};
+    return RowLayout{l->stride_b, l->stride_h, l->stride_t};
+}
+static void dps_views(MfmaDpsArgs& a, const tritt_layout* in, const tritt_layout* d_o, int H, int T, int D) {
+    a.H = H;
+    a.lq = row_layout(in, H, T, D); a.lk1 = row_layout(in ? in + 1 : nullptr, H, T, D);
+    a.lk2 = row_layout(in ? in + 2 : nullptr, H, T, D); a.lv1 = row_layout(in ? in + 3 : nullptr, H, T, D);
+    a.lv2 = row_layout(in ? in + 4 : nullptr, H, T, D); a.ldo = row_layout(d_o, H, T, D);
+}
+
 size_t tritt_dps_fwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags,
                                              const tritt_layout* in_layouts) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (use_mfma_dps(D, dtype, flags)) return round256(tritt_dps_fwd_workspace_bytes(B, H, T, D, dtype, flags));
     Views v;
     const void* none[5] = {};
     if (plan_all(v, 0, none, in_layouts, 5, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
@@ -825,7 +839,19 @@ int tritt_dps_fwd_strided(const void* q, const void* k1, const void* k2, const v
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse})) return TRITT_ERR_INVALID;
     if (any_misaligned({q, k1, k2, v1, v2, o})) return TRITT_ERR_INVALID;
+    if (causal && k_diff < 0) return TRITT_ERR_INVALID;
+    for (int i = 0; in_layouts && i < 5; ++i)
+        if ((rc = check_layout(in_layouts + i, dtype)) != TRITT_OK) return rc;
     const size_t plain = round256(tritt_dps_fwd_workspace_bytes(B, H, T, D, dtype, flags));
+    if (use_mfma_dps(D, dtype, flags)) {
+        if (!workspace || workspace_bytes < plain) return TRITT_ERR_WORKSPACE;
+        MfmaDpsArgs a{};
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o_out = o; a.lse_out = lse; a.workspace = workspace;
+        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0; a.k_diff = clampw(k_diff, T);
+        a.is_bf16 = dtype == TRITT_BF16;
+        dps_views(a, in_layouts, nullptr, H, T, D);
+        return (int)mfma_dps_fwd(a, (hipStream_t)stream);
+    }
     Views v;
     const void* src[5] = {q, k1, k2, v1, v2};
     rc = plan_all(v, 0, src, in_layouts, 5, workspace ? (char*)workspace + plain : nullptr, B, H, T, D, dtype);
@@ -839,6 +865,7 @@ int tritt_dps_fwd_strided(const void* q, const void* k1, const void* k2, const v
 size_t tritt_dps_bwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, unsigned flags,
                                              const tritt_layout* in_layouts, const tritt_layout* d_o_layout) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (use_mfma_dps(D, dtype, flags)) return round256(tritt_dps_bwd_workspace_bytes(B, H, T, D, dtype, flags));
     Views v;
     const void* none[5] = {};
     if (plan_all(v, 0, none, in_layouts, 5, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
@@ -856,7 +883,22 @@ int tritt_dps_bwd_strided(const void* q, const void* k1, const void* k2, const v
     if (rc != TRITT_OK) return rc;
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o})) return TRITT_ERR_INVALID;
     if (any_misaligned({q, k1, k2, v1, v2, o, d_o})) return TRITT_ERR_INVALID;
+    if (causal && k_diff < 0) return TRITT_ERR_INVALID;
+    for (int i = 0; in_layouts && i < 5; ++i)
+        if ((rc = check_layout(in_layouts + i, dtype)) != TRITT_OK) return rc;
+    if ((rc = check_layout(d_o_layout, dtype)) != TRITT_OK) return rc;
     const size_t plain = round256(tritt_dps_bwd_workspace_bytes(B, H, T, D, dtype, flags));
+    if (use_mfma_dps(D, dtype, flags)) {
+        if (any_misaligned({dq, dk1, dk2, dv1, dv2}) || any_null({dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
+        if (!workspace || workspace_bytes < plain) return TRITT_ERR_WORKSPACE;
+        MfmaDpsArgs a{};
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.d_o = d_o; a.lse_in = lse;
+        a.dq = dq; a.dk1 = dk1; a.dk2 = dk2; a.dv1 = dv1; a.dv2 = dv2; a.workspace = workspace;
+        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0; a.k_diff = clampw(k_diff, T);
+        a.is_bf16 = dtype == TRITT_BF16;
+        dps_views(a, in_layouts, d_o_layout, H, T, D);
+        return (int)mfma_dps_bwd(a, (hipStream_t)stream);
+    }
     Views v;
     const void* src[5] = {q, k1, k2, v1, v2};
     char* tail = workspace ? (char*)workspace + plain : nullptr;

@@ -24,8 +24,8 @@ struct FwdSharedShape {
 
 // BIAS: keys carry a bias (the outer pass); otherwise no bias is fetched (the inner pass).
 // With a multiplier (p.mul) every 16-bit output is the product out * mul, so `out` is for passes without one.
-template <typename E, int D, int kW, int kNS, bool BIAS>
-__global__ __launch_bounds__(64 * kW, 2) void attn_fwd_shared_kernel(AttnFwdP<E> p) {
+template <typename E, int D, int kW, int kNS, bool BIAS, bool SV>
+__global__ __launch_bounds__(64 * kW, 2) void attn_fwd_shared_kernel(AttnFwdP<E, SV> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using S = FwdSharedShape<D, kW, kNS>;
@@ -41,11 +41,11 @@ __global__ __launch_bounds__(64 * kW, 2) void attn_fwd_shared_kernel(AttnFwdP<E>
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
-    const E* __restrict__ X = p.x + base;
     const char* KP = reinterpret_cast<const char*>(uniform_ptr(p.kp + tb));
     const char* VP2 = reinterpret_cast<const char*>(uniform_ptr(p.vp2 + tb));
     const char* BP = BIAS ? reinterpret_cast<const char*>(uniform_ptr(p.bias + vb)) : nullptr;
     const int rw0 = r0 + 32 * wave, r = rw0 + n;
+    const int2 at = slice_at<SV>(bh, p.H);
 
     // streamed tiles of the workgroup and of this wave's rows
     const int last_row = min(T - 1, r0 + 32 * kW - 1);
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(64 * kW, 2) void attn_fwd_shared_kernel(AttnFwdP<E>
 
     v8 xb[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) xb[ks] = ld8<E>(X + (size_t)min(r, T - 1) * D + 16 * ks + 8 * g);
+    for (int ks = 0; ks < KS; ++ks) xb[ks] = ld8<E>(p.x.row(at, min(r, T - 1), T, D) + 16 * ks + 8 * g);
     // the rows must have arrived before the loop: a wait for them placed inside it would also wait for the
     // tiles fetched ahead, every time round
 #pragma unroll
@@ -85,10 +85,11 @@ __global__ __launch_bounds__(64 * kW, 2) void attn_fwd_shared_kernel(AttnFwdP<E>
     const size_t row_off = base + (size_t)min(r, T - 1) * D;
     v4 mv[DT][4];
     if (p.mul) {
+        const E* __restrict__ mul_row = p.mul.row(at, min(r, T - 1), T, D);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) mv[dt][q4] = *reinterpret_cast<const v4*>(p.mul + row_off + 32 * dt + 8 * q4 + 4 * g);
+            for (int q4 = 0; q4 < 4; ++q4) mv[dt][q4] = *reinterpret_cast<const v4*>(mul_row + 32 * dt + 8 * q4 + 4 * g);
     }
 
     f32x16 acc[DT];

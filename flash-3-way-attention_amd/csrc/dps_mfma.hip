@@ -100,6 +100,34 @@ __device__ __forceinline__ bool pair_ok(int T, int causal, int k_diff, int r, in
     return (r < T) & (a < T) & ((!causal) | ((a <= r) & (r - a <= k_diff)));
 }
 
+// A [B,H,T,D] tensor where it lies.  SV (strided views): element (b, h, t, d) at b sb + h sh + t st + d, the caller's
+// strides for the caller's tensors and dense ones for the workspace's own row-major tensors; slices are indexed
+// (batch, head).  Otherwise every tensor is dense [BH][T][D], the slice index is bh alone and the row pitch is the
+// compile-time D (the strided form costs the dense calls 2-4 % at B=4 H=8 T=1024, so they keep their own kernels).
+template <typename E, bool SV>
+struct View;
+template <typename E>
+struct View<E, true> {
+    const E* p;
+    long long sb, sh;
+    unsigned st;
+    __device__ __forceinline__ const E* row(int2 at, int r, int, int) const {
+        return p + (size_t)at.x * sb + (size_t)at.y * sh + (size_t)(unsigned)r * st;
+    }
+    __device__ __forceinline__ explicit operator bool() const { return p != nullptr; }
+};
+template <typename E>
+struct View<E, false> {
+    const E* p;
+    __device__ __forceinline__ const E* row(int2 at, int r, int T, int D) const { return p + ((size_t)at.x * T + r) * D; }
+    __device__ __forceinline__ explicit operator bool() const { return p != nullptr; }
+};
+// the slice's index in the views' terms: (batch, head), or (bh, -) for dense tensors
+template <bool SV>
+__device__ __forceinline__ int2 slice_at(int bh, int H) {
+    return SV ? make_int2(bh / H, bh % H) : make_int2(bh, 0);
+}
+
 template <int D>
 __device__ __forceinline__ void spill_tiles(float* sO, int wave, const f32x16 (&acc)[D / 32], int n, int g) {
 #pragma unroll
@@ -109,13 +137,13 @@ __device__ __forceinline__ void spill_tiles(float* sO, int wave, const f32x16 (&
 }
 
 // ------------------------------------------------------------------------------------ forward
-template <typename E>
+template <typename E, bool SV>
 struct AttnFwdP {
-    const E* x;         // [BH][T][D]   query-like rows
+    View<E, SV> x;      // query-like rows
     const E* kp;        // [BH][Tp*D]   key-like rows, packing P1
     const E* vp2;       // [BH][Tp*D]   values, packing P2
     const float* bias;  // [BH][Tp] per-key bias in log2 units, or null
-    const E* mul;       // [BH][T][D] or null
+    View<E, SV> mul;    // or null
     E* out;             // [BH][T][D] or null
     float* out_f32;     // [BH][T][D] or null
     E* outm;            // out * mul, [BH][T][D] or null
@@ -124,6 +152,7 @@ struct AttnFwdP {
     float* lse;         // [BH][lse_stride]
     int lse_stride;
     int BH;
+    int H;              // heads per batch entry in the views' indexing
     float lse_scale;    // lse = lse_scale * log2-sum-exp2
     int T, Tp;
     float scale_log2;
@@ -135,8 +164,8 @@ struct AttnFwdP {
 // Two waves per SIMD are asked for wherever the kernel fits 256 registers: a workgroup of 128 or 256 threads alone
 // would let the compiler plan for 512, and it then keeps every MFMA result in accumulation registers and copies the
 // accumulators to and from vector registers around the rescaling, every tile (80 of 240 vector instructions).
-template <typename E, int D, int kW>
-__global__ __launch_bounds__(64 * kW, 2) void attn_fwd_mfma_kernel(AttnFwdP<E> p) {
+template <typename E, int D, int kW, bool SV>
+__global__ __launch_bounds__(64 * kW, 2) void attn_fwd_mfma_kernel(AttnFwdP<E, SV> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
@@ -156,15 +185,16 @@ __global__ __launch_bounds__(64 * kW, 2) void attn_fwd_mfma_kernel(AttnFwdP<E> p
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T, Tp = p.Tp;
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp, vb = (size_t)bh * Tp;
-    const E* __restrict__ X = p.x + base;
     const E* __restrict__ KP = p.kp + tb;
     const E* __restrict__ VP2 = p.vp2 + tb;
     const float* __restrict__ bias = p.bias ? p.bias + vb : nullptr;
     const int r = r0 + n;
+    const int2 at = slice_at<SV>(bh, p.H);
+    const E* __restrict__ xrow = p.x.row(at, min(r, T - 1), T, D);
 
     v8 xb[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) xb[ks] = ld8<E>(X + (size_t)min(r, T - 1) * D + 16 * ks + 8 * g);
+    for (int ks = 0; ks < KS; ++ks) xb[ks] = ld8<E>(xrow + 16 * ks + 8 * g);
 
     const int a_lo = p.causal ? max(0, r0 - p.k_diff) : 0;
     const int a_hi = p.causal ? min(T - 1, r0 + 31) : T - 1;
@@ -319,7 +349,7 @@ __global__ __launch_bounds__(64 * kW, 2) void attn_fwd_mfma_kernel(AttnFwdP<E> p
             v8 mv;
 #pragma unroll
             for (int j = 0; j < 8; ++j) mv[j] = (E)0.f;
-            if (row < T) mv = ld8<E>(p.mul + off);
+            if (row < T) mv = ld8<E>(p.mul.row(at, row, T, D) + d0);
             v8 wv;
 #pragma unroll
             for (int j = 0; j < 8; ++j) wv[j] = (E)(row < T ? o[j] * (float)mv[j] : 0.f);
@@ -336,10 +366,10 @@ __global__ __launch_bounds__(64 * kW, 2) void attn_fwd_mfma_kernel(AttnFwdP<E> p
 #include "dps_fwd_shared.hpp"
 
 // ------------------------------------------------------------------------------ backward, rows
-template <typename E>
+template <typename E, bool SV>
 struct AttnBwdP {
-    // [BH][T][D] row-major: what the owner tile loads once (row kernel: x, g; column kernel: k, v)
-    const E *x, *g, *k, *v;
+    // row-major: what the owner tile loads once (row kernel: x, g; column kernel: k, v)
+    View<E, SV> x, g, k, v;
     // streamed, operand-packed [BH][Tp*D]: row kernel kp, vp (P1) and kp2 (P2);
     // column kernel xp, gp (P1) and xp2, gp2 (P2)
     const E *kp, *vp, *kp2, *xp, *gp, *xp2, *gp2;
@@ -347,6 +377,7 @@ struct AttnBwdP {
     const float* lse2;       // [BH][Tp] log2 units
     const float* delta;      // [BH][Tp]
     int BH, T, Tp;
+    int H;                   // heads per batch entry in the views' indexing
     float alpha;
     int causal, k_diff;
     int pair;                // a workgroup takes two owner tiles, a long and a short one (see owner_tiles)
@@ -357,17 +388,17 @@ struct AttnBwdP {
     float* dk_f32;           // alpha * sum  (fp32) or null
     E* dk;                   // alpha * sum  (16 bit) or null
     // LINK == false: dv = sum * SiLU'(v1)
-    const E* v1;
+    View<E, SV> v1;
     E* dv;
     // LINK == true: dW = sum;  dV2 = dW R;  dR = dW V2;  delta1 = rowsum(dR R) - dbias
     const float* r_f32;
-    const E* v2;
+    View<E, SV> v2;
     E *dv2, *dr, *dr_p1, *dr_p2;
     float* delta1;           // [BH][Tp]
 };
 
-template <typename E, int D, int kW>
-__global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_kernel(AttnBwdP<E> p) {
+template <typename E, int D, int kW, bool SV>
+__global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_kernel(AttnBwdP<E, SV> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
@@ -392,11 +423,12 @@ __global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_
     const int r = r0 + n, rc = min(r, T - 1);
     const float scale_log2 = p.alpha * kLog2e;
 
+    const int2 at = slice_at<SV>(bh, p.H);
     v8 xb[KS], gb[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        xb[ks] = ld8<E>(p.x + base + (size_t)rc * D + 16 * ks + 8 * g);
-        gb[ks] = ld8<E>(p.g + base + (size_t)rc * D + 16 * ks + 8 * g);
+        xb[ks] = ld8<E>(p.x.row(at, rc, T, D) + 16 * ks + 8 * g);
+        gb[ks] = ld8<E>(p.g.row(at, rc, T, D) + 16 * ks + 8 * g);
     }
     const float lse2 = p.lse2[vb + rc], dl = p.delta[vb + rc];
 
@@ -508,8 +540,8 @@ __global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_
 }
 
 // --------------------------------------------------------------------------- backward, columns
-template <typename E, int D, int kW, bool LINK>
-__global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_kernel(AttnBwdP<E> p) {
+template <typename E, int D, int kW, bool LINK, bool SV>
+__global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_kernel(AttnBwdP<E, SV> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
@@ -538,11 +570,12 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
     const int a = c0 + n, ac = min(a, T - 1);
     const float scale_log2 = p.alpha * kLog2e;
 
+    const int2 at = slice_at<SV>(bh, p.H);
     v8 kb[KS], vbv[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        kb[ks] = ld8<E>(p.k + base + (size_t)ac * D + 16 * ks + 8 * g);
-        vbv[ks] = ld8<E>(p.v + base + (size_t)ac * D + 16 * ks + 8 * g);
+        kb[ks] = ld8<E>(p.k.row(at, ac, T, D) + 16 * ks + 8 * g);
+        vbv[ks] = ld8<E>(p.v.row(at, ac, T, D) + 16 * ks + 8 * g);
     }
     const float ba = p.bias ? p.bias[vb + ac] : 0.f;
 
@@ -694,7 +727,7 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
         }
         if constexpr (!LINK) {
             if (row < T) {
-                const v8 x = ld8<E>(p.v1 + off);
+                const v8 x = ld8<E>(p.v1.row(at, row, T, D) + d0);
                 v8 ov;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) ov[j] = (E)(o[j] * silu_grad_f((float)x[j]));
@@ -708,7 +741,7 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
                 dr[j] = (E)0.f;
             }
             if (row < T) {
-                const v8 x = ld8<E>(p.v2 + off);
+                const v8 x = ld8<E>(p.v2.row(at, row, T, D) + d0);
                 const float4 ra = *reinterpret_cast<const float4*>(p.r_f32 + off);
                 const float4 rb = *reinterpret_cast<const float4*>(p.r_f32 + off + 4);
                 const float rv[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
@@ -746,30 +779,33 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
 // Operand-packed copies of the inputs (U = SiLU(V1); rows past T are written as zeros), U row-major, and
 // the padded per-row vectors of the backward (LSE in log2 units, Delta = rowsum(dO * O)).  Null
 // pointers are skipped.
-template <typename E>
+template <typename E, bool SV>
 struct PrepP {
-    const E *v1, *k1, *k2, *q, *o, *d_o;
+    View<E, SV> v1, k1, k2, q, d_o;
+    const E* o;  // dense: the library's own output
     const float* lse;
     E* u;                            // row-major
     E *up1, *k1p1, *k2p1, *qp1, *dop1;  // packing P1
     E *up2, *k1p2, *k2p2, *qp2, *dop2;  // packing P2
     float *lse2, *delta;
     int BH, T, Tp;
+    int H;  // heads per batch entry in the views' indexing
 };
 
-template <typename E, int D>
-__global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
+template <typename E, int D, bool SV>
+__global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E, SV> p) {
     using v8 = typename Mma<E>::v8;
     int bh, tile_id;
     if (!block_to_tile(p.BH, p.Tp / 32, bh, tile_id)) return;
     const int j0 = tile_id * 32, T = p.T, Tp = p.Tp;
+    const int2 at = slice_at<SV>(bh, p.H);
     const size_t base = (size_t)bh * T * D, tb = (size_t)bh * D * Tp;
     // One 16-byte piece (8 consecutive d of one row) per thread and step: it is one piece of P1 as it stands.
     // P2 wants 8 consecutive rows of one column in a piece, so the 32 x D tile goes through LDS and comes
     // back out transposed, again as whole 16-byte pieces (element-wise 2-byte stores were most of this
     // kernel's time).
     __shared__ E sT[32][D + 2];
-    auto emit = [&](const E* src, E* dst1, E* dst2, bool silu) {
+    auto emit = [&](const View<E, SV>& src, E* dst1, E* dst2, bool silu) {
         if (!dst1 && !dst2 && !(silu && p.u)) return;  // uniform over the workgroup
         for (int idx = threadIdx.x; idx < 32 * (D / 8); idx += 256) {
             const int jj = idx / (D / 8), j = j0 + jj, d0 = (idx % (D / 8)) * 8;
@@ -778,7 +814,7 @@ __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
             v8 x;
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = (E)0.f;
-            if (in) x = *reinterpret_cast<const v8*>(src + off);
+            if (in) x = *reinterpret_cast<const v8*>(src.row(at, j, T, D) + d0);
             if (silu) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) x[e] = (E)(in ? silu_f((float)x[e]) : 0.f);
@@ -819,7 +855,7 @@ __global__ __launch_bounds__(256) void dps_prep_kernel(PrepP<E> p) {
             float part = 0.f;
             if (j < T) {
                 const size_t off = base + (size_t)j * D + c * 8;
-                const v8 a = *reinterpret_cast<const v8*>(p.o + off), b = *reinterpret_cast<const v8*>(p.d_o + off);
+                const v8 a = *reinterpret_cast<const v8*>(p.o + off), b = *reinterpret_cast<const v8*>(p.d_o.row(at, j, T, D) + c * 8);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) part += (float)a[e] * (float)b[e];
             }
@@ -900,34 +936,49 @@ dim3 attn_grid(const MfmaDpsArgs& a, int Tp, bool pair) {
     return dim3(8 * xcd_slots(a.BH, pair ? (nt + 1) / 2 : nt));
 }
 
-template <typename E, int D, int kW>
+// one of the caller's tensors / a row-major tensor of the workspace as the kernels take them
+// one of the caller's tensors / a row-major tensor of the workspace as the kernels take them
+template <typename E, bool SV>
+View<E, SV> dense_view(const MfmaDpsArgs& a, const void* p) {
+    if constexpr (SV) return View<E, true>{(const E*)p, (long long)a.H * a.T * a.D, (long long)a.T * a.D, (unsigned)a.D};
+    else return View<E, false>{(const E*)p};
+}
+template <typename E, bool SV>
+View<E, SV> caller_view(const MfmaDpsArgs& a, const void* p, const RowLayout& l) {
+    if constexpr (SV) return View<E, true>{(const E*)p, l.sb, l.sh, (unsigned)l.st};
+    else return View<E, false>{(const E*)p};
+}
+
+template <typename E, int D, int kW, bool SV>
 hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, for_bwd);
     char* ws = static_cast<char*>(a.workspace);
     const dim3 grid(8 * xcd_slots(a.BH, Tp / 32));
     const bool pair_in = pair_tiles(a, a.k_diff, grid.x, for_bwd), pair_out = pair_tiles(a, a.T, grid.x, for_bwd);
-    auto kern = attn_fwd_mfma_kernel<E, D, kW>;
+    auto kern = attn_fwd_mfma_kernel<E, D, kW, SV>;
     hipError_t e = allow_smem(kern, fwd_smem<D, kW>());
     if (e != hipSuccess) return e;
     const float sl2 = a.alpha * kLog2e;
 
     if (!for_bwd) {  // the backward's prep kernel has already written these
-        PrepP<E> pp{};
-        pp.v1 = (const E*)a.v1; pp.k1 = (const E*)a.k1; pp.k2 = (const E*)a.k2;
+        PrepP<E, SV> pp{};
+        pp.v1 = caller_view<E, SV>(a, a.v1, a.lv1); pp.k1 = caller_view<E, SV>(a, a.k1, a.lk1); pp.k2 = caller_view<E, SV>(a, a.k2, a.lk2);
         pp.up2 = (E*)(ws + l.up2); pp.k1p1 = (E*)(ws + l.k1p1); pp.k2p1 = (E*)(ws + l.k2p1);
-        pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp;
-        hipLaunchKernelGGL((dps_prep_kernel<E, D>), dim3(grid.x, 3), dim3(256), 0, st, pp);
+        pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp; pp.H = a.H;
+        hipLaunchKernelGGL((dps_prep_kernel<E, D, SV>), dim3(grid.x, 3), dim3(256), 0, st, pp);
     }
     // inner: rows K2[t], keys K1, values U; R (fp32, backward only), W = R * V2 and W^T, lse1 (log2)
-    AttnFwdP<E> p{};
-    p.x = (const E*)a.k2; p.kp = (const E*)(ws + l.k1p1); p.vp2 = (const E*)(ws + l.up2); p.mul = (const E*)a.v2;
+    AttnFwdP<E, SV> p{};
+    p.x = caller_view<E, SV>(a, a.k2, a.lk2); p.kp = (const E*)(ws + l.k1p1); p.vp2 = (const E*)(ws + l.up2);
+    p.mul = caller_view<E, SV>(a, a.v2, a.lv2);
     p.out_f32 = for_bwd ? (float*)(ws + l.r) : nullptr;
     p.outm = for_bwd ? (E*)(ws + l.w) : nullptr;
     p.outm_p1 = for_bwd ? (E*)(ws + l.wp1) : nullptr;
     p.outm_p2 = (E*)(ws + l.wp2);
     p.lse = (float*)(ws + l.lse1); p.lse_stride = Tp; p.lse_scale = 1.0f;
-    p.BH = a.BH; p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff; p.pair = pair_in;
+    p.BH = a.BH; p.H = a.H; p.T = a.T; p.Tp = Tp; p.scale_log2 = sl2; p.causal = a.causal; p.k_diff = a.k_diff;
+    p.pair = pair_in;
     // Large grids take the kernel whose workgroups own 128 rows and share the streamed tiles through LDS
     // (dps_fwd_shared.hpp).  One wave per 32 rows walks all streamed tiles of its rows, so the kernel needs four of
     // its workgroups per CU to keep the SIMDs busy; measured forward, bf16 D = 64, one owner tile per workgroup ->
@@ -935,8 +986,8 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     // 277 -> 391 us and B=4 H=8 T=1024 (256) 45 -> 70 us.
     constexpr int kSW = 4, kNS = 4;  // its waves and ring slots
     using Shared = FwdSharedShape<D, kSW, kNS>;
-    auto kern_in = attn_fwd_shared_kernel<E, D, kSW, kNS, false>;
-    auto kern_out = attn_fwd_shared_kernel<E, D, kSW, kNS, true>;
+    auto kern_in = attn_fwd_shared_kernel<E, D, kSW, kNS, false, SV>;
+    auto kern_out = attn_fwd_shared_kernel<E, D, kSW, kNS, true, SV>;
     const int owners = (Tp / 32 + kSW - 1) / kSW;
     const bool shared = knobs().dps_shared ? knobs().dps_shared > 0 : (long long)a.BH * owners >= 1024;
     const dim3 grid_shared(8 * xcd_slots(a.BH, owners));
@@ -949,70 +1000,76 @@ hipError_t run_fwd(const MfmaDpsArgs& a, hipStream_t st, bool for_bwd) {
     }
     if (for_bwd) return hipGetLastError();
     // outer: rows Q[q], keys K2 with bias lse1, values W; O and LSE (natural log)
-    AttnFwdP<E> o{};
-    o.x = (const E*)a.q; o.kp = (const E*)(ws + l.k2p1); o.vp2 = (const E*)(ws + l.wp2); o.bias = (const float*)(ws + l.lse1);
+    AttnFwdP<E, SV> o{};
+    o.x = caller_view<E, SV>(a, a.q, a.lq); o.kp = (const E*)(ws + l.k2p1); o.vp2 = (const E*)(ws + l.wp2); o.bias = (const float*)(ws + l.lse1);
     o.out = (E*)a.o_out; o.lse = a.lse_out; o.lse_stride = a.T; o.lse_scale = kLn2;
-    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T; o.pair = pair_out;
+    o.BH = a.BH; o.H = a.H; o.T = a.T; o.Tp = Tp; o.scale_log2 = sl2; o.causal = a.causal; o.k_diff = a.T;
+    o.pair = pair_out;
     if (shared) hipLaunchKernelGGL(kern_out, grid_shared, dim3(64 * kSW), Shared::smem, st, o);
     else hipLaunchKernelGGL(kern, attn_grid(a, Tp, pair_out), dim3(64 * kW), (fwd_smem<D, kW>()), st, o);
     return hipGetLastError();
 }
 
-template <typename E, int D, int kW>
+template <typename E, int D, int kW, bool SV>
 hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     const int Tp = (a.T + 31) / 32 * 32;
     const Layout l = layout(a.BH, a.T, D, true);
     char* ws = static_cast<char*>(a.workspace);
     const dim3 grid(8 * xcd_slots(a.BH, Tp / 32));
     const bool pair_in = pair_tiles(a, a.k_diff, grid.x, true), pair_out = pair_tiles(a, a.T, grid.x, true);
-    auto krow = attn_bwd_row_mfma_kernel<E, D, kW>;
-    auto kcol_link = attn_bwd_col_mfma_kernel<E, D, kW, true>;
-    auto kcol = attn_bwd_col_mfma_kernel<E, D, kW, false>;
+    auto krow = attn_bwd_row_mfma_kernel<E, D, kW, SV>;
+    auto kcol_link = attn_bwd_col_mfma_kernel<E, D, kW, true, SV>;
+    auto kcol = attn_bwd_col_mfma_kernel<E, D, kW, false, SV>;
     hipError_t e = allow_smem(krow, row_smem<D, kW>());
     if (e == hipSuccess) e = allow_smem(kcol_link, col_smem<D, kW>());
     if (e == hipSuccess) e = allow_smem(kcol, col_smem<D, kW>());
     if (e != hipSuccess) return e;
 
-    PrepP<E> pp{};
-    pp.v1 = (const E*)a.v1; pp.k1 = (const E*)a.k1; pp.k2 = (const E*)a.k2; pp.q = (const E*)a.q;
-    pp.o = (const E*)a.o; pp.d_o = (const E*)a.d_o; pp.lse = a.lse_in;
+    PrepP<E, SV> pp{};
+    pp.v1 = caller_view<E, SV>(a, a.v1, a.lv1); pp.k1 = caller_view<E, SV>(a, a.k1, a.lk1); pp.k2 = caller_view<E, SV>(a, a.k2, a.lk2);
+    pp.q = caller_view<E, SV>(a, a.q, a.lq); pp.d_o = caller_view<E, SV>(a, a.d_o, a.ldo);
+    pp.o = (const E*)a.o; pp.lse = a.lse_in;
     pp.u = (E*)(ws + l.u);
     pp.up1 = (E*)(ws + l.up1); pp.k1p1 = (E*)(ws + l.k1p1); pp.k2p1 = (E*)(ws + l.k2p1);
     pp.qp1 = (E*)(ws + l.qp1); pp.dop1 = (E*)(ws + l.dop1);
     pp.up2 = (E*)(ws + l.up2); pp.k1p2 = (E*)(ws + l.k1p2); pp.k2p2 = (E*)(ws + l.k2p2);
     pp.qp2 = (E*)(ws + l.qp2); pp.dop2 = (E*)(ws + l.dop2);
     pp.lse2 = (float*)(ws + l.lse2); pp.delta = (float*)(ws + l.delta);
-    pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp;
-    hipLaunchKernelGGL((dps_prep_kernel<E, D>), dim3(grid.x, 6), dim3(256), 0, st, pp);
+    pp.BH = a.BH; pp.T = a.T; pp.Tp = Tp; pp.H = a.H;
+    hipLaunchKernelGGL((dps_prep_kernel<E, D, SV>), dim3(grid.x, 6), dim3(256), 0, st, pp);
     // recompute the inner pass: R, W, W^T, lse1
-    e = run_fwd<E, D, kW>(a, st, true);
+    e = run_fwd<E, D, kW, SV>(a, st, true);
     if (e != hipSuccess) return e;
 
     // outer pass: X = Q, G = dO, K = K2 (bias lse1), V = W
-    AttnBwdP<E> o{};
-    o.x = (const E*)a.q; o.g = (const E*)a.d_o; o.k = (const E*)a.k2; o.v = (const E*)(ws + l.w);
+    AttnBwdP<E, SV> o{};
+    o.x = caller_view<E, SV>(a, a.q, a.lq); o.g = caller_view<E, SV>(a, a.d_o, a.ldo); o.k = caller_view<E, SV>(a, a.k2, a.lk2);
+    o.v = dense_view<E, SV>(a, ws + l.w);
     o.kp = (const E*)(ws + l.k2p1); o.vp = (const E*)(ws + l.wp1); o.kp2 = (const E*)(ws + l.k2p2);
     o.xp = (const E*)(ws + l.qp1); o.gp = (const E*)(ws + l.dop1);
     o.xp2 = (const E*)(ws + l.qp2); o.gp2 = (const E*)(ws + l.dop2);
     o.bias = (const float*)(ws + l.lse1); o.lse2 = (const float*)(ws + l.lse2); o.delta = (const float*)(ws + l.delta);
-    o.BH = a.BH; o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T; o.pair = pair_out;
+    o.BH = a.BH; o.H = a.H; o.T = a.T; o.Tp = Tp; o.alpha = a.alpha; o.causal = a.causal; o.k_diff = a.T;
+    o.pair = pair_out;
     o.dx = (E*)a.dq;
     o.dk_f32 = (float*)(ws + l.dk2p);
-    o.r_f32 = (const float*)(ws + l.r); o.v2 = (const E*)a.v2; o.dv2 = (E*)a.dv2;
+    o.r_f32 = (const float*)(ws + l.r); o.v2 = caller_view<E, SV>(a, a.v2, a.lv2); o.dv2 = (E*)a.dv2;
     o.dr = (E*)(ws + l.dr); o.dr_p1 = (E*)(ws + l.drp1); o.dr_p2 = (E*)(ws + l.drp2); o.delta1 = (float*)(ws + l.delta1);
     hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_out), dim3(64 * kW), (row_smem<D, kW>()), st, o);
     hipLaunchKernelGGL(kcol_link, attn_grid(a, Tp, pair_out), dim3(64 * kW), (col_smem<D, kW>()), st, o);
 
     // inner pass: X = K2, G = dR, K = K1, V = U
-    AttnBwdP<E> i{};
-    i.x = (const E*)a.k2; i.g = (const E*)(ws + l.dr); i.k = (const E*)a.k1; i.v = (const E*)(ws + l.u);
+    AttnBwdP<E, SV> i{};
+    i.x = caller_view<E, SV>(a, a.k2, a.lk2); i.g = dense_view<E, SV>(a, ws + l.dr); i.k = caller_view<E, SV>(a, a.k1, a.lk1);
+    i.v = dense_view<E, SV>(a, ws + l.u);
     i.kp = (const E*)(ws + l.k1p1); i.vp = (const E*)(ws + l.up1); i.kp2 = (const E*)(ws + l.k1p2);
     i.xp = (const E*)(ws + l.k2p1); i.gp = (const E*)(ws + l.drp1);
     i.xp2 = (const E*)(ws + l.k2p2); i.gp2 = (const E*)(ws + l.drp2);
     i.lse2 = (const float*)(ws + l.lse1); i.delta = (const float*)(ws + l.delta1);
-    i.BH = a.BH; i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff; i.pair = pair_in;
+    i.BH = a.BH; i.H = a.H; i.T = a.T; i.Tp = Tp; i.alpha = a.alpha; i.causal = a.causal; i.k_diff = a.k_diff;
+    i.pair = pair_in;
     i.addend = (const float*)(ws + l.dk2p); i.dx = (E*)a.dk2;
-    i.dk = (E*)a.dk1; i.v1 = (const E*)a.v1; i.dv = (E*)a.dv1;
+    i.dk = (E*)a.dk1; i.v1 = caller_view<E, SV>(a, a.v1, a.lv1); i.dv = (E*)a.dv1;
     hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_in), dim3(64 * kW), (row_smem<D, kW>()), st, i);
     hipLaunchKernelGGL(kcol, attn_grid(a, Tp, pair_in), dim3(64 * kW), (col_smem<D, kW>()), st, i);
     return hipGetLastError();
@@ -1037,27 +1094,30 @@ static bool two_waves(const MfmaDpsArgs& a, bool backward) {
     return a.T < (backward ? 2048 : 1024);
 }
 
-template <typename E>
+template <typename E, bool SV>
 static hipError_t dps_fwd_typed(const MfmaDpsArgs& a, hipStream_t st) {
-    if (a.D == 32) return run_fwd<E, 32, 4>(a, st, false);
-    if (a.D == 64) return two_waves(a, false) ? run_fwd<E, 64, 2>(a, st, false) : run_fwd<E, 64, 4>(a, st, false);
-    if (a.D == 128) return run_fwd<E, 128, 2>(a, st, false);
+    if (a.D == 32) return run_fwd<E, 32, 4, SV>(a, st, false);
+    if (a.D == 64) return two_waves(a, false) ? run_fwd<E, 64, 2, SV>(a, st, false) : run_fwd<E, 64, 4, SV>(a, st, false);
+    if (a.D == 128) return run_fwd<E, 128, 2, SV>(a, st, false);
     return hipErrorInvalidValue;
 }
-template <typename E>
+template <typename E, bool SV>
 static hipError_t dps_bwd_typed(const MfmaDpsArgs& a, hipStream_t st) {
-    if (a.D == 32) return run_bwd<E, 32, 4>(a, st);
-    if (a.D == 64) return two_waves(a, true) ? run_bwd<E, 64, 2>(a, st) : run_bwd<E, 64, 4>(a, st);
-    if (a.D == 128) return run_bwd<E, 128, 2>(a, st);
+    if (a.D == 32) return run_bwd<E, 32, 4, SV>(a, st);
+    if (a.D == 64) return two_waves(a, true) ? run_bwd<E, 64, 2, SV>(a, st) : run_bwd<E, 64, 4, SV>(a, st);
+    if (a.D == 128) return run_bwd<E, 128, 2, SV>(a, st);
     return hipErrorInvalidValue;
 }
 
+// a.H > 0: the caller's tensors are strided views (the kernels that take strides); otherwise the dense kernels
 hipError_t mfma_dps_fwd(const MfmaDpsArgs& a, hipStream_t st) {
-    return a.is_bf16 ? dps_fwd_typed<__bf16>(a, st) : dps_fwd_typed<_Float16>(a, st);
+    if (a.H > 0) return a.is_bf16 ? dps_fwd_typed<__bf16, true>(a, st) : dps_fwd_typed<_Float16, true>(a, st);
+    return a.is_bf16 ? dps_fwd_typed<__bf16, false>(a, st) : dps_fwd_typed<_Float16, false>(a, st);
 }
 
 hipError_t mfma_dps_bwd(const MfmaDpsArgs& a, hipStream_t st) {
-    return a.is_bf16 ? dps_bwd_typed<__bf16>(a, st) : dps_bwd_typed<_Float16>(a, st);
+    if (a.H > 0) return a.is_bf16 ? dps_bwd_typed<__bf16, true>(a, st) : dps_bwd_typed<_Float16, true>(a, st);
+    return a.is_bf16 ? dps_bwd_typed<__bf16, false>(a, st) : dps_bwd_typed<_Float16, false>(a, st);
 }
 
 }  // namespace tritt

@@ -146,8 +146,15 @@ bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit);
 hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st);
 
 // 16-bit MFMA dot-product-sum (two chained banded attentions; D = 32, 64 or 128).
+// strides of a [B,H,T,D] view in elements (tritt_layout)
+struct RowLayout {
+    long long sb, sh, st;
+};
 struct MfmaDpsArgs {
     const void *q, *k1, *k2, *v1, *v2;
+    // H > 0: q, k1, k2, v1, v2 and d_o are views with these strides (read where they lie); H == 0: all dense
+    int H;
+    RowLayout lq, lk1, lk2, lv1, lv2, ldo;
     void* o_out;          // forward output
     float* lse_out;       // forward output [BH, T] (natural log)
     const void *o, *d_o;  // backward inputs

@@ -159,6 +159,53 @@ def test_triple_dot_forward_reads_the_views_in_place():
     del fused
 
 
+def test_dot_product_sum_reads_the_views_in_place():
+    """The 16-bit matrix-core kernels of dot-product-sum take [B,T,H,D] tensors transposed, and dO likewise, without a
+    copy: forward and backward ask for the dense calls' workspaces, and the peak of device memory over each call is
+    its outputs plus that workspace."""
+    from flash_trittention import _lib, _ops
+
+    B, H, T, D = 4, 8, 1024, 64
+    views = [bthd_view(B, H, T, D, torch.bfloat16, seed=20 + i) for i in range(5)]
+    d_o = bthd_view(B, H, T, D, torch.bfloat16, seed=26)
+    lay, lay_do = _lib.layouts(views), _lib.layouts([d_o])
+    api = _lib.lib()
+    args = (B, H, T, D, _lib.TRITT_BF16, 0)
+    plain_f, plain_b = api.tritt_dps_fwd_workspace_bytes(*args), api.tritt_dps_bwd_workspace_bytes(*args)
+    assert api.tritt_dps_fwd_strided_workspace_bytes(*args, lay) == (plain_f + 255) // 256 * 256
+    assert api.tritt_dps_bwd_strided_workspace_bytes(*args, lay, lay_do) == (plain_b + 255) // 256 * 256
+    n_bytes = B * H * T * D * 2
+
+    o, m = _ops.dps_fwd_impl(*views, 1 / 8, True, T, 0)  # first calls: kernel attributes, allocator pools
+    _ops.dps_bwd_impl(*views, o, m, d_o, 1 / 8, True, T, 0)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    o, m = _ops.dps_fwd_impl(*views, 1 / 8, True, T, 0)
+    torch.cuda.synchronize()
+    grown = torch.cuda.max_memory_allocated() - before
+    slack = 2 << 20  # the allocator rounds a large block up to 2 MiB; one copy of one view would add n_bytes = 4 MiB
+    assert grown < o.numel() * 2 + m.numel() * 4 + plain_f + slack, (grown, plain_f)
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    grads = _ops.dps_bwd_impl(*views, o, m, d_o, 1 / 8, True, T, 0)
+    torch.cuda.synchronize()
+    grown = torch.cuda.max_memory_allocated() - before
+    assert grown < 5 * n_bytes + plain_b + slack, (grown, plain_b)
+    dense = [v.contiguous() for v in views]
+    o_d, m_d = _ops.dps_fwd_impl(*dense, 1 / 8, True, T, 0)
+    grads_d = _ops.dps_bwd_impl(*dense, o_d, m_d, d_o.contiguous(), 1 / 8, True, T, 0)
+    assert torch.equal(o, o_d) and torch.equal(m, m_d)
+    for name, a, b in zip(util.NAMES, grads, grads_d):
+        assert torch.equal(a, b), name
+    # broadcast views (a stride of zero) are read in place as well
+    one = torch.randn(1, 1, T, D, generator=torch.Generator().manual_seed(5)).bfloat16().cuda()
+    shared = [one.expand(B, H, T, D) for _ in range(5)]
+    o_b, m_b = _ops.dps_fwd_impl(*shared, 1 / 8, True, T, 0)
+    o_c, m_c = _ops.dps_fwd_impl(*(t.contiguous() for t in shared), 1 / 8, True, T, 0)
+    assert torch.equal(o_b, o_c) and torch.equal(m_b, m_c)
+
+
 def test_split_operands_and_static_layout_cases():
     """convert_to_float32 (split operands) on strided views; extent-1 dimensions with arbitrary strides; a broadcast
     (stride 0) head dimension."""
@@ -210,17 +257,18 @@ def test_layouts_the_library_refuses():
     st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125, 1,
                                           T, _lib.ptr(ws), ws.numel(), 0, _lib.stream_ptr(o.device))
     assert st == -1
-    # too small a workspace for the gathered copies
+    # too small a workspace: for the gathered copy of the fp32 path, for the call itself on the matrix-core path
     lay[0].stride_t = 2 * D
-    need = _lib.lib().tritt_dps_fwd_strided_workspace_bytes(B, H, T, D, _lib.TRITT_BF16, 0, lay)
-    plain = _lib.lib().tritt_dps_fwd_workspace_bytes(B, H, T, D, _lib.TRITT_BF16, 0)
-    assert need == (plain + 255) // 256 * 256 + B * H * T * D * 2
     wide = torch.randn(B, H, T, 2 * D, generator=g).bfloat16().cuda()
     ptrs[0] = _lib.ptr(wide)
-    st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125, 1,
-                                          T, _lib.ptr(ws), need - 1, 0, _lib.stream_ptr(o.device))
-    assert st == -3  # TRITT_ERR_WORKSPACE
-    st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125, 1,
-                                          T, _lib.ptr(ws), need, 0, _lib.stream_ptr(o.device))
-    assert st == 0
+    for flags, copies in ((_lib.FLAG_FORCE_GENERIC, 1), (0, 0)):
+        need = _lib.lib().tritt_dps_fwd_strided_workspace_bytes(B, H, T, D, _lib.TRITT_BF16, flags, lay)
+        plain = _lib.lib().tritt_dps_fwd_workspace_bytes(B, H, T, D, _lib.TRITT_BF16, flags)
+        assert need == (plain + 255) // 256 * 256 + copies * B * H * T * D * 2
+        st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125,
+                                              1, T, _lib.ptr(ws), need - 1, flags, _lib.stream_ptr(o.device))
+        assert st == -3  # TRITT_ERR_WORKSPACE
+        st = _lib.lib().tritt_dps_fwd_strided(*ptrs, lay, _lib.ptr(o), _lib.ptr(lse), B, H, T, D, _lib.TRITT_BF16, 0.125,
+                                              1, T, _lib.ptr(ws), need, flags, _lib.stream_ptr(o.device))
+        assert st == 0
     torch.cuda.synchronize()
