@@ -911,10 +911,31 @@ int tritt_dps_bwd_strided(const void* q, const void* k1, const void* k2, const v
                          D, dtype, alpha, causal, k_diff, workspace, plain, flags, stream);
 }
 
+// The triple-dot backward on the 16-bit matrix-core path reads the six views where they lie when every row stride
+// fits the kernels' 32-bit byte offsets and none is a broadcast along t (the transposing pass reads a pitch of 0 as
+// "dense"); otherwise, and on the fp32 path, the views are gathered into the workspace first.
+static bool bwd_reads_in_place(const tritt_layout* in, const tritt_layout* d_o, int dtype, int T) {
+    auto fits = [&](const tritt_layout* l) {
+        return !l || (check_layout(l, dtype) == TRITT_OK && (long long)T * l->stride_t <= 0x7fffffffLL &&
+                      (T == 1 || l->stride_t != 0));
+    };
+    for (int i = 0; in && i < 5; ++i)
+        if (!fits(in + i)) return false;
+    return fits(d_o);
+}
+static TensorAt tensor_at(const tritt_layout* l, int H, int T, int D) {
+    if (!l) return dense_at(H, T, D);
+    return TensorAt{l->stride_b, l->stride_h, (unsigned)(T == 1 ? D : l->stride_t)};
+}
+
 size_t tritt_tdp_bwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window,
                                              int k2_window, int kk_left, int kk_right, unsigned flags,
                                              const tritt_layout* in_layouts, const tritt_layout* d_o_layout) {
     if (check_common(B, H, T, D, dtype) != TRITT_OK) return 0;
+    if (use_mfma_bwd(T, D, dtype, causal, clampw(k1_window, T), clampw(k2_window, T), clampw(kk_left, T), clampw(kk_right, T),
+                     flags) &&
+        bwd_reads_in_place(in_layouts, d_o_layout, dtype, T))
+        return round256(tritt_tdp_bwd_workspace_bytes(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags));
     Views v;
     const void* none[5] = {};
     if (plan_all(v, 0, none, in_layouts, 5, nullptr, B, H, T, D, dtype) != TRITT_OK) return 0;
@@ -935,8 +956,35 @@ int tritt_tdp_bwd_strided(const void* q, const void* k1, const void* k2, const v
     if (any_null({q, k1, k2, v1, v2, o, lse, d_o})) return TRITT_ERR_INVALID;
     if (any_misaligned({q, k1, k2, v1, v2, o, d_o})) return TRITT_ERR_INVALID;
     if (!dq && !dk1 && !dk2 && !dv1 && !dv2) return TRITT_OK;
+    if (causal && (k1_window < 0 || k2_window < 0 || kk_left < 0 || kk_right < 0)) return TRITT_ERR_INVALID;
+    for (int i = 0; in_layouts && i < 5; ++i)
+        if ((rc = check_layout(in_layouts + i, dtype)) != TRITT_OK) return rc;
+    if ((rc = check_layout(d_o_layout, dtype)) != TRITT_OK) return rc;
     const size_t plain =
         round256(tritt_tdp_bwd_workspace_bytes(B, H, T, D, dtype, causal, k1_window, k2_window, kk_left, kk_right, flags));
+    const int w1 = clampw(k1_window, T), w2 = clampw(k2_window, T), kl = clampw(kk_left, T), kr = clampw(kk_right, T);
+    if (use_mfma_bwd(T, D, dtype, causal, w1, w2, kl, kr, flags) && (in_layouts || d_o_layout) &&
+        bwd_reads_in_place(in_layouts, d_o_layout, dtype, T)) {
+        if (any_misaligned({dq, dk1, dk2, dv1, dv2})) return TRITT_ERR_INVALID;
+        if ((flags & TRITT_FLAG_SPLIT_OPERANDS) && !use_split(D, dtype, flags)) return TRITT_ERR_UNSUPPORTED;
+        if (!workspace || workspace_bytes < plain) return TRITT_ERR_WORKSPACE;
+        MfmaBwdArgs a{};
+        a.q = q; a.k1 = k1; a.k2 = k2; a.v1 = v1; a.v2 = v2; a.o = o; a.d_o = d_o; a.lse = lse;
+        a.dq = dq; a.dk1 = dk1; a.dk2 = dk2; a.dv1 = dv1; a.dv2 = dv2; a.workspace = workspace;
+        a.BH = B * H; a.T = T; a.D = D; a.alpha = alpha; a.causal = causal ? 1 : 0;
+        a.is_bf16 = dtype == TRITT_BF16;
+        a.windowed = full_windows(T, causal, w1, w2, kl, kr) ? 0 : 1;
+        a.k1_window = w1; a.k2_window = w2; a.kk_left = kl; a.kk_right = kr;
+        a.deterministic = (flags & TRITT_FLAG_FLOAT_ATOMICS) ? 0 : 1;
+        a.split = use_split(D, dtype, flags) ? 1 : 0;
+        a.H = H;
+        a.at_q = tensor_at(in_layouts, H, T, D); a.at_k1 = tensor_at(in_layouts ? in_layouts + 1 : nullptr, H, T, D);
+        a.at_k2 = tensor_at(in_layouts ? in_layouts + 2 : nullptr, H, T, D);
+        a.at_v1 = tensor_at(in_layouts ? in_layouts + 3 : nullptr, H, T, D);
+        a.at_v2 = tensor_at(in_layouts ? in_layouts + 4 : nullptr, H, T, D);
+        a.at_do = tensor_at(d_o_layout, H, T, D);
+        return (int)mfma_tdp_bwd(a, (hipStream_t)stream);
+    }
     Views v;
     const void* src[5] = {q, k1, k2, v1, v2};
     char* tail = workspace ? (char*)workspace + plain : nullptr;

@@ -171,13 +171,16 @@ __device__ __forceinline__ void shared_add(void* acc, size_t idx, float v, float
 }
 // block-wide maximum of the finite |x| bit patterns of `count` 16-byte pieces (E8 = 8 elements of E, or 4 floats)
 // starting at src; every thread of the 256-thread block returns the same value; `red` = 4 words of LDS
+// (row_pieces > 0: the pieces form rows of row_pieces pieces that lie `pitch` elements apart)
 template <typename E>
-__device__ __forceinline__ unsigned block_absmax_bits(const E* __restrict__ src, size_t count, unsigned* red) {
+__device__ __forceinline__ unsigned block_absmax_bits(const E* __restrict__ src, size_t count, unsigned* red,
+                                                      unsigned row_pieces = 0, unsigned pitch = 0) {
     constexpr int PER = 16 / sizeof(E);
     typedef __attribute__((ext_vector_type(PER))) E ev;
     unsigned m = 0;
     for (size_t i = threadIdx.x; i < count; i += 256) {
-        const ev x = *reinterpret_cast<const ev*>(src + i * PER);
+        const size_t at = row_pieces ? (i / row_pieces) * pitch + (i % row_pieces) * PER : i * PER;
+        const ev x = *reinterpret_cast<const ev*>(src + at);
 #pragma unroll
         for (int e = 0; e < PER; ++e) m = max(m, finite_abs_bits((float)x[e]));
     }

@@ -19,6 +19,14 @@ struct Knobs {
 };
 Knobs knobs();
 
+// Where slice (b, h) of a [B,H,T,D] tensor starts and how far its rows lie apart, in elements (a strided view of the
+// caller's, or a dense tensor: sb = H T D, sh = T D, st = D).
+struct TensorAt {
+    long long sb, sh;
+    unsigned st;
+};
+inline TensorAt dense_at(int H, int T, int D) { return TensorAt{(long long)H * T * D, (long long)T * D, (unsigned)D}; }
+
 // hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per (device, kernel): the attribute belongs to the
 // device's copy of the kernel, and a process may drive several devices.
 hipError_t ensure_dynamic_smem(const void* kernel, size_t bytes);
@@ -51,7 +59,10 @@ hipError_t f32_mfma_tdp_bwd(const GenericTdpArgs& a, long long* scratch, hipStre
 // 16-bit tensors (D = 32, 64 or 128) and added to the accumulators of the 16-bit MFMA backward, which then starts
 // at the tile after them.
 struct FirstTileArgs {
-    const void *q, *d_o, *k1, *u, *k2, *v2;  // 16-bit [BH][T][D]; u = SiLU(V1)
+    const void *q, *d_o, *k1, *u, *k2, *v2;  // 16-bit; u = SiLU(V1) is dense [BH][T][D]
+    // the other five lie where the caller has them: H heads per batch entry and these strides (H = 0: all dense)
+    int H;
+    TensorAt at_q, at_do, at_k1, at_k2, at_v2;
     // scratch, [BH][T] floats each: the covered rows' LSE and Delta, recomputed in fp32 (tiles == 1: delta_f32 holds
     // the per-round partials of tile 0 instead, [BH][32][4][3])
     float *lse_f32, *delta_f32;
@@ -127,6 +138,10 @@ hipError_t mfma_tdp_fwd(const MfmaFwdArgs& a, hipStream_t st);
 // 16-bit MFMA triple-dot backward (any mask; D = 32, 64 or 128).
 struct MfmaBwdArgs {
     const void *q, *k1, *k2, *v1, *v2, *o, *d_o;
+    // H > 0: q, k1, k2, v1, v2 and d_o are strided views (heads per batch entry, strides in elements) that the kernels
+    // read where they lie; H == 0: all dense [BH][T][D]
+    int H;
+    TensorAt at_q, at_k1, at_k2, at_v1, at_v2, at_do;
     const float* lse;
     void *dq, *dk1, *dk2, *dv1, *dv2;
     void* workspace;  // mfma_tdp_bwd_workspace() bytes

@@ -28,6 +28,11 @@ __device__ __forceinline__ int wave_of(unsigned tid) { return __builtin_amdgcn_r
 template <typename E>
 struct BwdParams {
     const E *q, *d_o;
+    // SV ("strided views") instantiations only: layouts of q, d_o, row_k, row_v, st_k, st_v (the caller's strides for
+    // the caller's tensors, dense ones for SiLU(V1), which the workspace holds) and heads per batch entry; the other
+    // instantiations take every tensor as dense [BH][T][D]
+    TensorAt at_q, at_do, at_row_k, at_row_v, at_st_k, at_st_v;
+    int H;
     const E *row_k, *row_v;    // [BH][T][D] "row" tensors: one row per wave and round (K2,V2 | K1,U)
     const E *st_k, *st_v;      // [BH][T][D] streamed tensors (K1,U | K2,V2) ...
     const E *st_kt, *st_vt;    // ... and their transposes [BH][D][Tp], zero padded
@@ -56,6 +61,18 @@ struct BwdParams {
 
 // the 16-bit kernels' accumulators resolve 2^-30 of the slice's max |dO| and cover sums up to 2^33 times it
 constexpr int kFixedBias = 30;
+
+// slice bh of a row-major tensor and its row pitch in elements (the compile-time D without SV)
+template <bool SV, int D, typename E>
+__device__ __forceinline__ const E* slice_of(const E* t, const TensorAt& at, int bh, int H, int T) {
+    if constexpr (SV) return t + (size_t)(bh / H) * at.sb + (size_t)(bh % H) * at.sh;
+    else return t + (size_t)bh * T * D;
+}
+template <bool SV, int D>
+__device__ __forceinline__ unsigned pitch_of(const TensorAt& at) {
+    if constexpr (SV) return at.st;
+    else return (unsigned)D;
+}
 
 // scale of the fixed-point accumulators of slice bh (0: the accumulators are fp32)
 template <typename E>
@@ -97,7 +114,7 @@ namespace tritt {
 //  * stages are fetched direct-to-LDS two ahead into three buffers and the workgroup barrier
 //    sits in the middle of a stage: by then the next stage has landed for every wave, so its
 //    first row operands are read during the second half and nothing waits at the stage boundary.
-template <typename E, int D, bool WITH_DQ>
+template <typename E, int D, bool WITH_DQ, bool SV = false>
 __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -136,10 +153,15 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
-    const E* __restrict__ K1 = p.st_k + base;
-    const E* __restrict__ U = p.st_v + base;
-    const E* __restrict__ K2 = p.row_k + base;
-    const E* __restrict__ V2 = p.row_v + base;
+    const E* __restrict__ K1 = slice_of<SV, D>(p.st_k, p.at_st_k, bh, p.H, T);
+    const E* __restrict__ U = slice_of<SV, D>(p.st_v, p.at_st_v, bh, p.H, T);
+    const E* __restrict__ K2 = slice_of<SV, D>(p.row_k, p.at_row_k, bh, p.H, T);
+    const E* __restrict__ V2 = slice_of<SV, D>(p.row_v, p.at_row_v, bh, p.H, T);
+    const E* __restrict__ Qs = slice_of<SV, D>(p.q, p.at_q, bh, p.H, T);
+    const E* __restrict__ Os = slice_of<SV, D>(p.d_o, p.at_do, bh, p.H, T);
+    // row pitches in elements
+    const unsigned pK1 = pitch_of<SV, D>(p.at_st_k), pU = pitch_of<SV, D>(p.at_st_v), pK2 = pitch_of<SV, D>(p.at_row_k),
+                   pV2 = pitch_of<SV, D>(p.at_row_v), pQ = pitch_of<SV, D>(p.at_q), pO = pitch_of<SV, D>(p.at_do);
     const E* __restrict__ K1T = p.st_kt + tbase;
     const E* __restrict__ UT = p.st_vt + tbase;
 
@@ -164,13 +186,14 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     // Per-lane byte offsets of the wave's four blocks inside a stage; the stage itself only moves
     // the (scalar) base.  Row-major tensors clamp rows past the end of the sequence (last stage of
     // a ragged T only): that path recomputes the offsets.
+    const unsigned pitch = tensor == 0 ? pK1 : pU;  // of this wave's row-major tensor
     unsigned soff[LW];
     {
         const int pos = lane & 7, rr = lane >> 3;
 #pragma unroll
         for (int c = 0; c < LW; ++c) {
             const int r = ((wave & 1) * 4 + c) * 8 + rr;
-            soff[c] = rowmajor ? (unsigned)r * (D * 2) + ((pos ^ swz_perm(r)) * 16)
+            soff[c] = rowmajor ? (unsigned)r * (pitch * 2) + ((pos ^ swz_perm(r)) * 16)
                                : (unsigned)r * p.Tp * 2 + ((pos ^ swz_seq(r)) * 16);
         }
     }
@@ -182,10 +205,10 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
 #pragma unroll
             for (int c = 0; c < LW; ++c) {
                 const int r = ((wave & 1) * 4 + c) * 8 + rr;
-                direct_load_16(gsrc, (unsigned)min(jb + r, T - 1) * (D * 2) + ((pos ^ swz_perm(r)) * 16), dst + c * 512);
+                direct_load_16(gsrc, (unsigned)min(jb + r, T - 1) * (pitch * 2) + ((pos ^ swz_perm(r)) * 16), dst + c * 512);
             }
         } else {
-            const E* sbase = gsrc + (size_t)jb * (rowmajor ? D : 1);
+            const E* sbase = gsrc + (size_t)jb * (rowmajor ? pitch : 1u);
 #pragma unroll
             for (int c = 0; c < LW; ++c) direct_load_16(sbase, soff[c], dst + c * 512);
         }
@@ -194,7 +217,7 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
         if (wave < 2) {
             int ln = lane;
             asm volatile("" : "+v"(ln));
-            const unsigned off = (unsigned)min(m * 8 + (ln >> 3), T - 1) * (D * 2) + (ln & 7) * 16;
+            const unsigned off = (unsigned)min(m * 8 + (ln >> 3), T - 1) * ((wave ? pV2 : pK2) * 2) + (ln & 7) * 16;
             direct_load_16(uniform_ptr(wave ? V2 : K2), off, (wave ? sVr : sKr) + buf * 8 * D);
         }
     };
@@ -203,16 +226,16 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     // every round, so stage numbers simply cycle: stage of running index x is x mod nst)
     for (int idx = tid; idx < BQ * D; idx += NTH) {
         const int r = idx / D, d = idx % D;
-        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
-        const E qv = p.q[off], ov = p.d_o[off];
+        const unsigned row = (unsigned)min(q0 + r, T - 1);
+        const E qv = Qs[(size_t)row * pQ + d], ov = Os[(size_t)row * pO + d];
         sQb[r * LDQ + d] = (float)qv * scale_log2;
         sOb[r * LDQ + d] = (float)ov;
     }
     for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
         const int i = idx & 15, ln = (idx >> 4) & 63, dt = idx >> 10;
-        const size_t off = base + (size_t)min(q0 + c_row(ln >> 5, i), T - 1) * D + dt * 32 + (ln & 31);
-        sQe[idx] = p.q[off];
-        sOe[idx] = p.d_o[off];
+        const unsigned row = (unsigned)min(q0 + c_row(ln >> 5, i), T - 1);
+        sQe[idx] = Qs[(size_t)row * pQ + dt * 32 + (ln & 31)];
+        sOe[idx] = Os[(size_t)row * pO + dt * 32 + (ln & 31)];
     }
     if constexpr (WITH_DQ) {
         float* all = sOb + BQ * LDQ;
@@ -483,9 +506,15 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
                                                        int Tp, int D, int zero_width,
                                                        unsigned* __restrict__ scale_parts,
                                                        unsigned* __restrict__ poison,
-                                                       const E* __restrict__ o_res) {
+                                                       const E* __restrict__ o_res, int H, TensorAt at_v1,
+                                                       TensorAt at_k1, TensorAt at_k2, TensorAt at_v2, TensorAt at_do) {
+    // v1, k1, k2, v2 and d_o lie where the caller has them (H heads per batch entry, strides in elements; a dense
+    // call passes H = 1 and dense strides); everything else is dense
     const int bh = blockIdx.y, j0 = blockIdx.x * 64;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * Tp;
+    const int b_ = bh / H, h_ = bh % H;
+    auto slice = [&](const E* t, const TensorAt& at) { return t + (size_t)b_ * at.sb + (size_t)h_ * at.sh; };
+    v1 = slice(v1, at_v1); k1 = slice(k1, at_k1); k2 = slice(k2, at_k2); v2 = slice(v2, at_v2); d_o = slice(d_o, at_do);
     if (scale_parts) {
         // fixed-point accumulators: clear the poison words of this block's rows; the first blocks of a slice
         // also leave the partial maxima of |dO| that fix the slice's scale (part s = 64-row blocks s, s + 8, ...)
@@ -494,21 +523,21 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
         for (int part = blockIdx.x; part < kScaleParts; part += gridDim.x) {
             unsigned m = 0;
             for (int r0 = part * 64; r0 < T; r0 += kScaleParts * 64)
-                m = max(m, block_absmax_bits<E>(d_o + base + (size_t)r0 * D, (size_t)min(64, T - r0) * D / 8, red));
+                m = max(m, block_absmax_bits<E>(d_o + (size_t)r0 * at_do.st, (size_t)min(64, T - r0) * D / 8, red, D / 8, at_do.st));
             if (threadIdx.x == 0) scale_parts[bh * kScaleParts + part] = m;
         }
     }
     // two tiles at a time (static LDS stays under 64 KB at D = 128): their loads are in flight together
     constexpr int kTile = 64 * (128 + 2);
     __shared__ E tiles[2 * kTile];
-    transpose_load<E, true>(v1 + base, u + base, tiles, j0, T, D);
-    transpose_load<E, false>(k1 + base, nullptr, tiles + kTile, j0, T, D);
+    transpose_load<E, true>(v1, u + base, tiles, j0, T, D, at_v1.st);
+    transpose_load<E, false>(k1, nullptr, tiles + kTile, j0, T, D, at_k1.st);
     __syncthreads();
     transpose_store<E>(ut + tbase, tiles, j0, Tp, D);
     transpose_store<E>(k1t + tbase, tiles + kTile, j0, Tp, D);
     __syncthreads();
-    transpose_load<E, false>(k2 + base, nullptr, tiles, j0, T, D);
-    transpose_load<E, false>(v2 + base, nullptr, tiles + kTile, j0, T, D);
+    transpose_load<E, false>(k2, nullptr, tiles, j0, T, D, at_k2.st);
+    transpose_load<E, false>(v2, nullptr, tiles + kTile, j0, T, D, at_v2.st);
     __syncthreads();
     transpose_store<E>(k2t + tbase, tiles, j0, Tp, D);
     transpose_store<E>(v2t + tbase, tiles + kTile, j0, Tp, D);
@@ -533,7 +562,8 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const E* __restrict__ v1,
         float part = 0.f;
         if (j < T) {
             const size_t off = base + (size_t)j * D + c * 8;
-            const e8 a = *reinterpret_cast<const e8*>(o + off), b = *reinterpret_cast<const e8*>(d_o + off);
+            const e8 a = *reinterpret_cast<const e8*>(o + off);
+            const e8 b = *reinterpret_cast<const e8*>(d_o + (size_t)j * at_do.st + c * 8);
             if (o_res) {  // split operands: the output to 16 mantissa bits (rounded value + rounding residual)
                 const e8 r = *reinterpret_cast<const e8*>(o_res + off);
 #pragma unroll
@@ -560,8 +590,8 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
                                                          E* __restrict__ dv2, size_t n, int fixed_point,
                                                          const float* __restrict__ dq0acc, int T, int D,
                                                          const unsigned* __restrict__ scale_parts,
-                                                         const unsigned* __restrict__ poison) {
-    // a null output is a gradient the caller does not want
+                                                         const unsigned* __restrict__ poison, int H, TensorAt at_v1) {
+    // a null output is a gradient the caller does not want; v1 lies where the caller has it (see bwd_prep_kernel)
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
         const size_t row = i / D, t = row % T;
         double inv = 0.0;
@@ -576,7 +606,11 @@ __global__ __launch_bounds__(256) void bwd_finish_kernel(const float* __restrict
             return (float)((double)reinterpret_cast<const long long*>(acc)[at] * inv);
         };
         if (dk1) dk1[i] = (E)value(dk1acc, i, kPoisonDK1);
-        if (dv1) dv1[i] = (E)(value(duacc, i, kPoisonDU) * silu_grad_f((float)v1[i]));
+        if (dv1) {
+            const size_t bh = row / T;
+            const E x = v1[(bh / H) * at_v1.sb + (bh % H) * at_v1.sh + t * at_v1.st + i % D];
+            dv1[i] = (E)(value(duacc, i, kPoisonDU) * silu_grad_f((float)x));
+        }
         if (dk2) dk2[i] = (E)value(dk2acc, i, kPoisonDK2);
         if (dv2) dv2[i] = (E)value(dv2acc, i, kPoisonDV2);
         if (dqacc && dq) dq[i] = (E)(value(dqacc, i, kPoisonDQ) * alpha);
@@ -620,7 +654,8 @@ static BwdLayout bwd_layout(int BH, int T, int D, bool fixed_point) {
     return l;
 }
 
-template <typename E, int D>
+// SV: the caller's tensors are strided views, read where they lie (the kernels' SV instantiations)
+template <typename E, int D, bool SV>
 static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     const int Tp = (a.T + 63) / 64 * 64;
     const BwdLayout l = bwd_layout(a.BH, a.T, D, a.deterministic);
@@ -645,9 +680,15 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
                        (float*)(ws + l.delta), dk1acc, duacc, dk2acc, dv2acc, dqacc, a.T, Tp, D,
                        a.deterministic ? 2 * D : D, a.deterministic ? (unsigned*)(ws + l.scale_parts) : nullptr,
                        (unsigned*)(ws + l.poison),
-                       a.split ? (const E*)a.o + (size_t)a.BH * a.T * D : (const E*)nullptr);
+                       a.split ? (const E*)a.o + (size_t)a.BH * a.T * D : (const E*)nullptr, SV ? a.H : 1,
+                       SV ? a.at_v1 : dense_at(1, a.T, D), SV ? a.at_k1 : dense_at(1, a.T, D),
+                       SV ? a.at_k2 : dense_at(1, a.T, D), SV ? a.at_v2 : dense_at(1, a.T, D),
+                       SV ? a.at_do : dense_at(1, a.T, D));
 
     BwdParams<E> p;
+    p.H = SV ? a.H : 1;
+    const TensorAt at_u = dense_at(p.H, a.T, D);  // SiLU(V1), in the workspace
+    p.at_q = a.at_q; p.at_do = a.at_do;
     p.q = (const E*)a.q; p.d_o = (const E*)a.d_o;
     p.lse = a.lse; p.delta = (const float*)(ws + l.delta);
     p.dq = (E*)a.dq;
@@ -665,18 +706,18 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     if constexpr (D == 32) {
         // one shape, the banded instantiation for every mask (full windows are windows of T)
         smem = bwdg_smem(32, 8, 32, true);
-        kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true>;
-        kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true>;
+        kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true, false, SV>;
+        kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true, false, SV>;
         if (a.split) {
-            kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true, true>;
-            kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true, true>;
+            kern_dq = tdp_bwd_rows_general_kernel<E, 32, true, 8, 32, true, true, SV>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 32, false, 8, 32, true, true, SV>;
         }
     } else if (a.split) {
         // split operands: the general kernel (banded instantiation: full windows are windows of T)
         if constexpr (D == 64) {
             smem = bwdg_smem(64, 8, 64, true);
-            kern_dq = tdp_bwd_rows_general_kernel<E, 64, true, 8, 64, true, true>;
-            kern_nodq = tdp_bwd_rows_general_kernel<E, 64, false, 8, 64, true, true>;
+            kern_dq = tdp_bwd_rows_general_kernel<E, 64, true, 8, 64, true, true, SV>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 64, false, 8, 64, true, true, SV>;
         } else {
             return hipErrorInvalidValue;
         }
@@ -684,13 +725,13 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         // the 16-query kernel (tdp_bwd_rows_q16.hpp), banded instantiation
         if constexpr (D == 128) {
             smem = bwd_q16_smem();
-            kern_dq = tdp_bwd_rows_q16_kernel<E, true, true>;
-            kern_nodq = tdp_bwd_rows_q16_kernel<E, false, true>;
+            kern_dq = tdp_bwd_rows_q16_kernel<E, true, true, SV>;
+            kern_nodq = tdp_bwd_rows_q16_kernel<E, false, true, SV>;
         }
     } else if (a.windowed) {
         smem = bwdg_smem(D, 8, 64, true);
-        kern_dq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), true, 8, 64, true>;
-        kern_nodq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), false, 8, 64, true>;
+        kern_dq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), true, 8, 64, true, false, SV>;
+        kern_nodq = tdp_bwd_rows_general_kernel<E, (D < 64 ? 64 : D), false, 8, 64, true, false, SV>;
         col_parts = D / 64;
     } else if constexpr (D == 128) {
         // Default: 16 queries per wave on 16x16x32 tiles, every gradient column in one wave, S and dP formed once
@@ -700,24 +741,24 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         const int variant = knobs().bwd128_variant;
         if (variant != 4 && variant != 8) {
             smem = bwd_q16_smem();
-            kern_dq = tdp_bwd_rows_q16_kernel<E, true, false>;
-            kern_nodq = tdp_bwd_rows_q16_kernel<E, false, false>;
+            kern_dq = tdp_bwd_rows_q16_kernel<E, true, false, SV>;
+            kern_nodq = tdp_bwd_rows_q16_kernel<E, false, false, SV>;
         } else if (variant == 8) {
             smem = bwdg_smem(128, 8, 64, true);
-            kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 8, 64, false>;
-            kern_nodq = tdp_bwd_rows_general_kernel<E, 128, false, 8, 64, false>;
+            kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 8, 64, false, false, SV>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 128, false, 8, 64, false, false, SV>;
             col_parts = 2;
         } else {
             smem = bwdg_smem(128, 4, 128, true);
-            kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 4, 128, false>;
-            kern_nodq = tdp_bwd_rows_general_kernel<E, 128, false, 4, 128, false>;
+            kern_dq = tdp_bwd_rows_general_kernel<E, 128, true, 4, 128, false, false, SV>;
+            kern_nodq = tdp_bwd_rows_general_kernel<E, 128, false, 4, 128, false, false, SV>;
             nthreads = 256;
         }
     } else {
         smem = 2 * (size_t)(3 * 4 * 64 * 64 + 2 * 2 * 8 * 64 + 2 * (64 / 32) * 64 * 16) +
                4 * (size_t)(2 * 32 * (64 + 4) + 4 * 32 * 64);
-        kern_dq = tdp_bwd_rows_kernel<E, 64, true>;
-        kern_nodq = tdp_bwd_rows_kernel<E, 64, false>;
+        kern_dq = tdp_bwd_rows_kernel<E, 64, true, SV>;
+        kern_nodq = tdp_bwd_rows_kernel<E, 64, false, SV>;
     }
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
@@ -734,6 +775,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     if (first_in_f32) {
         FirstTileArgs f{};
         f.q = a.q; f.d_o = a.d_o; f.k1 = a.k1; f.u = u; f.k2 = a.k2; f.v2 = a.v2;
+        f.H = SV ? a.H : 0; f.at_q = a.at_q; f.at_do = a.at_do; f.at_k1 = a.at_k1; f.at_k2 = a.at_k2; f.at_v2 = a.at_v2;
         f.lse_f32 = (float*)(ws + l.lse_f32); f.delta_f32 = (float*)(ws + l.delta_f32);
         f.dq0_acc = ws + l.dq0acc;
         f.dq = a.dq; f.acc_k2 = dk2acc; f.acc_v2 = dv2acc; f.acc_k1 = dk1acc; f.acc_u = duacc; f.acc_q = dqacc;
@@ -752,6 +794,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.row_k = (const E*)a.k2; p.row_v = (const E*)a.v2;
     p.st_k = (const E*)a.k1; p.st_v = u; p.st_kt = k1t; p.st_vt = ut;
+    p.at_row_k = a.at_k2; p.at_row_v = a.at_v2; p.at_st_k = a.at_k1; p.at_st_v = at_u;
     p.acc_k = dk2acc; p.acc_v = dv2acc; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
     // a launch whose gradients the caller does not want (null outputs) is skipped
@@ -760,6 +803,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     // rows = (K1, U), streamed = (K2, V2): dK1, dU
     p.row_k = (const E*)a.k1; p.row_v = u;
     p.st_k = (const E*)a.k2; p.st_v = (const E*)a.v2; p.st_kt = k2t; p.st_vt = v2t;
+    p.at_row_k = a.at_k1; p.at_row_v = at_u; p.at_st_k = a.at_k2; p.at_st_v = a.at_v2;
     p.acc_k = dk1acc; p.acc_v = duacc; p.bit_k = kPoisonDK1; p.bit_v = kPoisonDU;
     p.wa = a.k2_window; p.wb = a.k1_window; p.lab = a.kk_right; p.rab = a.kk_left;  // the mask with j and k exchanged
     if (tiles_here > 0 && want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
@@ -772,7 +816,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
                        (E*)a.dq, (const E*)a.v1, (E*)a.dk1, (E*)a.dv1, (E*)a.dk2, (E*)a.dv2, n,
                        a.deterministic ? 1 : 0,
                        (first_in_f32 && !all_in_f32 && !dqacc) ? (const float*)(ws + l.dq0acc) : nullptr, a.T, D,
-                       p.scale_parts, p.poison);
+                       p.scale_parts, p.poison, p.H, SV ? a.at_v1 : dense_at(1, a.T, D));
     return hipGetLastError();
 }
 
@@ -781,11 +825,15 @@ size_t mfma_tdp_bwd_workspace(int BH, int T, int D, bool deterministic) {
 }
 bool mfma_tdp_bwd_supported(int D, int dtype_is_16bit) { return dtype_is_16bit && (D == 32 || D == 64 || D == 128); }
 
-hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st) {
-    if (a.D == 32) return a.is_bf16 ? launch_bwd<__bf16, 32>(a, st) : launch_bwd<_Float16, 32>(a, st);
-    if (a.D == 64) return a.is_bf16 ? launch_bwd<__bf16, 64>(a, st) : launch_bwd<_Float16, 64>(a, st);
-    if (a.D == 128) return a.is_bf16 ? launch_bwd<__bf16, 128>(a, st) : launch_bwd<_Float16, 128>(a, st);
+template <bool SV>
+static hipError_t bwd_by_shape(const MfmaBwdArgs& a, hipStream_t st) {
+    if (a.D == 32) return a.is_bf16 ? launch_bwd<__bf16, 32, SV>(a, st) : launch_bwd<_Float16, 32, SV>(a, st);
+    if (a.D == 64) return a.is_bf16 ? launch_bwd<__bf16, 64, SV>(a, st) : launch_bwd<_Float16, 64, SV>(a, st);
+    if (a.D == 128) return a.is_bf16 ? launch_bwd<__bf16, 128, SV>(a, st) : launch_bwd<_Float16, 128, SV>(a, st);
     return hipErrorInvalidValue;
+}
+hipError_t mfma_tdp_bwd(const MfmaBwdArgs& a, hipStream_t st) {
+    return a.H > 0 ? bwd_by_shape<true>(a, st) : bwd_by_shape<false>(a, st);
 }
 
 }  // namespace tritt

@@ -70,7 +70,8 @@ constexpr size_t bwdg_smem(int d, int nw, int ncol, bool with_dq) {
 // of 16-bit numbers (16 mantissa bits together; the streamed K1 / U operands are exact), two MFMAs per k-step: S
 // and dP then carry fp32 accumulation error only, and dS = P (dP - Delta) no longer cancels numbers that carry
 // 16-bit operand rounding.
-template <typename E, int D, bool WITH_DQ, int NW, int NCOL, bool WIN, bool SPLIT = false>
+// SV: the caller's tensors are strided views (BwdParams::at_*); otherwise everything is dense.
+template <typename E, int D, bool WITH_DQ, int NW, int NCOL, bool WIN, bool SPLIT = false, bool SV = false>
 __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -127,8 +128,13 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     const int T = p.T;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
     const float fscale = acc_scale(p, bh);
-    const E* __restrict__ K2 = p.row_k + base;
-    const E* __restrict__ V2 = p.row_v + base;
+    const E* __restrict__ K2 = slice_of<SV, D>(p.row_k, p.at_row_k, bh, p.H, T);
+    const E* __restrict__ V2 = slice_of<SV, D>(p.row_v, p.at_row_v, bh, p.H, T);
+    const E* __restrict__ Qs = slice_of<SV, D>(p.q, p.at_q, bh, p.H, T);
+    const E* __restrict__ Os = slice_of<SV, D>(p.d_o, p.at_do, bh, p.H, T);
+    // row pitches in elements
+    const unsigned pK2 = pitch_of<SV, D>(p.at_row_k), pV2 = pitch_of<SV, D>(p.at_row_v), pQ = pitch_of<SV, D>(p.at_q),
+                   pO = pitch_of<SV, D>(p.at_do), pSK = pitch_of<SV, D>(p.at_st_k), pSV = pitch_of<SV, D>(p.at_st_v);
 
     const int q0 = qt * BQ;
     const int qlast = min(T - 1, q0 + BQ - 1);
@@ -165,11 +171,12 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
         if (b < 2 * RB) {
             const int R = (b % RB) * RPB + lane / CPR, hh = R >> 5, r = R & 31;
             const int chunk = (lane % CPR) ^ (D == 32 ? swz_t(r) : swz_perm(r));
-            gsrc[c] = uniform_ptr((b < RB ? p.st_k : p.st_v) + base);
+            gsrc[c] = uniform_ptr(b < RB ? slice_of<SV, D>(p.st_k, p.at_st_k, bh, p.H, T)
+                                         : slice_of<SV, D>(p.st_v, p.at_st_v, bh, p.H, T));
             rowkey[c] = r;
             rowrest[c] = (unsigned)(hh * 64 + chunk * 8) * 2;
-            goff[c] = (unsigned)r * (D * 2) + rowrest[c];
-            gstep[c] = D * 2;
+            gstep[c] = (b < RB ? pSK : pSV) * 2;
+            goff[c] = (unsigned)r * gstep[c] + rowrest[c];
         } else {
             const int dl = ((b - 2 * RB) % (NCOL / 16)) * 16 + (lane >> 2);
             const int chunk = (lane & 3) ^ swz_t(dl);
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
 #pragma unroll
         for (int c = 0; c < LW; ++c) {
             unsigned off = goff[c] + (unsigned)jb * gstep[c];
-            if (ragged && rowkey[c] >= 0) off = (unsigned)min(jb + rowkey[c], T - 1) * (D * 2) + rowrest[c];
+            if (ragged && rowkey[c] >= 0) off = (unsigned)min(jb + rowkey[c], T - 1) * gstep[c] + rowrest[c];
             direct_load_16(gsrc[c], off, dst + c * 1024);
         }
     };
@@ -201,7 +208,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             asm volatile("" : "+v"(ln));
             const int part = wave % LR;
             const bool second = wave >= LR;
-            const unsigned off = (unsigned)min(m * NW + part * RPL + ln / LPR, T - 1) * (D * 2) + (ln % LPR) * 16;
+            const unsigned off = (unsigned)min(m * NW + part * RPL + ln / LPR, T - 1) * ((second ? pV2 : pK2) * 2) + (ln % LPR) * 16;
             direct_load_16(uniform_ptr(second ? V2 : K2), off, (second ? sVr : sKr) + buf * RR * D + part * RPL * D);
         }
     };
@@ -209,21 +216,22 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     // ---- prologue
     for (int idx = tid; idx < BQ * D; idx += NTH) {
         const int r = idx / D, d = idx % D;
-        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
+        const unsigned row = (unsigned)min(q0 + r, T - 1);
+        const E qv = Qs[(size_t)row * pQ + d], ov = Os[(size_t)row * pO + d];
         if constexpr (QF) {
-            sQf[r * LDQ + d] = (float)p.q[off] * scale_log2;
-            sOf[r * LDQ + d] = (float)p.d_o[off];
+            sQf[r * LDQ + d] = (float)qv * scale_log2;
+            sOf[r * LDQ + d] = (float)ov;
         } else {
-            sQb[r * LDK + d] = p.q[off];
-            sOb[r * LDK + d] = p.d_o[off];
+            sQb[r * LDK + d] = qv;
+            sOb[r * LDK + d] = ov;
         }
     }
     if constexpr (EPI_TILES) {
         for (int idx = tid; idx < DT * 64 * 16; idx += NTH) {
             const int i = idx & 15, ln = (idx >> 4) & 63, dt = idx >> 10;
-            const size_t off = base + (size_t)min(q0 + c_row(ln >> 5, i), T - 1) * D + c0 + dt * 32 + (ln & 31);
-            sQe[idx] = p.q[off];
-            sOe[idx] = p.d_o[off];
+            const unsigned row = (unsigned)min(q0 + c_row(ln >> 5, i), T - 1);
+            sQe[idx] = Qs[(size_t)row * pQ + c0 + dt * 32 + (ln & 31)];
+            sOe[idx] = Os[(size_t)row * pO + c0 + dt * 32 + (ln & 31)];
         }
     }
     if constexpr (WITH_DQ) {

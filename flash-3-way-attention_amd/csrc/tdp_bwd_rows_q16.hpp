@@ -64,7 +64,7 @@ constexpr size_t bwd_q16_smem() {
            + 2 * (size_t)(32 * (128 + 8) * 2);  // Q and dO tiles
 }
 
-template <typename E, bool WITH_DQ, bool WIN>
+template <typename E, bool WITH_DQ, bool WIN, bool SV = false>
 __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     using M = Mma<E>;
     using M16 = Mma16<E>;
@@ -98,8 +98,13 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     const int T = p.T;
     const size_t base = (size_t)bh * T * D, tbase = (size_t)bh * D * p.Tp;
     const float fscale = acc_scale(p, bh);
-    const E* __restrict__ K2 = p.row_k + base;
-    const E* __restrict__ V2 = p.row_v + base;
+    const E* __restrict__ K2 = slice_of<SV, D>(p.row_k, p.at_row_k, bh, p.H, T);
+    const E* __restrict__ V2 = slice_of<SV, D>(p.row_v, p.at_row_v, bh, p.H, T);
+    const E* __restrict__ Qs = slice_of<SV, D>(p.q, p.at_q, bh, p.H, T);
+    const E* __restrict__ Os = slice_of<SV, D>(p.d_o, p.at_do, bh, p.H, T);
+    // row pitches in elements
+    const unsigned pK2 = pitch_of<SV, D>(p.at_row_k), pV2 = pitch_of<SV, D>(p.at_row_v), pQ = pitch_of<SV, D>(p.at_q),
+                   pO = pitch_of<SV, D>(p.at_do);
 
     const int q0 = qt * BQ;
     const int qlast = min(T - 1, q0 + BQ - 1);
@@ -123,7 +128,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
 
     // ---- stage loader: wave w fetches blocks 2 w, 2 w + 1 of 8 blocks of K1 rows and 8 of U rows (tile rows
     //   8 b .. 8 b + 7; blocks 0..3 are keys 0..31 of columns 0..63, blocks 4..7 the same keys of columns 64..127)
-    const E* gsrc = uniform_ptr((wave < 4 ? p.st_k : p.st_v) + base);
+    const E* gsrc = uniform_ptr(wave < 4 ? slice_of<SV, D>(p.st_k, p.at_st_k, bh, p.H, T)
+                                         : slice_of<SV, D>(p.st_v, p.at_st_v, bh, p.H, T));
+    const unsigned gpitch2 = (wave < 4 ? pitch_of<SV, D>(p.at_st_k) : pitch_of<SV, D>(p.at_st_v)) * 2;  // bytes per key
     unsigned grest[LW];  // per-lane byte offset apart from the key term
     int gkey[LW];        // key offset of this lane's row inside the stage
 #pragma unroll
@@ -138,14 +145,14 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
         char* dst = reinterpret_cast<char*>(sStage + buf * STAGE) + wave * LW * 1024;
 #pragma unroll
         for (int c = 0; c < LW; ++c)  // rows past the end of the sequence are clamped (their keys are masked)
-            direct_load_16(gsrc, grest[c] + (unsigned)min(jb + gkey[c], T - 1) * (D * 2), dst + c * 1024);
+            direct_load_16(gsrc, grest[c] + (unsigned)min(jb + gkey[c], T - 1) * gpitch2, dst + c * 1024);
     };
     // the round's K2 / V2 rows RPR m .. RPR m + 3: one 1 KB load per tensor
     auto issue_round = [&](int m, int buf) {
         if (wave < 2) {
             int ln = lane;
             asm volatile("" : "+v"(ln));
-            const unsigned off = (unsigned)min(m * RPR + (ln >> 4), T - 1) * (D * 2) + (ln & 15) * 16;
+            const unsigned off = (unsigned)min(m * RPR + (ln >> 4), T - 1) * ((wave ? pV2 : pK2) * 2) + (ln & 15) * 16;
             direct_load_16(uniform_ptr(wave ? V2 : K2), off, (wave ? sVr : sKr) + buf * RPR * D);
         }
     };
@@ -153,9 +160,9 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_q16_kernel(BwdParams<E> p) {
     // ---- prologue
     for (int idx = tid; idx < BQ * D; idx += NTH) {
         const int r = idx / D, d = idx % D;
-        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
-        sQb[r * LDK + d] = p.q[off];
-        sOb[r * LDK + d] = p.d_o[off];
+        const unsigned row = (unsigned)min(q0 + r, T - 1);
+        sQb[r * LDK + d] = Qs[(size_t)row * pQ + d];
+        sOb[r * LDK + d] = Os[(size_t)row * pO + d];
     }
     // (round, step) of the stage fetched next: the sequence the main loop walks, wrapping to the first round after
     // the last (those fetches are never used)

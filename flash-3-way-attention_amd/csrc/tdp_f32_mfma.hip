@@ -35,6 +35,10 @@ __device__ __forceinline__ f32x16 mma_f32(float a, float b, f32x16 c) {
 template <typename E>
 struct F32Params {
     const E *q, *ka, *kb, *va, *vb;  // streamed = (ka, va), rows = (kb, vb)
+    // where these five and d_o lie: H heads per batch entry and each tensor's strides (dense tensors: H = 1 and
+    // sb = T D, st = D); the outputs are dense
+    int H;
+    TensorAt at_q, at_ka, at_kb, at_va, at_vb, at_do;
     E* o;
     float* lse;
     // STATS mode (the 16-bit backward's fp32 tiles): O is not written; lse receives the fp32 log-sum-exp of the
@@ -76,17 +80,18 @@ struct StageE {
 };
 template <typename E, int D>
 __device__ __forceinline__ void stage_fetch_e(StageE<E, D>& r, const E* __restrict__ ka, const E* __restrict__ va, int a0,
-                                              int T) {
+                                              int T, unsigned pitch_ka, unsigned pitch_va) {
     using S = StageE<E, D>;
     constexpr int kVec = D / S::VE;
     const int t = threadIdx.x & 255;
     const E* src = threadIdx.x < 256 ? ka : va;
+    const unsigned pitch = threadIdx.x < 256 ? pitch_ka : pitch_va;
 #pragma unroll
     for (int i = 0; i < S::kPer; ++i) {
         const int idx = t + i * 256;
         if (idx < S::kPieces) {
             const int row = idx / kVec, c = idx % kVec;
-            r.x[i] = *reinterpret_cast<const uint4*>(src + (size_t)min(a0 + row, T - 1) * D + c * S::VE);
+            r.x[i] = *reinterpret_cast<const uint4*>(src + (size_t)min(a0 + row, T - 1) * pitch + c * S::VE);
         }
     }
 }
@@ -132,17 +137,20 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
     const size_t base = (size_t)bh * T * D;
-    const E* __restrict__ KA = p.ka + base;
-    const E* __restrict__ VA = p.va + base;
-    const E* __restrict__ KB = p.kb + base;
-    const E* __restrict__ VB = p.vb + base;
+    const int b_ = bh / p.H, h_ = bh % p.H;
+    auto slice = [&](const E* t, const TensorAt& at) { return t + (size_t)b_ * at.sb + (size_t)h_ * at.sh; };
+    const E* __restrict__ KA = slice(p.ka, p.at_ka);
+    const E* __restrict__ VA = slice(p.va, p.at_va);
+    const E* __restrict__ KB = slice(p.kb, p.at_kb);
+    const E* __restrict__ VB = slice(p.vb, p.at_vb);
+    const E* __restrict__ Qs = slice(p.q, p.at_q);
     const TdpMask mask = p.mask;
 
     const int q0 = qt * 32, q1 = min(T - 1, q0 + 31);
     const int q = q0 + n;  // this lane's query (column of every tile)
     for (int idx = tid; idx < 32 * D; idx += 512) {
         const int r = idx / D, d = idx % D;
-        sQ[r * LD + d] = (float)p.q[base + (size_t)min(q0 + r, T - 1) * D + d] * p.scale_log2;
+        sQ[r * LD + d] = (float)Qs[(size_t)min(q0 + r, T - 1) * p.at_q.st + d] * p.scale_log2;
     }
 
     const Range rows = row_range(mask, q0, q1, T);
@@ -174,12 +182,12 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
         __syncthreads();  // previous round: everyone is done with sKb / sVb and the stage buffers
         for (int idx = tid; idx < NW * D; idx += 512) {
             const int r = idx / D, d = idx % D;
-            const size_t off = (size_t)min(m * NW + r, T - 1) * D + d;
-            sKb[idx] = (float)KB[off];
-            sVb[idx] = (float)VB[off];
+            const size_t row = (size_t)min(m * NW + r, T - 1);
+            sKb[idx] = (float)KB[row * p.at_kb.st + d];
+            sVb[idx] = (float)VB[row * p.at_vb.st + d];
         }
         if (st_lo <= st_hi) {
-            stage_fetch_e<E, D>(regs, KA, VA, st_lo * 32, T);
+            stage_fetch_e<E, D>(regs, KA, VA, st_lo * 32, T, p.at_ka.st, p.at_va.st);
             stage_store_e<E, D>(regs, sK, sV);
         }
         __syncthreads();
@@ -202,7 +210,7 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
             const float* cK = sK + buf * 32 * LD;
             const float* cV = sV + buf * 32 * LD;
             const bool more = st < st_hi;
-            if (more) stage_fetch_e<E, D>(regs, KA, VA, (st + 1) * 32, T);
+            if (more) stage_fetch_e<E, D>(regs, KA, VA, (st + 1) * 32, T, p.at_ka.st, p.at_va.st);
             const int a0 = st * 32;
             if (row_ok && a0 + 31 >= mine.lo && a0 <= mine.hi) {
                 f32x16 s;
@@ -293,7 +301,7 @@ __global__ __launch_bounds__(512) void tdp_f32_fwd_kernel(F32Params<E> p) {
         // Delta[q] = sum_d dO[q, d] O[q, d] with O in fp32 (lane n of wave 0 walks its query's row)
         if (wave == 0 && g == 0 && q < T) {
             float dsum = 0.f;
-            for (int d = 0; d < D; ++d) dsum += (float)p.d_o[base + (size_t)q * D + d] * sO[d * 33 + n];
+            for (int d = 0; d < D; ++d) dsum += (float)slice(p.d_o, p.at_do)[(size_t)q * p.at_do.st + d] * sO[d * 33 + n];
             if (p.split_rounds) {
                 float* part = p.delta + (((size_t)bh * 32 + n) * p.split_rounds + blockIdx.y) * 3;
                 part[0] = M; part[1] = L; part[2] = dsum;
@@ -342,6 +350,8 @@ constexpr int kF32FixedBias = 36;
 template <typename E>
 struct F32BwdParams {
     const E *q, *d_o, *ka, *kb, *va, *vb;
+    int H;  // layouts of the six inputs, as in F32Params
+    TensorAt at_q, at_ka, at_kb, at_va, at_vb, at_do;
     const float *lse, *delta;
     E* dq;                 // WITH_DQ, when acc_q is null
     void *acc_k, *acc_v;   // [BH][T][D] gradients of the rows: fixed point (long long) or float
@@ -395,10 +405,13 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = p.T;
     const size_t base = (size_t)bh * T * D;
-    const E* __restrict__ KA = p.ka + base;
-    const E* __restrict__ VA = p.va + base;
-    const E* __restrict__ KB = p.kb + base;
-    const E* __restrict__ VB = p.vb + base;
+    const int b_ = bh / p.H, h_ = bh % p.H;
+    auto slice = [&](const E* t, const TensorAt& at) { return t + (size_t)b_ * at.sb + (size_t)h_ * at.sh; };
+    const E* __restrict__ KA = slice(p.ka, p.at_ka);
+    const E* __restrict__ VA = slice(p.va, p.at_va);
+    const E* __restrict__ KB = slice(p.kb, p.at_kb);
+    const E* __restrict__ VB = slice(p.vb, p.at_vb);
+    const E* __restrict__ Qs = slice(p.q, p.at_q);
     const TdpMask mask = p.mask;
     const float scale_log2 = p.alpha * kLog2e;
     const float fscale = p.scale_parts ? fixed_scale_value(fixed_scale_field(p.scale_parts, bh, p.scale_bias)) : 0.f;
@@ -414,9 +427,9 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
     if (parts > 1 && m_lo > m_hi) return;  // fewer rounds than workgroups: nothing to add (uniform, before any barrier)
     for (int idx = tid; idx < 32 * D; idx += 512) {
         const int r = idx / D, d = idx % D;
-        const size_t off = base + (size_t)min(q0 + r, T - 1) * D + d;
-        sQ[r * LD + d] = (float)p.q[off] * scale_log2;
-        sDO[r * LD + d] = (float)p.d_o[off];
+        const size_t row = (size_t)min(q0 + r, T - 1);
+        sQ[r * LD + d] = (float)Qs[row * p.at_q.st + d] * scale_log2;
+        sDO[r * LD + d] = (float)slice(p.d_o, p.at_do)[row * p.at_do.st + d];
     }
     // a query past the end of the sequence gets a huge LSE: its P is exactly 0
     float lse2 = 1.0e30f, delta = 0.f;
@@ -456,12 +469,12 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
         __syncthreads();
         for (int idx = tid; idx < NW * D; idx += 512) {
             const int r = idx / D, d = idx % D;
-            const size_t off = (size_t)min(m * NW + r, T - 1) * D + d;
-            sKb[idx] = (float)KB[off];
-            sVb[idx] = (float)VB[off];
+            const size_t row = (size_t)min(m * NW + r, T - 1);
+            sKb[idx] = (float)KB[row * p.at_kb.st + d];
+            sVb[idx] = (float)VB[row * p.at_vb.st + d];
         }
         if (st_lo <= st_hi) {
-            stage_fetch_e<E, D>(regs, KA, VA, st_lo * 32, T);
+            stage_fetch_e<E, D>(regs, KA, VA, st_lo * 32, T, p.at_ka.st, p.at_va.st);
             stage_store_e<E, D>(regs, sK, sV);
         }
         __syncthreads();
@@ -486,7 +499,7 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
             const float* cK = sK + buf * 32 * LD;
             const float* cV = sV + buf * 32 * LD;
             const bool more = st < st_hi;
-            if (more) stage_fetch_e<E, D>(regs, KA, VA, (st + 1) * 32, T);
+            if (more) stage_fetch_e<E, D>(regs, KA, VA, (st + 1) * 32, T, p.at_ka.st, p.at_va.st);
             const int a0 = st * 32;
             if (row_ok && a0 + 31 >= mine.lo && a0 <= mine.hi) {
                 f32x16 s, dp;
@@ -645,11 +658,32 @@ constexpr size_t f32_bwd_smem() {
     return sizeof(float) * (size_t)(4 * 32 * (D + 1) + 2 * 32 * (D + 1) + 2 * kF32Waves * D);
 }
 
+// where the six inputs lie (F32Params::H and at_*)
+struct InputsAt {
+    int H;
+    TensorAt q, d_o, k1, u, k2, v2;
+};
+InputsAt dense_inputs(int T, int D) {
+    const TensorAt d = dense_at(1, T, D);
+    return InputsAt{1, d, d, d, d, d, d};
+}
+InputsAt inputs_of(const FirstTileArgs& a) {
+    if (a.H <= 0) return dense_inputs(a.T, a.D);
+    return InputsAt{a.H, a.at_q, a.at_do, a.at_k1, dense_at(a.H, a.T, a.D), a.at_k2, a.at_v2};
+}
+// streamed = (K1, U), rows = (K2, V2), or the two exchanged
+template <typename P>
+void place_inputs(P& p, const InputsAt& at, bool exchanged) {
+    p.H = at.H; p.at_q = at.q; p.at_do = at.d_o;
+    p.at_ka = exchanged ? at.k2 : at.k1; p.at_va = exchanged ? at.v2 : at.u;
+    p.at_kb = exchanged ? at.k1 : at.k2; p.at_vb = exchanged ? at.u : at.v2;
+}
+
 // both launches of the backward over query tiles 0 .. nqt - 1
 template <typename E, int D>
 hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, const E* k2, const E* v2, void* acc_k2,
                                 void* acc_v2, void* acc_k1, void* acc_u, const TdpMask& natural, bool want_q,
-                                bool want_k2, bool want_k1, hipStream_t st) {
+                                bool want_k2, bool want_k1, hipStream_t st, const InputsAt& at) {
     // D = 128: the launch that also accumulates dQ produces 64 gradient columns per workgroup (both column halves
     // form S and dP); without the dQ accumulators a workgroup holds all 128 columns and forms them once
     constexpr int DOUT = D > 64 ? 64 : D, DOUT_NODQ = D;
@@ -664,12 +698,14 @@ hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, cons
     const dim3 grid(8 * xcd_slots(p.BH, p.nqt), D / DOUT, p.acc_q ? parts : 1), grid_nodq(8 * xcd_slots(p.BH, p.nqt), D / DOUT_NODQ, parts);
     // rows = (K2, V2), streamed = (K1, U): dQ, dK2, dV2
     p.ka = k1; p.va = u; p.kb = k2; p.vb = v2;
+    place_inputs(p, at, false);
     p.acc_k = acc_k2; p.acc_v = acc_v2; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
     p.mask = natural;
     if (want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(512), smem, st, p);
     else if (want_k2) hipLaunchKernelGGL(kern_nodq, grid_nodq, dim3(512), smem, st, p);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU (the mask with the two key indices exchanged)
     p.ka = k2; p.va = v2; p.kb = k1; p.vb = u;
+    place_inputs(p, at, true);
     p.acc_k = acc_k1; p.acc_v = acc_u; p.bit_k = kPoisonDK1; p.bit_v = kPoisonDU;
     p.mask = TdpMask{natural.causal, natural.wb, natural.wa, natural.rab, natural.lab};
     if (want_k1) hipLaunchKernelGGL(kern_nodq, grid_nodq, dim3(512), smem, st, p);
@@ -700,7 +736,7 @@ hipError_t launch_f32_bwd(const GenericTdpArgs& a, long long* acc, hipStream_t s
     hipLaunchKernelGGL(f32_scale_kernel, dim3(kScaleParts, a.BH), dim3(256), 0, st, a.d_o, parts, (size_t)a.T * D);
     const TdpMask natural{a.causal, a.k1_window, a.k2_window, a.kk_left, a.kk_right};
     if (hipError_t e = launch_f32_bwd_tiles<float, D>(p, a.k1, a.u, a.k2, a.v2, acc, acc + n, acc + 2 * n, acc + 3 * n,
-                                                      natural, want_q, want_k2, want_k1, st);
+                                                      natural, want_q, want_k2, want_k1, st, dense_inputs(a.T, D));
         e != hipSuccess)
         return e;
     size_t gf = (n + 255) / 256;
@@ -726,6 +762,7 @@ template <int D>
 hipError_t launch_f32_fwd(const GenericTdpArgs& a, hipStream_t st) {
     F32Params<float> p{};
     p.q = a.q; p.ka = a.k1; p.kb = a.k2; p.va = a.u; p.vb = a.v2;
+    place_inputs(p, dense_inputs(a.T, D), false);
     p.o = a.o; p.lse = a.lse;
     p.d_o = nullptr; p.delta = nullptr; p.split_rounds = 0; p.zero_ptr = nullptr; p.zero_words = 0;
     p.T = a.T; p.BH = a.BH; p.nqt = (a.T + 31) / 32;
@@ -756,6 +793,7 @@ template <typename E, int D>
 static hipError_t launch_stats(const FirstTileArgs& a, hipStream_t st) {
     F32Params<E> p{};
     p.q = (const E*)a.q; p.ka = (const E*)a.k1; p.kb = (const E*)a.k2; p.va = (const E*)a.u; p.vb = (const E*)a.v2;
+    place_inputs(p, inputs_of(a), false);
     p.o = nullptr; p.lse = a.lse_f32; p.d_o = (const E*)a.d_o; p.delta = a.delta_f32;
     p.split_rounds = 0; p.zero_ptr = nullptr; p.zero_words = 0;
     p.T = a.T; p.BH = a.BH; p.nqt = a.tiles;
@@ -779,6 +817,7 @@ static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
     {
         F32Params<E> p{};
         p.q = (const E*)a.q; p.ka = (const E*)a.k1; p.kb = (const E*)a.k2; p.va = (const E*)a.u; p.vb = (const E*)a.v2;
+        place_inputs(p, inputs_of(a), false);
         p.o = nullptr; p.lse = nullptr; p.d_o = (const E*)a.d_o; p.delta = a.delta_f32;
         p.split_rounds = rounds;
         p.zero_ptr = own_dq_acc ? (unsigned*)a.dq0_acc : nullptr;
@@ -799,8 +838,10 @@ static hipError_t launch_tile0_split(const FirstTileArgs& a, hipStream_t st) {
     r0.T = a.T; r0.BH = a.BH; r0.nqt = 1; r0.alpha = a.alpha;
     F32BwdParams<E> r1 = r0;
     r0.ka = (const E*)a.k1; r0.va = (const E*)a.u; r0.kb = (const E*)a.k2; r0.vb = (const E*)a.v2;
+    place_inputs(r0, inputs_of(a), false);
     r0.acc_k = a.acc_k2; r0.acc_v = a.acc_v2; r0.bit_k = kPoisonDK2; r0.bit_v = kPoisonDV2; r0.mask = natural;
     r1.ka = (const E*)a.k2; r1.va = (const E*)a.v2; r1.kb = (const E*)a.k1; r1.vb = (const E*)a.u;
+    place_inputs(r1, inputs_of(a), true);
     r1.acc_k = a.acc_k1; r1.acc_v = a.acc_u; r1.bit_k = kPoisonDK1; r1.bit_v = kPoisonDU;
     r1.mask = TdpMask{natural.causal, natural.wb, natural.wa, natural.rab, natural.lab};
     const int roles = ((a.want_q || a.want_k2) ? 1 : 0) | (a.want_k1 ? 2 : 0) | (a.want_q ? 4 : 0);
@@ -833,11 +874,11 @@ static hipError_t first_tile_typed(const FirstTileArgs& a, hipStream_t st) {
     const E *k1 = (const E*)a.k1, *u = (const E*)a.u, *k2 = (const E*)a.k2, *v2 = (const E*)a.v2;
     const bool wq = a.want_q, wk2 = a.want_k2, wk1 = a.want_k1;
     if (a.D == 32)
-        return launch_f32_bwd_tiles<E, 32>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st);
+        return launch_f32_bwd_tiles<E, 32>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st, inputs_of(a));
     if (a.D == 64)
-        return launch_f32_bwd_tiles<E, 64>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st);
+        return launch_f32_bwd_tiles<E, 64>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st, inputs_of(a));
     if (a.D == 128)
-        return launch_f32_bwd_tiles<E, 128>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st);
+        return launch_f32_bwd_tiles<E, 128>(p, k1, u, k2, v2, a.acc_k2, a.acc_v2, a.acc_k1, a.acc_u, natural, wq, wk2, wk1, st, inputs_of(a));
     return hipErrorInvalidValue;
 }
 hipError_t f32_mfma_tdp_bwd_first_tile(const FirstTileArgs& a, hipStream_t st) {

@@ -159,6 +159,51 @@ def test_triple_dot_forward_reads_the_views_in_place():
     del fused
 
 
+@pytest.mark.parametrize("shape,windows,flags", [((2, 8, 512, 64), (None,) * 4, 0), ((1, 4, 384, 128), (None,) * 4, 0),
+                                                 ((2, 4, 320, 64), (100, 64, 33, 16), 0), ((1, 4, 256, 32), (None,) * 4, 0),
+                                                 ((1, 4, 200, 64), (None,) * 4, 8)])
+def test_triple_dot_backward_reads_the_views_in_place(shape, windows, flags):
+    """The 16-bit matrix-core backward takes slices of a fused projection and a transposed dO without a copy: its
+    workspace is the dense call's, the peak of device memory over the call is the gradients plus that workspace, and
+    every gradient is bitwise what the dense call returns (the D = 64 kernel, the 16-query kernel at D = 128, the banded
+    kernels, D = 32, split operands; the first query tile runs on the fp32 kernels, which take the strides too)."""
+    from flash_trittention import _lib, _ops
+
+    print(f"case strided triple-dot backward in place {shape} {windows} flags={flags}", flush=True)
+    B, H, T, D = shape
+    views, fused = fused_views(B, H, T, D, torch.bfloat16, seed=41)
+    d_o = bthd_view(B, H, T, D, torch.bfloat16, seed=42)
+    w = [T if x is None else x for x in windows]
+    lay, lay_do = _lib.layouts(views), _lib.layouts([d_o])
+    args = (B, H, T, D, _lib.TRITT_BF16, 1, *w, flags)
+    api = _lib.lib()
+    plain = api.tritt_tdp_bwd_workspace_bytes(*args)
+    assert api.tritt_tdp_bwd_strided_workspace_bytes(*args, lay, lay_do) == (plain + 255) // 256 * 256
+    n_bytes = B * H * T * D * 2
+    o, lse = _ops.tdp_fwd_impl(*views, 1 / 8, True, *w, flags)
+    _ops.tdp_bwd_impl(*views, o, lse, d_o, 1 / 8, True, *w, flags, 31)  # first call: kernel attributes, allocator pools
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    grads = _ops.tdp_bwd_impl(*views, o, lse, d_o, 1 / 8, True, *w, flags, 31)
+    torch.cuda.synchronize()
+    grown = torch.cuda.max_memory_allocated() - before
+    # the allocator rounds a large block up to 2 MiB; six gathered views would add 6 n_bytes
+    assert grown < 5 * n_bytes + plain + (2 << 20) + n_bytes, (grown, plain, n_bytes)
+    dense = [v.contiguous() for v in views]
+    o_d, lse_d = _ops.tdp_fwd_impl(*dense, 1 / 8, True, *w, flags)
+    assert torch.equal(o, o_d) and torch.equal(lse, lse_d)
+    grads_d = _ops.tdp_bwd_impl(*dense, o_d, lse_d, d_o.contiguous(), 1 / 8, True, *w, flags, 31)
+    for name, a, b in zip(util.NAMES, grads, grads_d):
+        assert torch.equal(a, b), name
+    # a dense dO with strided inputs, and the other way round
+    for ins, g in ((views, d_o.contiguous()), (dense, d_o)):
+        mixed = _ops.tdp_bwd_impl(*ins, o, lse, g, 1 / 8, True, *w, flags, 31)
+        for name, a, b in zip(util.NAMES, mixed, grads_d):
+            assert torch.equal(a, b), name
+    del fused
+
+
 def test_dot_product_sum_reads_the_views_in_place():
     """The 16-bit matrix-core kernels of dot-product-sum take [B,T,H,D] tensors transposed, and dO likewise, without a
     copy: forward and backward ask for the dense calls' workspaces, and the peak of device memory over each call is
