@@ -198,14 +198,21 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
  * order (NULL: all dense); `d_o_layout` to the one of dO (NULL: dense).  Strides are non-negative multiples of 16
  * bytes (8 elements of a 16-bit type, 4 of fp32), the row stride below 2^31 elements, pointers 16-byte aligned as
  * before; else TRITT_ERR_INVALID.  Outputs (o, lse, the gradients) and the saved `o` are dense.
- *   tritt_tdp_fwd_strided on the 16-bit matrix-core path (see tritt_tdp_fwd) reads the views in place: V1 through
- *     the SiLU/transpose pass it makes anyway, Q, K1, K2 and V2 inside the main kernel when the four share one layout.
- *   Everywhere else (the backward calls, dot-product-sum, fp32 tensors, four differing layouts) the views that are
- *     not dense are first gathered into the tail of the workspace by one launch for all of them, and the dense
- *     code runs on the copies: one read and one write of each such tensor (B=4 H=8 T=1024 D=64: 12 us for six
- *     tensors, against 11 ms of triple-dot backward), no allocation, no per-tensor launches.
- * The *_strided_workspace_bytes queries take the same layouts and return the dense call's size plus the room of those
- * copies; everything else is as in the dense call of the same name. */
+ * On the 16-bit matrix-core paths the views are read where they lie, and the workspace is the dense call's:
+ *   tritt_tdp_fwd_strided: V1 through the SiLU/transpose pass it makes anyway, Q, K1, K2 and V2 inside the main kernel
+ *     when the four share one layout (slices of one fused tensor, or tensors transposed alike);
+ *   tritt_tdp_bwd_strided: all six views, each on its own layout (the transposing pass, the row kernels, the fp32
+ *     kernels of the first query tile and the final pass take the strides);
+ *   tritt_dps_fwd_strided, tritt_dps_bwd_strided: all views, each on its own layout (the packing pass, the owner-tile
+ *     loads and the epilogues take the strides; broadcast views with a stride of zero included).
+ *   The triple-dot calls read in place only while T * stride_t stays below 2^31 elements and no view is a broadcast
+ *   along t.
+ * Everywhere else (fp32 tensors, head dimensions without a matrix-core kernel, a triple-dot forward whose four views
+ *   differ in layout) the views that are not dense are first gathered into the tail of the workspace by one launch for
+ *   all of them, and the dense code runs on the copies: one read and one write of each such tensor, no allocation,
+ *   no per-tensor launches.
+ * The *_strided_workspace_bytes queries take the same layouts and return the dense call's size plus the room of such
+ * copies where they are made; everything else is as in the dense call of the same name. */
 typedef struct tritt_layout {
     long long stride_b, stride_h, stride_t;
 } tritt_layout;
