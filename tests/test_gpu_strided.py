@@ -1,7 +1,7 @@
 """Strided [B,H,T,D] views at the C ABI (tritt_*_strided): a projection layer's [B,T,H,D] output transposed, slices of
 one fused [B,T,5,H,D] tensor, mixed layouts.  The reference accepts such views and copies them
-(triple_dot_product/flash_trittention.py:64-68; its test: tests/test_dot_product_sum.py:121-134); here the triple-dot
-forward reads them where they lie and the other calls gather them inside the library's workspace.
+(triple_dot_product/flash_trittention.py:64-68; its test: tests/test_dot_product_sum.py:121-134); here the 16-bit
+matrix-core kernels read them where they lie and the other paths gather them inside the library's workspace.
 
 Every case is held to two bars: the oracle at the dtype's tolerance, and the dense call on `.contiguous()` copies of
 the same views bit for bit (the same kernels see the same numbers)."""
