@@ -35,12 +35,16 @@ __device__ __forceinline__ void direct_load_16(const void* gbase, unsigned byte_
                  : "memory");
 }
 
-// the same with 4 bytes per lane: one instruction fills 256 consecutive bytes
+// the same with 4 bytes per lane: one instruction fills 256 consecutive bytes.  (Both wave-uniform operands are made
+// scalar here: callers that pick the destination from a ring slot do not always get them as scalars.)
 __device__ __forceinline__ void direct_load_4(const void* gbase, unsigned byte_off, void* lds_dst) {
-    const unsigned lds = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_dst;
+    const unsigned lds =
+        __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_dst);
+    const unsigned long long a = reinterpret_cast<unsigned long long>(gbase);
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                  :
-                 : "s"(lds), "v"(byte_off), "s"(gbase)
+                 : "s"(lds), "v"(byte_off), "s"(((unsigned long long)hi << 32) | lo)
                  : "memory");
 }
 

@@ -775,6 +775,8 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
     }  // owner tiles of this workgroup
 }
 
+#include "dps_bwd_shared.hpp"
+
 // --------------------------------------------------------------------------------------- prep
 // Operand-packed copies of the inputs (U = SiLU(V1); rows past T are written as zeros), U row-major, and
 // the padded per-row vectors of the backward (LSE in log2 units, Delta = rowsum(dO * O)).  Null
@@ -1055,8 +1057,33 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     o.dk_f32 = (float*)(ws + l.dk2p);
     o.r_f32 = (const float*)(ws + l.r); o.v2 = caller_view<E, SV>(a, a.v2, a.lv2); o.dv2 = (E*)a.dv2;
     o.dr = (E*)(ws + l.dr); o.dr_p1 = (E*)(ws + l.drp1); o.dr_p2 = (E*)(ws + l.drp2); o.delta1 = (float*)(ws + l.delta1);
-    hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_out), dim3(64 * kW), (row_smem<D, kW>()), st, o);
-    hipLaunchKernelGGL(kcol_link, attn_grid(a, Tp, pair_out), dim3(64 * kW), (col_smem<D, kW>()), st, o);
+    // Large grids: the kernels whose workgroups own 128 rows and share the streamed tiles through LDS
+    // (dps_bwd_shared.hpp), as the forward passes do (run_fwd).  They pay from 512 such workgroups on; measured
+    // backward, bf16 D = 64, one owner tile per workgroup -> shared tiles: B=8 H=16 T=2048 1650 -> 972 us, B=4 H=8
+    // T=4096 1245 -> 825 us, B=8 H=16 T=1024 510 -> 376 us, B=4 H=8 T=2048 (512 workgroups) 387 -> 313 us, B=1 H=8
+    // T=8192 (512) 1040 -> 1000 us, but B=1 H=8 T=4096 (256) 306 -> 506 us and B=4 H=8 T=1024 (256) 136 -> 175 us;
+    // D = 128, B=4 H=8 T=4096: 2120 -> 1935 us.
+    constexpr int kSW = 4, kRowNS = 4, kColNS = D > 64 ? 3 : 4;
+    using RowShape = BwdSharedShape<D, kSW, kRowNS, 3>;
+    using ColShape = BwdSharedShape<D, kSW, kColNS, 4>;
+    const int owners = (Tp / 32 + kSW - 1) / kSW;
+    bool shared = false;
+    if constexpr (D >= 64) shared = knobs().dps_shared ? knobs().dps_shared > 0 : (long long)a.BH * owners >= 512;
+    const dim3 grid_shared(8 * xcd_slots(a.BH, owners));
+    if constexpr (D >= 64) {
+        if (shared) {
+            auto srow_out = attn_bwd_row_shared_kernel<E, D, kSW, kRowNS, true, SV>;
+            auto scol_out = attn_bwd_col_shared_kernel<E, D, kSW, kColNS, true, SV>;
+            if (e = allow_smem(srow_out, RowShape::smem); e != hipSuccess) return e;
+            if (e = allow_smem(scol_out, ColShape::smem); e != hipSuccess) return e;
+            hipLaunchKernelGGL(srow_out, grid_shared, dim3(64 * kSW), RowShape::smem, st, o);
+            hipLaunchKernelGGL(scol_out, grid_shared, dim3(64 * kSW), ColShape::smem, st, o);
+        }
+    }
+    if (!shared) {
+        hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_out), dim3(64 * kW), (row_smem<D, kW>()), st, o);
+        hipLaunchKernelGGL(kcol_link, attn_grid(a, Tp, pair_out), dim3(64 * kW), (col_smem<D, kW>()), st, o);
+    }
 
     // inner pass: X = K2, G = dR, K = K1, V = U
     AttnBwdP<E, SV> i{};
@@ -1070,8 +1097,20 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     i.pair = pair_in;
     i.addend = (const float*)(ws + l.dk2p); i.dx = (E*)a.dk2;
     i.dk = (E*)a.dk1; i.v1 = caller_view<E, SV>(a, a.v1, a.lv1); i.dv = (E*)a.dv1;
-    hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_in), dim3(64 * kW), (row_smem<D, kW>()), st, i);
-    hipLaunchKernelGGL(kcol, attn_grid(a, Tp, pair_in), dim3(64 * kW), (col_smem<D, kW>()), st, i);
+    if constexpr (D >= 64) {
+        if (shared) {
+            auto srow_in = attn_bwd_row_shared_kernel<E, D, kSW, kRowNS, false, SV>;
+            auto scol_in = attn_bwd_col_shared_kernel<E, D, kSW, kColNS, false, SV>;
+            if (e = allow_smem(srow_in, RowShape::smem); e != hipSuccess) return e;
+            if (e = allow_smem(scol_in, ColShape::smem); e != hipSuccess) return e;
+            hipLaunchKernelGGL(srow_in, grid_shared, dim3(64 * kSW), RowShape::smem, st, i);
+            hipLaunchKernelGGL(scol_in, grid_shared, dim3(64 * kSW), ColShape::smem, st, i);
+        }
+    }
+    if (!shared) {
+        hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_in), dim3(64 * kW), (row_smem<D, kW>()), st, i);
+        hipLaunchKernelGGL(kcol, attn_grid(a, Tp, pair_in), dim3(64 * kW), (col_smem<D, kW>()), st, i);
+    }
     return hipGetLastError();
 }
 

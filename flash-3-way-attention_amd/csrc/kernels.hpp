@@ -15,7 +15,7 @@ struct Knobs {
     int f32_valu;        // TRITT_TUNE_F32_VALU: 1 = fp32 tensors take the VALU kernels at every head dimension
     int dps_waves;       // TRITT_TUNE_DPS_WAVES: waves per workgroup of the dot-product-sum MFMA kernels at D = 64 (2 | 4)
     int dps_pair;        // TRITT_TUNE_DPS_PAIR: 1 / -1 = owner tiles always / never paired in those kernels
-    int dps_shared;      // TRITT_TUNE_DPS_SHARED: 1 / -1 = the shared-tile forward kernel always / never
+    int dps_shared;      // TRITT_TUNE_DPS_SHARED: 1 / -1 = the shared-tile dot-product-sum kernels always / never
 };
 Knobs knobs();
 

@@ -85,8 +85,9 @@ const char* tritt_status_string(int status);
  *   TRITT_TUNE_DPS_WAVES    waves per workgroup of the dot-product-sum MFMA kernels at D = 64: 2 | 4
  *   TRITT_TUNE_DPS_PAIR     dot-product-sum MFMA kernels: 1 = a workgroup always takes two owner tiles (a long and a
  *                           short one), -1 = never
- *   TRITT_TUNE_DPS_SHARED   dot-product-sum forward passes: 1 = always the kernel whose workgroups own 128 rows and share
- *                           the streamed tiles through LDS, -1 = never (0: from 1024 such workgroups on) */
+ *   TRITT_TUNE_DPS_SHARED   dot-product-sum on the 16-bit matrix cores: 1 = always the kernels whose workgroups own 128 rows
+ *                           and share the streamed tiles through LDS, -1 = never (0: the forward passes from 1024 such
+ *                           workgroups on, the backward kernels at D = 64 and 128 from 512 on) */
 enum { TRITT_TUNE_FWD_SPLITS = 0, TRITT_TUNE_FWD_BAND = 1, TRITT_TUNE_BWD_SPLITS = 2, TRITT_TUNE_BWD128_WAVES = 3,
        TRITT_TUNE_F32_VALU = 4, TRITT_TUNE_DPS_WAVES = 5, TRITT_TUNE_DPS_PAIR = 6, TRITT_TUNE_DPS_SHARED = 7,
        TRITT_TUNE_COUNT_ = 8 };

@@ -197,13 +197,13 @@ def test_paired_owner_tiles_change_nothing(T, D, k_diff, causal, waves, tune):
     (1, 3, 160, 128, 160, True, torch.bfloat16), (2, 2, 130, 32, 40, True, torch.bfloat16),
     (1, 2, 257, 64, 257, False, torch.bfloat16), (1, 1, 33, 64, 5, True, torch.float16),
     (1, 2, 128, 64, 0, True, torch.bfloat16), (1, 1, 1, 64, 1, True, torch.bfloat16)])
-def test_shared_tile_forward_kernel(B, H, T, D, k_diff, causal, dtype, tune):
-    """The forward kernel whose workgroups own 128 rows and read the streamed tiles from an LDS ring (the one large
-    grids take), forced on: output, LSE and, through the inner pass the backward runs again, all gradients against
-    the oracle; ragged lengths, bands narrower than a tile, no mask, one row, the three head dimensions."""
+def test_shared_tile_kernels(B, H, T, D, k_diff, causal, dtype, tune):
+    """The kernels whose workgroups own 128 rows and read the streamed tiles from an LDS ring (the ones large grids
+    take: forward at every head dimension, backward rows and columns at D = 64 and 128), forced on: output, LSE and
+    all gradients against the oracle; ragged lengths, bands narrower than a tile, no mask, one row."""
     from flash_trittention import _lib
 
-    print(f"case dps shared-tile forward B={B} H={H} T={T} D={D} k_diff={k_diff} causal={causal} {dtype}", flush=True)
+    print(f"case dps shared-tile kernels B={B} H={H} T={T} D={D} k_diff={k_diff} causal={causal} {dtype}", flush=True)
     inputs = orc.make_inputs(B, H, T, D, dtype, seed=T + D + k_diff)
     alpha = 1 / math.sqrt(D)
     tune(_lib.TUNE_DPS_SHARED, 1)
@@ -219,24 +219,33 @@ def test_shared_tile_forward_kernel(B, H, T, D, k_diff, causal, dtype, tune):
     util.assert_close("out vs the per-tile kernel", out, other[0].float().cpu(), rtol=2e-2, atol=1e-2)
 
 
-def test_large_grids_take_the_shared_tile_forward(tune):
-    """B=16 H=16 T=500 D=64 (1024 workgroups of 128 rows): the default dispatch is the shared-tile kernel, bitwise what
-    the knob forces, and it matches the oracle on the heads checked."""
+@pytest.mark.parametrize("B,H,fwd_shared", [(16, 16, True), (8, 16, False)])
+def test_large_grids_take_the_shared_tile_kernels(B, H, fwd_shared, tune):
+    """T=500 D=64: 1024 workgroups of 128 rows (B=16 H=16) send the forward passes and the backward kernels to the
+    shared-tile kernels, 512 (B=8 H=16) the backward kernels only.  The default dispatch is bitwise what the knob
+    forces for the kernels it picks, and matches the oracle on the heads checked."""
     from flash_trittention import _lib
 
-    B, H, T, D = 16, 16, 500, 64
+    T, D = 500, 64
     inputs = orc.make_inputs(B, H, T, D, torch.bfloat16, seed=77)
-    default = util.run_dps(inputs, 1 / 8, True, T, backward=False)
+    default = util.run_dps(inputs, 1 / 8, True, T)
     tune(_lib.TUNE_DPS_SHARED, 1)
-    forced = util.run_dps(inputs, 1 / 8, True, T, backward=False)
+    forced = util.run_dps(inputs, 1 / 8, True, T)
     tune(_lib.TUNE_DPS_SHARED, -1)
-    never = util.run_dps(inputs, 1 / 8, True, T, backward=False)
-    assert torch.equal(default[0], forced[0]) and torch.equal(default[1], forced[1])
-    assert not torch.equal(default[0], never[0])
-    for b, h in ((0, 0), (7, 9), (15, 15)):
-        z, lse, _ = util.oracle_dps([t[b:b + 1, h:h + 1] for t in inputs], 1 / 8, True, T)
+    never = util.run_dps(inputs, 1 / 8, True, T)
+    assert torch.equal(default[0], (forced if fwd_shared else never)[0])
+    assert torch.equal(default[1], (forced if fwd_shared else never)[1])
+    assert not torch.equal(forced[0], never[0])
+    if fwd_shared:  # every kernel of the default path is the forced one
+        for name, a, b in zip(util.NAMES, default[2], forced[2]):
+            assert torch.equal(a, b), name
+    assert not all(torch.equal(a, b) for a, b in zip(default[2], never[2]))
+    for b, h in ((0, 0), (B // 2, 9), (B - 1, H - 1)):
+        z, lse, grads = util.oracle_dps([t[b:b + 1, h:h + 1] for t in inputs], 1 / 8, True, T)
         util.assert_close("out", default[0][b:b + 1, h:h + 1], z, **LOWP)
         util.assert_close("m", default[1][b:b + 1, h:h + 1], lse, rtol=1e-3, atol=2e-2)
+        for name, a, ref in zip(util.NAMES, default[2], grads):
+            util.assert_close(name, a[b:b + 1, h:h + 1], ref, **LOWP)
 
 
 def test_rejects_mismatched_shapes():
