@@ -718,6 +718,10 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
             smem = bwdg_smem(64, 8, 64, true);
             kern_dq = tdp_bwd_rows_general_kernel<E, 64, true, 8, 64, true, true, SV>;
             kern_nodq = tdp_bwd_rows_general_kernel<E, 64, false, 8, 64, true, true, SV>;
+            if (!a.windowed) {
+                kern_dq = tdp_bwd_rows_general_kernel<E, 64, true, 8, 64, false, true, SV>;
+                kern_nodq = tdp_bwd_rows_general_kernel<E, 64, false, 8, 64, false, true, SV>;
+            }
         } else {
             return hipErrorInvalidValue;
         }
