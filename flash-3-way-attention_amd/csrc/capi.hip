@@ -419,6 +419,11 @@ int check_layout(const tritt_layout* l, int dtype) {
     if (l->stride_b % unit || l->stride_h % unit || l->stride_t % unit) return TRITT_ERR_INVALID;
     return TRITT_OK;
 }
+// a view's strides as the kernels take them (null: dense)
+TensorAt tensor_at(const tritt_layout* l, int H, int T, int D) {
+    if (!l) return dense_at(H, T, D);
+    return TensorAt{l->stride_b, l->stride_h, (unsigned)(T == 1 ? D : l->stride_t)};
+}
 bool same_layout(const tritt_layout& a, const tritt_layout& b) {
     return a.stride_b == b.stride_b && a.stride_h == b.stride_h && a.stride_t == b.stride_t;
 }
@@ -735,12 +740,11 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
 }
 
 // ---------------------------------------------------------------- strided entry points
-// The triple-dot forward on the 16-bit matrix-core path reads strided views in place: V1 always (the SiLU / transpose
-// pass takes its layout), the other four when they share one layout with a row stride the kernels' 32-bit field holds.
+// The triple-dot forward on the 16-bit matrix-core path reads strided views in place: V1 through the SiLU / transpose
+// pass, which takes its layout, the other four inside the main kernel (on one common layout, or each on its own: a
+// second instantiation), when every row stride fits the kernels' 32-bit field.
 static bool fwd_reads_in_place(const tritt_layout* l, int dtype, int T) {
     if (!l) return true;
-    for (int i : {1, 2, 4})
-        if (!same_layout(l[0], l[i])) return false;
     for (int i = 0; i < 5; ++i)
         // the kernels form row offsets in 32 bits; a row stride of 0 (a broadcast view) would read as "dense" in the
         // launch arguments
@@ -795,6 +799,16 @@ int tritt_tdp_fwd_strided(const void* q, const void* k1, const void* k2, const v
         if (!layout_dense(in_layouts + 3, B, H, T, D)) {
             a.v1_sb = in_layouts[3].stride_b; a.v1_sh = in_layouts[3].stride_h; a.v1_st = in_layouts[3].stride_t;
             if (T == 1) a.v1_st = D;
+        }
+        // K1, K2 or V2 laid out differently from Q: every tensor on its own layout
+        if (!same_layout(in_layouts[0], in_layouts[1]) || !same_layout(in_layouts[0], in_layouts[2]) ||
+            !same_layout(in_layouts[0], in_layouts[4])) {
+            a.many_views = 1;
+            a.at_k1 = tensor_at(in_layouts + 1, H, T, D); a.at_k2 = tensor_at(in_layouts + 2, H, T, D);
+            a.at_v2 = tensor_at(in_layouts + 4, H, T, D);
+            if (layout_dense(in_layouts, B, H, T, D)) {  // Q itself dense: its strides in (batch, head) terms
+                a.in_sb = (long long)H * T * D; a.in_sh = (long long)T * D; a.in_st = D;
+            }
         }
         return (int)mfma_tdp_fwd(a, (hipStream_t)stream);
     }
@@ -922,10 +936,6 @@ static bool bwd_reads_in_place(const tritt_layout* in, const tritt_layout* d_o, 
     for (int i = 0; in && i < 5; ++i)
         if (!fits(in + i)) return false;
     return fits(d_o);
-}
-static TensorAt tensor_at(const tritt_layout* l, int H, int T, int D) {
-    if (!l) return dense_at(H, T, D);
-    return TensorAt{l->stride_b, l->stride_h, (unsigned)(T == 1 ? D : l->stride_t)};
 }
 
 size_t tritt_tdp_bwd_strided_workspace_bytes(int B, int H, int T, int D, int dtype, int causal, int k1_window,

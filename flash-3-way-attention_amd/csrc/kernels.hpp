@@ -128,6 +128,9 @@ struct MfmaFwdArgs {
     // v1_* strides; H = heads (BH = batch * H).  in_st == 0 / v1_st == 0: dense [BH][T][D].  Row strides below 2^32.
     long long in_sb, in_sh, in_st, v1_sb, v1_sh, v1_st;
     int H;
+    // many_views != 0: K1, K2 and V2 lie on layouts of their own (at_k1, at_k2, at_v2; in_* is then Q's alone)
+    int many_views;
+    TensorAt at_k1, at_k2, at_v2;
 };
 bool mfma_tdp_split_supported(int D, int dtype_is_16bit);
 // needs BH, T, D, causal, windowed, split and the four windows of `a`

@@ -32,7 +32,7 @@ constexpr size_t band_smem_bytes(int nr) {
     return sizeof(uint16_t) * ((size_t)3 * nr * (D + 8) + (size_t)D * (nr + 8)) + sizeof(float) * (kBandQ * D + 8 * 32 + 5 * 16 * 64);
 }
 
-template <typename E, int D>
+template <typename E, int D, bool MV = false>
 __global__ __launch_bounds__(512, 2) void tdp_fwd_band_kernel(FwdParams<E> p, int NR) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -66,17 +66,21 @@ __global__ __launch_bounds__(512, 2) void tdp_fwd_band_kernel(FwdParams<E> p, in
 
     // ---- load the band ---------------------------------------------------------------------------
     {
-        const E* __restrict__ K1 = p.k1 + in_base;
-        const E* __restrict__ K2 = p.k2 + in_base;
-        const E* __restrict__ V2 = p.v2 + in_base;
+        auto slice = [&](const E* t, const TensorAt& at) {
+            return MV ? t + (size_t)(bh / p.H) * at.sb + (size_t)(bh % p.H) * at.sh : t + in_base;
+        };
+        const E* __restrict__ K1 = slice(p.k1, p.at_k1);
+        const E* __restrict__ K2 = slice(p.k2, p.at_k2);
+        const E* __restrict__ V2 = slice(p.v2, p.at_v2);
+        const unsigned st_k1 = MV ? p.at_k1.st : in_st, st_k2 = MV ? p.at_k2.st : in_st, st_v2 = MV ? p.at_v2.st : in_st;
         const E* __restrict__ UT = p.ut + (size_t)bh * D * p.Tp;
         const int row_chunks = NR * (D / 8);
         for (int c = tid; c < row_chunks; c += 512) {
             const int r = c / (D / 8), ch = c % (D / 8);
-            const size_t src = (size_t)((unsigned)min(rlo + r, T - 1) * in_st) + ch * 8;
-            const uint4 a = *reinterpret_cast<const uint4*>(K1 + src);
-            const uint4 b = *reinterpret_cast<const uint4*>(K2 + src);
-            const uint4 v = *reinterpret_cast<const uint4*>(V2 + src);
+            const unsigned row = (unsigned)min(rlo + r, T - 1);
+            const uint4 a = *reinterpret_cast<const uint4*>(K1 + (size_t)(row * st_k1) + ch * 8);
+            const uint4 b = *reinterpret_cast<const uint4*>(K2 + (size_t)(row * st_k2) + ch * 8);
+            const uint4 v = *reinterpret_cast<const uint4*>(V2 + (size_t)(row * st_v2) + ch * 8);
             *reinterpret_cast<uint4*>(sK1 + r * LDK + ch * 8) = a;
             *reinterpret_cast<uint4*>(sK2 + r * LDK + ch * 8) = b;
             *reinterpret_cast<uint4*>(sV2 + r * LDK + ch * 8) = v;

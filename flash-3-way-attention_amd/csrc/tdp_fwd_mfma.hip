@@ -43,6 +43,8 @@ struct FwdParams {
     long long in_sb, in_sh;
     unsigned in_st;
     int H;
+    // MV ("many views") instantiations only: K1, K2 and V2 on layouts of their own (in_* is then Q's)
+    TensorAt at_k1, at_k2, at_v2;
     E* o;
     E* o_res;  // SPLIT: the rounding residual of every output element, O(fp32) - O(16 bit), as a second tensor
     float* lse;
@@ -87,7 +89,9 @@ __device__ __forceinline__ constexpr float fast_row_sum_floor() {
 // kilobyte per tile and k-step, private to the wave).  The output is stored with its rounding residual (o_res), so
 // the backward's Delta = rowsum(dO * O) does not inherit the 16-bit rounding of O.  (P as a hi + lo pair in the
 // value product was measured as well: no effect on any gradient at scores spanning hundreds, 40 % more time.)
-template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false, bool SPLIT = false>
+// MV: Q, K1, K2 and V2 each on a layout of its own (FwdParams::at_*) instead of one common layout.
+template <typename E, int D, int NT, int WAVES, int MINW, int JS, bool WIN = false, bool MDIAG = false, bool SPLIT = false,
+          bool MV = false>
 __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParams<E> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
@@ -133,9 +137,13 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     const size_t in_base = (size_t)(bh / p.H) * p.in_sb + (size_t)(bh % p.H) * p.in_sh;
     const unsigned in_st = p.in_st;  // row stride of the inputs, elements; (T - 1) in_st + D fits 32 bits
     const E* __restrict__ Q = p.q + in_base;
-    const E* __restrict__ K1 = p.k1 + in_base;
-    const E* __restrict__ K2 = p.k2 + in_base;
-    const E* __restrict__ V2 = p.v2 + in_base;
+    auto slice = [&](const E* t, const TensorAt& at) {
+        return MV ? t + (size_t)(bh / p.H) * at.sb + (size_t)(bh % p.H) * at.sh : t + in_base;
+    };
+    const E* __restrict__ K1 = slice(p.k1, p.at_k1);
+    const E* __restrict__ K2 = slice(p.k2, p.at_k2);
+    const E* __restrict__ V2 = slice(p.v2, p.at_v2);
+    const unsigned st_k1 = MV ? p.at_k1.st : in_st, st_k2 = MV ? p.at_k2.st : in_st, st_v2 = MV ? p.at_v2.st : in_st;
     const E* __restrict__ UT = p.ut + (size_t)bh * D * p.Tp;
     float* sWw = sW + wave * 32;
 
@@ -177,7 +185,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     uint4 ra0, ra1, rb0, rb1, rkv0, rkv1;
     auto k1_chunk = [&](int item, int jb) {
         const int r = item / (D / 8), ch = item % (D / 8);
-        return reinterpret_cast<const uint4*>(K1 + (size_t)((unsigned)min(jb + r, T - 1) * in_st) + ch * 8);
+        return reinterpret_cast<const uint4*>(K1 + (size_t)((unsigned)min(jb + r, T - 1) * st_k1) + ch * 8);
     };
     auto ut_chunk = [&](int i2, int jb) {
         const int d = i2 / (JS / 8), cj = i2 % (JS / 8);
@@ -224,7 +232,7 @@ __global__ __launch_bounds__(64 * WAVES, MINW) void tdp_fwd_mfma_kernel(FwdParam
     auto kt_src = [&](int item, int kt) {
         const int which = item / (4 * D), rem = item % (4 * D);
         const int r = rem / (D / 8), ch = rem % (D / 8);
-        return reinterpret_cast<const uint4*>((which ? V2 : K2) + (size_t)((unsigned)min(kt * 32 + r, T - 1) * in_st) + ch * 8);
+        return reinterpret_cast<const uint4*>((which ? V2 : K2) + (size_t)((unsigned)min(kt * 32 + r, T - 1) * (which ? st_v2 : st_k2)) + ch * 8);
     };
     auto kt_dst = [&](int item, int buf) {
         const int which = item / (4 * D), rem = item % (4 * D);
@@ -977,7 +985,8 @@ static hipError_t launch_band(const MfmaFwdArgs& a, hipStream_t st) {
     p.part = nullptr;
     const int nr = band_rows(p.wa, p.wb);
     const size_t smem = band_smem_bytes<D>(nr);
-    auto kern = tdp_fwd_band_kernel<E, D>;
+    auto kern = a.many_views ? tdp_fwd_band_kernel<E, D, true> : tdp_fwd_band_kernel<E, D, false>;
+    p.at_k1 = a.at_k1; p.at_k2 = a.at_k2; p.at_v2 = a.at_v2;
     hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, p.nqt)), dim3(512), smem, st, p, nr);
@@ -1015,7 +1024,9 @@ static hipError_t launch(const MfmaFwdArgs& a, hipStream_t st) {
     p.splits = fwd_splits(a, BQ);
     p.part = reinterpret_cast<float*>(static_cast<char*>(a.ut) + ut_bytes(a.BH, a.T, D));
     constexpr size_t smem = fwd_smem_bytes<D, NT, WAVES, JS, SPLIT>();
-    auto kern = tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG, SPLIT>;
+    auto kern = a.many_views ? tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG, SPLIT, true>
+                             : tdp_fwd_mfma_kernel<E, D, NT, WAVES, MINW, JS, WIN, MDIAG, SPLIT, false>;
+    p.at_k1 = a.at_k1; p.at_k2 = a.at_k2; p.at_v2 = a.at_v2;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern), smem); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(8 * xcd_slots(a.BH, p.nqt) * p.splits), dim3(64 * WAVES), smem, st, p);
     if (p.splits > 1) {

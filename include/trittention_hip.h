@@ -201,15 +201,16 @@ int tritt_dps_bwd(const void* q, const void* k1, const void* k2, const void* v1,
  * before; else TRITT_ERR_INVALID.  Outputs (o, lse, the gradients) and the saved `o` are dense.
  * On the 16-bit matrix-core paths the views are read where they lie, and the workspace is the dense call's:
  *   tritt_tdp_fwd_strided: V1 through the SiLU/transpose pass it makes anyway, Q, K1, K2 and V2 inside the main kernel
- *     when the four share one layout (slices of one fused tensor, or tensors transposed alike);
+ *     (one instantiation for four tensors on a common layout: slices of one fused tensor, or tensors transposed alike;
+ *     another for a layout per tensor);
  *   tritt_tdp_bwd_strided: all six views, each on its own layout (the transposing pass, the row kernels, the fp32
  *     kernels of the first query tile and the final pass take the strides);
  *   tritt_dps_fwd_strided, tritt_dps_bwd_strided: all views, each on its own layout (the packing pass, the owner-tile
  *     loads and the epilogues take the strides; broadcast views with a stride of zero included).
  *   The triple-dot calls read in place only while T * stride_t stays below 2^31 elements and no view is a broadcast
  *   along t.
- * Everywhere else (fp32 tensors, head dimensions without a matrix-core kernel, a triple-dot forward whose four views
- *   differ in layout) the views that are not dense are first gathered into the tail of the workspace by one launch for
+ * Everywhere else (fp32 tensors, head dimensions without a matrix-core kernel, the two triple-dot limits just named)
+ *   the views that are not dense are first gathered into the tail of the workspace by one launch for
  *   all of them, and the dense code runs on the copies: one read and one write of each such tensor, no allocation,
  *   no per-tensor launches.
  * The *_strided_workspace_bytes queries take the same layouts and return the dense call's size plus the room of such

@@ -128,13 +128,23 @@ def test_triple_dot_forward_reads_the_views_in_place():
     args = (B, H, T, D, _lib.TRITT_BF16, 1, T, T, T, T, 0)
     plain = _lib.lib().tritt_tdp_fwd_workspace_bytes(*args)
     assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, lay) == (plain + 255) // 256 * 256
-    # four equal layouts and a dense V1 still need no copy; K2 on a layout of its own makes all five be gathered
+    # four equal layouts and a dense V1 need no copy; nor do tensors that each have a layout of their own (K2 from
+    # another projection, a dense Q): the kernel's second instantiation takes a layout per tensor
     mixed = [views[0], views[1], views[2], views[3].contiguous(), views[4]]
     assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(mixed)) == (plain + 255) // 256 * 256
-    odd = [views[0], views[1], bthd_view(B, H, T, D, torch.bfloat16, 4), views[3], views[4]]
+    odd = [views[0].contiguous(), views[1], bthd_view(B, H, T, D, torch.bfloat16, 4), views[3], views[4].contiguous()]
     n_bytes = B * H * T * D * 2
-    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(odd)) == \
+    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(odd)) == (plain + 255) // 256 * 256
+    o_odd, lse_odd = _ops.tdp_fwd_impl(*odd, 1 / 8, True, T, T, T, T, 0)
+    o_ref, lse_ref = _ops.tdp_fwd_impl(*(t.contiguous() for t in odd), 1 / 8, True, T, T, T, T, 0)
+    assert torch.equal(o_odd, o_ref) and torch.equal(lse_odd, lse_ref)
+    # a view that is a broadcast along t is gathered (its row stride of 0 would read as "dense" in the launch arguments)
+    flat = [views[0], views[1], views[2], views[3], views[4][:, :, :1].expand(B, H, T, D)]
+    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(flat)) == \
         (plain + 255) // 256 * 256 + 5 * n_bytes
+    o_flat, lse_flat = _ops.tdp_fwd_impl(*flat, 1 / 8, True, T, T, T, T, 0)
+    o_ref, lse_ref = _ops.tdp_fwd_impl(*(t.contiguous() for t in flat), 1 / 8, True, T, T, T, T, 0)
+    assert torch.equal(o_flat, o_ref) and torch.equal(lse_flat, lse_ref)
 
     _ops.tdp_fwd_impl(*views, 1 / 8, True, T, T, T, T, 0)  # first call: kernel attributes, allocator pools
     torch.cuda.synchronize()
@@ -157,6 +167,29 @@ def test_triple_dot_forward_reads_the_views_in_place():
     o_v, lse_v = _ops.tdp_fwd_impl(*only_v1, 1 / 8, True, T, T, T, T, 0)
     assert torch.equal(o_v, o_d) and torch.equal(lse_v, lse_d)
     del fused
+
+
+@pytest.mark.parametrize("shape,windows,flags", [((2, 3, 300, 64), (None,) * 4, 0), ((1, 5, 200, 128), (None,) * 4, 0),
+                                                 ((2, 2, 300, 64), (100, 64, 33, 16), 0), ((2, 2, 300, 64), (24, 22, 300, 300), 0),
+                                                 ((1, 3, 130, 32), (None,) * 4, 0), ((1, 4, 200, 64), (None,) * 4, 8)])
+def test_triple_dot_forward_with_a_layout_per_tensor(shape, windows, flags):
+    """Q dense, K1 and V2 slices of a fused tensor, K2 a transposed projection, V1 a slice: the forward's second
+    instantiation reads each where it lies (streaming, banded, band-resident and split-operand kernels, three head
+    dimensions): the dense call's workspace, bitwise the dense call's results."""
+    from flash_trittention import _lib, _ops
+
+    print(f"case strided triple-dot forward, a layout per tensor {shape} {windows} flags={flags}", flush=True)
+    B, H, T, D = shape
+    fused, keep = fused_views(B, H, T, D, torch.bfloat16, seed=51)
+    tensors = [fused[0].contiguous(), fused[1], bthd_view(B, H, T, D, torch.bfloat16, 52), fused[3], fused[4]]
+    w = [T if x is None else x for x in windows]
+    args = (B, H, T, D, _lib.TRITT_BF16, 1, *w, flags)
+    plain = _lib.lib().tritt_tdp_fwd_workspace_bytes(*args)
+    assert _lib.lib().tritt_tdp_fwd_strided_workspace_bytes(*args, _lib.layouts(tensors)) == (plain + 255) // 256 * 256
+    o, lse = _ops.tdp_fwd_impl(*tensors, 1 / 8, True, *w, flags)
+    o_d, lse_d = _ops.tdp_fwd_impl(*(t.contiguous() for t in tensors), 1 / 8, True, *w, flags)
+    assert torch.equal(o, o_d) and torch.equal(lse, lse_d)
+    del keep
 
 
 @pytest.mark.parametrize("shape,windows,flags", [((2, 8, 512, 64), (None,) * 4, 0), ((1, 4, 384, 128), (None,) * 4, 0),
