@@ -18,17 +18,6 @@ struct BwdSharedShape {
     static_assert(CH % kW == 0, "the blocks of a tile are dealt out evenly to the waves");
 };
 
-// 16 floats of a lane from a 32-float vector in LDS: element i is the value of key / row key_of(g, i)
-__device__ __forceinline__ void tile_vector(const float* sv, int g, float (&out)[16]) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const float4 v = *reinterpret_cast<const float4*>(sv + 16 * h + 8 * g + 4 * c);
-            out[8 * h + 4 * c] = v.x; out[8 * h + 4 * c + 1] = v.y; out[8 * h + 4 * c + 2] = v.z; out[8 * h + 4 * c + 3] = v.w;
-        }
-}
-
 // ------------------------------------------------------------------------------ rows: dX
 // streamed per tile: K in packing P1 (scores), V in packing P1 (dP), K in packing P2 (dX), the per-key bias
 template <typename E, int D, int kW, int kNS, bool BIAS, bool SV>

@@ -95,6 +95,17 @@ __device__ __forceinline__ void pack16(const float (&x)[16], typename Mma<E>::v8
         }
 }
 
+// 16 floats of a lane from a 32-float vector in LDS: element i is the value of key / row key_of(g, i)
+__device__ __forceinline__ void tile_vector(const float* sv, int g, float (&out)[16]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const float4 v = *reinterpret_cast<const float4*>(sv + 16 * h + 8 * g + 4 * c);
+            out[8 * h + 4 * c] = v.x; out[8 * h + 4 * c + 1] = v.y; out[8 * h + 4 * c + 2] = v.z; out[8 * h + 4 * c + 3] = v.w;
+        }
+}
+
 // pair (query-like row r, key-like row a) takes part
 __device__ __forceinline__ bool pair_ok(int T, int causal, int k_diff, int r, int a) {
     return (r < T) & (a < T) & ((!causal) | ((a <= r) & (r - a <= k_diff)));
@@ -540,11 +551,17 @@ __global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_
 }
 
 // --------------------------------------------------------------------------- backward, columns
-template <typename E, int D, int kW, bool LINK, bool SV>
-__global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_kernel(AttnBwdP<E, SV> p) {
+// RING: every wave fetches its streamed tiles into a two-slot LDS ring of its own (direct-to-LDS loads, one tile ahead)
+// and reads the MFMA operands and the rows' statistics from there at the point of use, instead of holding the next
+// tile in registers: the kernel then fits 256 registers and two waves per SIMD (D = 64: 36 KB of LDS per wave).
+template <int D>
+constexpr int col_ring_tile_bytes() { return 4 * (D / 16) * 1024 + 2 * 256; }
+template <typename E, int D, int kW, bool LINK, bool SV, bool RING = false>
+__global__ __launch_bounds__(64 * kW, ((D <= 32 || RING) ? 2 : 1)) void attn_bwd_col_mfma_kernel(AttnBwdP<E, SV> p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
+    constexpr int kTileBytes = col_ring_tile_bytes<D>();
     extern __shared__ __align__(16) char smem_raw[];
     float* sO = reinterpret_cast<float*>(smem_raw);  // [kW][D][kLdr]
     float* sB = sO + kW * D * kLdr;                  // [kW][32]  dbias partials
@@ -591,6 +608,83 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
         }
     float db = 0.f;
 
+    const int t_first = r_lo / 32 + wave, t_last = r_hi / 32;
+    if constexpr (RING) {
+        char* ring = smem_raw + wave * 2 * kTileBytes;  // the merge tiles alias the rings: barrier before they are written
+        const char* XPc = reinterpret_cast<const char*>(uniform_ptr(XP));
+        const char* GPc = reinterpret_cast<const char*>(uniform_ptr(GP));
+        const char* XP2c = reinterpret_cast<const char*>(uniform_ptr(XP2));
+        const char* GP2c = reinterpret_cast<const char*>(uniform_ptr(GP2));
+        auto fetch = [&](int t, int slot) {
+            char* dst = ring + __builtin_amdgcn_readfirstlane(slot * kTileBytes);
+            const size_t tile_off = (size_t)__builtin_amdgcn_readfirstlane(t) * KS * 1024;
+#pragma unroll
+            for (int c = 0; c < KS; ++c) {
+                direct_load_16(uniform_ptr(XPc + tile_off + c * 1024), lane * 16, dst + c * 1024);
+                direct_load_16(uniform_ptr(GPc + tile_off + c * 1024), lane * 16, dst + (KS + c) * 1024);
+                direct_load_16(uniform_ptr(XP2c + tile_off + c * 1024), lane * 16, dst + (2 * KS + c) * 1024);
+                direct_load_16(uniform_ptr(GP2c + tile_off + c * 1024), lane * 16, dst + (3 * KS + c) * 1024);
+            }
+            const unsigned voff = (unsigned)min(t * 32 + lane, Tp - 1) * 4;
+            direct_load_4(lse2, voff, dst + 4 * KS * 1024);
+            direct_load_4(delta, voff, dst + 4 * KS * 1024 + 256);
+        };
+        if (t_first <= t_last) fetch(t_first, 0);
+        int slot = 0;
+        for (int t = t_first; t <= t_last; t += kW) {
+            const int r0 = t * 32;
+            // tile t has landed, and this wave's reads of the other slot are done: it may be overwritten
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));
+            asm volatile("" ::: "memory");
+            if (t + kW <= t_last) fetch(t + kW, slot ^ 1);
+            const char* st = ring + slot * kTileBytes;
+            slot ^= 1;
+            f32x16 s, dp;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[i] = 0.f;
+                dp[i] = 0.f;
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) s = M::mma(*reinterpret_cast<const v8*>(st + ks * 1024 + lane * 16), kb[ks], s);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) dp = M::mma(*reinterpret_cast<const v8*>(st + (KS + ks) * 1024 + lane * 16), vbv[ks], dp);
+            float ls[16], dl[16];
+            tile_vector(reinterpret_cast<const float*>(st + 4 * KS * 1024), g, ls);
+            tile_vector(reinterpret_cast<const float*>(st + 4 * KS * 1024 + 256), g, dl);
+            const bool edge = (r0 + 31 >= T) || (c0 + 31 >= T) || (p.causal && ((c0 + 31 > r0) || (r0 + 31 - c0 > p.k_diff)));
+            float pr[16], ds[16];
+            if (edge) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int r = r0 + key_of(g, i);
+                    const bool ok = pair_ok(T, p.causal, p.k_diff, r, a);
+                    pr[i] = ok ? fast_exp2(fmaf(s[i], scale_log2, ba - ls[i])) : 0.f;
+                    ds[i] = ok ? pr[i] * (dp[i] - dl[i]) : 0.f;
+                    db += ds[i];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    pr[i] = fast_exp2(fmaf(s[i], scale_log2, ba - ls[i]));
+                    ds[i] = pr[i] * (dp[i] - dl[i]);
+                    db += ds[i];
+                }
+            }
+            v8 pb[2], dsb[2];
+            pack16<E>(pr, pb);
+            pack16<E>(ds, dsb);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk) {
+                    acck[dt] = M::mma(*reinterpret_cast<const v8*>(st + (2 * KS + dt * 2 + kk) * 1024 + lane * 16), dsb[kk], acck[dt]);
+                    accv[dt] = M::mma(*reinterpret_cast<const v8*>(st + (3 * KS + dt * 2 + kk) * 1024 + lane * 16), pb[kk], accv[dt]);
+                }
+        }
+        __syncthreads();  // every wave is done with its ring: the merge tiles go on top of them
+    } else {
     // streamed operands and the per-row statistics of a tile are fetched one tile ahead, into the
     // registers the previous tile has just consumed
     v8 xn[KS], gn[KS], x2n[DT][2], g2n[DT][2];
@@ -622,7 +716,6 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
                 g2n[dt][kk] = ld8<E>(p2_at<E, D>(GP2, t, dt, kk, lane));
             }
     };
-    const int t_first = r_lo / 32 + wave, t_last = r_hi / 32;
     if (t_first <= t_last) {
         fetch_rows(t_first);
         fetch_stats(t_first);
@@ -676,6 +769,7 @@ __global__ __launch_bounds__(64 * kW, (D <= 32 ? 2 : 1)) void attn_bwd_col_mfma_
             }
         if (more) fetch_cols(t + kW);
     }
+    }  // operands from registers
     db += __shfl_xor(db, 32, 64);
 
     const int aa = tid & 31, dg = tid >> 5, row = c0 + aa;
@@ -917,8 +1011,11 @@ Layout layout(int BH, int T, int D, bool bwd) {
 
 template <int D, int kW>
 constexpr size_t fwd_smem() { return 4 * (size_t)(kW * D * kLdr + 2 * kW * 32); }
-template <int D, int kW>
-constexpr size_t col_smem() { return 4 * (size_t)(kW * D * kLdr + kW * 32 + 2 * kW * 32); }
+template <int D, int kW, bool RING = false>
+constexpr size_t col_smem() {
+    const size_t merge = 4 * (size_t)(kW * D * kLdr + kW * 32 + 2 * kW * 32), ring = (size_t)kW * 2 * col_ring_tile_bytes<D>();
+    return RING && ring > merge ? ring : merge;
+}
 template <int D, int kW>
 constexpr size_t row_smem() { return 4 * (size_t)(kW * D * kLdr); }
 
@@ -1020,11 +1117,15 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     const dim3 grid(8 * xcd_slots(a.BH, Tp / 32));
     const bool pair_in = pair_tiles(a, a.k_diff, grid.x, true), pair_out = pair_tiles(a, a.T, grid.x, true);
     auto krow = attn_bwd_row_mfma_kernel<E, D, kW, SV>;
-    auto kcol_link = attn_bwd_col_mfma_kernel<E, D, kW, true, SV>;
-    auto kcol = attn_bwd_col_mfma_kernel<E, D, kW, false, SV>;
+    // the column kernel's operands through per-wave LDS rings (see the kernel) where four waves split the streamed tiles,
+    // i.e. from T = 2048 on; measured backward, bf16: B=1 H=8 T=4096 306 -> 291 us, B=2 H=8 T=2048 199 -> 191 us; with two
+    // waves (B=4 H=8 T=1024) 136.5 -> 138.7 us, so those keep the operands in registers
+    constexpr bool kRing = D == 64 && kW == 4;
+    auto kcol_link = attn_bwd_col_mfma_kernel<E, D, kW, true, SV, kRing>;
+    auto kcol = attn_bwd_col_mfma_kernel<E, D, kW, false, SV, kRing>;
     hipError_t e = allow_smem(krow, row_smem<D, kW>());
-    if (e == hipSuccess) e = allow_smem(kcol_link, col_smem<D, kW>());
-    if (e == hipSuccess) e = allow_smem(kcol, col_smem<D, kW>());
+    if (e == hipSuccess) e = allow_smem(kcol_link, col_smem<D, kW, kRing>());
+    if (e == hipSuccess) e = allow_smem(kcol, col_smem<D, kW, kRing>());
     if (e != hipSuccess) return e;
 
     PrepP<E, SV> pp{};
@@ -1082,7 +1183,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     }
     if (!shared) {
         hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_out), dim3(64 * kW), (row_smem<D, kW>()), st, o);
-        hipLaunchKernelGGL(kcol_link, attn_grid(a, Tp, pair_out), dim3(64 * kW), (col_smem<D, kW>()), st, o);
+        hipLaunchKernelGGL(kcol_link, attn_grid(a, Tp, pair_out), dim3(64 * kW), (col_smem<D, kW, kRing>()), st, o);
     }
 
     // inner pass: X = K2, G = dR, K = K1, V = U
@@ -1109,7 +1210,7 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
     }
     if (!shared) {
         hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_in), dim3(64 * kW), (row_smem<D, kW>()), st, i);
-        hipLaunchKernelGGL(kcol, attn_grid(a, Tp, pair_in), dim3(64 * kW), (col_smem<D, kW>()), st, i);
+        hipLaunchKernelGGL(kcol, attn_grid(a, Tp, pair_in), dim3(64 * kW), (col_smem<D, kW, kRing>()), st, i);
     }
     return hipGetLastError();
 }
