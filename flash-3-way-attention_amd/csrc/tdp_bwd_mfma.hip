@@ -671,6 +671,9 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     const int tiles = 8 * ((a.BH + 7) / 8) * ((a.T + 31) / 32);
     int splits = 1;
     if (tiles < 1024) splits = std::min(16, (1024 + tiles - 1) / tiles);
+    // a few waves of long tiles: the last tiles of each head are the costliest (the work of a tile grows with the
+    // square of its position), and halving them shortens the tail by about 1 % (measured: B=4 H=8 T=1024, 2048)
+    else if (tiles < 4096 && a.T >= 1024) splits = 2;
     if (knobs().bwd_splits > 0) splits = std::min(16, knobs().bwd_splits);  // tuning sweeps
     float* dqacc = splits > 1 ? (float*)(ws + l.dqacc) : nullptr;
 
