@@ -387,6 +387,9 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
     // holding D / 2 of each in registers where the accumulators leave no room for them: both at D = 128, those of
     // dP alone at D = 64 in the launch that also carries the dQ accumulators
     constexpr bool FLY = D > 64, FLY_G = FLY || (D == 64 && WITH_DQ);
+    // dQ of the tile, summed over the rounds: in registers up to 64 columns; beyond that the accumulators of a round
+    // leave no room for it and it lives in LDS, where the waves add their round's share one after another
+    constexpr bool DQ_LDS = WITH_DQ && DOUT > 64;
     extern __shared__ __align__(16) float smem_f[];
     float* sK = smem_f;                 // [2][32][LD]
     float* sV = sK + 2 * 32 * LD;       // [2][32][LD]
@@ -394,7 +397,7 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
     float* sDO = sQ + 32 * LD;          // [32][LD]
     float* sKb = sDO + 32 * LD;         // [NW][D]
     float* sVb = sKb + NW * D;          // [NW][D]
-    float* sO = sK;                     // [DOUT][33]   end of kernel: dQ of the tile (aliases the stages)
+    float* sO = DQ_LDS ? sVb + NW * D : sK;  // [DOUT][33]  dQ of the tile (aliases the stages when it is only formed at the end)
 
     int bh, order;
     if (!xcd_tile(p.BH, p.nqt, blockIdx.x >> 3, blockIdx.x & 7, bh, order)) return;
@@ -451,11 +454,13 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
         }
     }
 
-    f32x16 accDQ[DTO];
+    f32x16 accDQ[DQ_LDS ? 1 : DTO];
 #pragma unroll
-    for (int dt = 0; dt < DTO; ++dt)
+    for (int dt = 0; dt < (DQ_LDS ? 1 : DTO); ++dt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) accDQ[dt][i] = 0.f;
+    if constexpr (DQ_LDS)  // the first round's opening barrier orders this before the first addition
+        for (int idx = tid; idx < DOUT * 33; idx += 512) sO[idx] = 0.f;
 
     StageE<E, D> regs;
     for (int m = m_lo; m <= m_hi; m += parts) {
@@ -555,7 +560,7 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int d = c0 + dt * 32 + c_row(g, i), dc = dt * 32 + c_row(0, i);
-                    if constexpr (WITH_DQ) accDQ[dt][i] += accQ[dt][i] * sKb[kb_base + dc];
+                    if constexpr (WITH_DQ && !DQ_LDS) accDQ[dt][i] += accQ[dt][i] * sKb[kb_base + dc];
                     // sQ holds Q * alpha * log2(e): alpha is wanted, log2(e) is not
                     const float rk = half_sum(accQ[dt][i] * sQ[q_base + dc]) * kLn2;
                     const float rv = half_sum(accT[dt][i] * sDO[q_base + dc]);
@@ -567,20 +572,40 @@ __device__ __forceinline__ void f32_bwd_body(const F32BwdParams<E>& p, int only_
                     }
                 }
         }
+        if constexpr (DQ_LDS) {
+            // dQ[q] += Yq (.) K2[b], one wave after another: a fixed summation order (every wave takes part in the
+            // barriers, whether or not it had a row this round)
+            for (int w = 0; w < NW; ++w) {
+                if (wave == w && row_ok) {
+                    int kb_base = wave * D + c0 + 4 * g, o_base = 4 * g * 33 + n;
+                    asm volatile("" : "+v"(kb_base), "+v"(o_base));
+#pragma unroll
+                    for (int dt = 0; dt < DTO; ++dt)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            const int dc = dt * 32 + c_row(0, i);
+                            sO[o_base + dc * 33] += accQ[dt][i] * sKb[kb_base + dc];
+                        }
+                }
+                __syncthreads();
+            }
+        }
     }
 
     if constexpr (WITH_DQ) {
         __syncthreads();
-        for (int idx = tid; idx < DOUT * 33; idx += 512) sO[idx] = 0.f;
-        __syncthreads();
-        for (int w = 0; w < NW; ++w) {  // one wave after another: a fixed summation order
-            if (wave == w) {
-#pragma unroll
-                for (int dt = 0; dt < DTO; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) sO[(dt * 32 + c_row(g, i)) * 33 + n] += accDQ[dt][i];
-            }
+        if constexpr (!DQ_LDS) {
+            for (int idx = tid; idx < DOUT * 33; idx += 512) sO[idx] = 0.f;
             __syncthreads();
+            for (int w = 0; w < NW; ++w) {  // one wave after another: a fixed summation order
+                if (wave == w) {
+#pragma unroll
+                    for (int dt = 0; dt < DTO; ++dt)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) sO[(dt * 32 + c_row(g, i)) * 33 + n] += accDQ[dt][i];
+                }
+                __syncthreads();
+            }
         }
         for (int idx = tid; idx < 32 * DOUT; idx += 512) {
             const int r = idx / DOUT, d = idx % DOUT;
@@ -655,7 +680,8 @@ __global__ __launch_bounds__(256) void f32_finish_kernel(const long long* __rest
 
 template <int D>
 constexpr size_t f32_bwd_smem() {
-    return sizeof(float) * (size_t)(4 * 32 * (D + 1) + 2 * 32 * (D + 1) + 2 * kF32Waves * D);
+    // stages, Q and dO, the rows of a round; D = 128: dQ of the tile (f32_bwd_body's DQ_LDS)
+    return sizeof(float) * (size_t)(4 * 32 * (D + 1) + 2 * 32 * (D + 1) + 2 * kF32Waves * D + (D > 64 ? D * 33 : 0));
 }
 
 // where the six inputs lie (F32Params::H and at_*)
@@ -684,13 +710,12 @@ template <typename E, int D>
 hipError_t launch_f32_bwd_tiles(F32BwdParams<E> p, const E* k1, const E* u, const E* k2, const E* v2, void* acc_k2,
                                 void* acc_v2, void* acc_k1, void* acc_u, const TdpMask& natural, bool want_q,
                                 bool want_k2, bool want_k1, hipStream_t st, const InputsAt& at) {
-    // D = 128: the launch that also accumulates dQ produces 64 gradient columns per workgroup (both column halves
-    // form S and dP); without the dQ accumulators a workgroup holds all 128 columns and forms them once
-    constexpr int DOUT = D > 64 ? 64 : D, DOUT_NODQ = D;
+    // a workgroup holds all D gradient columns and forms S and dP once (D = 128: dQ's running sum is kept in LDS)
+    constexpr int DOUT = D, DOUT_NODQ = D;
     auto kern_dq = tdp_f32_bwd_kernel<E, D, DOUT, true>;
     auto kern_nodq = tdp_f32_bwd_kernel<E, D, DOUT_NODQ, false>;
     constexpr size_t smem = f32_bwd_smem<D>();
-    static_assert(DOUT * 33 <= 4 * 32 * (D + 1), "dQ of the tile aliases the stage buffers");
+    static_assert(DOUT * 33 <= 4 * 32 * (D + 1), "dQ of the tile aliases the stage buffers (D <= 64)");
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
     // small grids: the rounds of a tile dealt out to several workgroups (the launch with dQ only when dQ has an accumulator)

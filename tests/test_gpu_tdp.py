@@ -92,6 +92,25 @@ def test_fp32_tensors_on_the_matrix_cores(D, causal, windows, tune):
         util.assert_close(f"{name} vs VALU kernels", a, b, **FP32)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_fp32_head_dim_128_large_grid_on_the_matrix_cores(causal, tune):
+    """D = 128 with enough query tiles that each is walked by one workgroup (dQ written by that workgroup, its running
+    sum kept in LDS): against the fp32 VALU kernels of the same library, bitwise the same on a second run."""
+    print(f"case fp32 mfma D=128 large grid causal={causal}", flush=True)
+    inputs = orc.make_inputs(2, 4, 530, 128, torch.float32, seed=11)
+    alpha = 1 / math.sqrt(128)
+    out, g = util.run_tdp(inputs, alpha, causal)
+    out2, g2 = util.run_tdp(inputs, alpha, causal)
+    for name, a, b in zip(util.NAMES, g, g2):
+        assert torch.equal(a, b), name
+    tune(_lib.TUNE_F32_VALU, 1)
+    out_v, g_v = util.run_tdp(inputs, alpha, causal)
+    assert not torch.equal(out, out_v), "both runs took the same kernels"
+    util.assert_close("out vs VALU kernels", out, out_v, **FP32)
+    for name, a, b in zip(util.NAMES, g, g_v):
+        util.assert_close(f"{name} vs VALU kernels", a, b, **FP32)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_config2_lowp_forward_backward(dtype):
     """B=2 H=4 T=256 D=64, 16-bit tensors with fp32 accumulation, all five gradients."""
