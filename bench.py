@@ -31,13 +31,13 @@ NOMINAL_CLOCK_MHZ = 2400.0  # the clock behind the published peak
 # default workload only, scaled by a plain 256 MiB copy (summary and commands:
 # profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt).  Reported only when the workload is the default one.
 TRAFFIC_SOURCE = "profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt (rocprofv3 --pmc, default workload only)"
-# 27.4 MiB fetched + 15.0 MiB written: the algorithmic 20 + 4 MiB, and 28 bytes per lane that the kernel's prologue
+# 26.8 MiB fetched + 15.0 MiB written: the algorithmic 20 + 4 MiB, and 28 bytes per lane that the kernel's prologue
 # spills (a million lanes: ~11 MiB written once; spill-free builds of the kernel measured 2 % slower)
-TRAFFIC_FWD = 44.4e6
-# average of the two launches: ~530 MiB written by 64-bit atomics each, 34 / 40 MiB fetched (some runs: up to 440 MiB in the first
+TRAFFIC_FWD = 43.8e6
+# average of the two launches: 558 / 527 MiB written by 64-bit atomics, 35 / 42 MiB fetched (some runs: up to 440 MiB in the first
 # launch, when its accumulators fall out of their XCD's L2; the bytes are L2 <-> fabric traffic, which the 256 MB Infinity
 # Cache absorbs)
-TRAFFIC_BWD_ROWS = 593e6
+TRAFFIC_BWD_ROWS = 609e6
 
 
 def triples(B, H, T, causal=True):
