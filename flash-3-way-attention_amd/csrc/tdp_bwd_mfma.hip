@@ -84,6 +84,7 @@ __device__ __forceinline__ float acc_scale(const BwdParams<E>& p, int bh) {
 
 #include "tdp_bwd_rows_general.hpp"
 #include "tdp_bwd_rows_q16.hpp"
+#include "tdp_f32_tiles.hpp"
 
 namespace tritt {
 
@@ -114,8 +115,8 @@ namespace tritt {
 //  * stages are fetched direct-to-LDS two ahead into three buffers and the workgroup barrier
 //    sits in the middle of a stage: by then the next stage has landed for every wave, so its
 //    first row operands are read during the second half and nothing waits at the stage boundary.
-template <typename E, int D, bool WITH_DQ, bool SV = false>
-__global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
+template <typename E, int D, bool WITH_DQ, bool SV>
+__device__ __forceinline__ void tdp_bwd_rows_body(const BwdParams<E>& p, const int block) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     using v2 = typename M::v2;
@@ -141,8 +142,8 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     E* sQe = reinterpret_cast<E*>(sOb + BQ * LDQ + (NW / 2) * (BQ * D));
     E* sOe = sQe + DT * 64 * 16;
 
-    const int xcd = blockIdx.x & 7;
-    int slot = blockIdx.x >> 3;
+    const int xcd = block & 7;
+    int slot = block >> 3;
     const int split = slot % p.splits;  // which share of the tile's rounds this workgroup walks (small grids)
     slot /= p.splits;
     int bh, order;
@@ -490,6 +491,31 @@ __global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
     }
 }
 
+template <typename E, int D, bool WITH_DQ, bool SV = false>
+__global__ __launch_bounds__(512) void tdp_bwd_rows_kernel(BwdParams<E> p) {
+    tdp_bwd_rows_body<E, D, WITH_DQ, SV>(p, blockIdx.x);
+}
+
+// The same grid together with the fp32 workgroups of query tile 0 (tdp_f32_tiles.hpp: both roles, one workgroup per
+// round of eight rows; t0_x * 2 * rounds of them).  As a launch of their own they are 64 short workgroups between two
+// launches that fill the chip, 30 us in which most of it idles.  Here they come after the main blocks, beside the
+// last and lightest tiles of the launch (t0_first = 0: large grids, whose heavy tiles should start at once), or
+// before them (small grids: the main blocks are as short as these, and a latency-bound workgroup that starts last
+// is the launch's tail).  They add to the same accumulators as every other workgroup, in fixed point, so the order
+// changes nothing.
+template <typename E, int D, bool WITH_DQ, bool SV>
+__global__ __launch_bounds__(512) void tdp_bwd_rows_tile0_kernel(BwdParams<E> p, F32BwdParams<E> r0, F32BwdParams<E> r1,
+                                                                 int roles_mask, int main_blocks, int t0_x, int t0_first) {
+    const int t0_blocks = t0_x * 2 * r0.split_rounds;
+    const int block = (int)blockIdx.x - (t0_first ? t0_blocks : 0);  // main blocks: 0 .. main_blocks - 1
+    if (block >= 0 && block < main_blocks) {
+        tdp_bwd_rows_body<E, D, WITH_DQ, SV>(p, block);
+    } else {
+        const int extra = t0_first ? (int)blockIdx.x : block - main_blocks;
+        f32_tile0_block<E, D, D>(r0, r1, roles_mask, extra / t0_x, extra % t0_x);
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // scratch producers / consumers
 // U = SiLU(V1) row-major; U^T and K1^T as [D][Tp] (zero padded); Delta = rowsum(dO*O);
@@ -706,6 +732,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     void (*kern_dq)(BwdParams<E>);
     void (*kern_nodq)(BwdParams<E>);
     int nthreads = 512, col_parts = 1;
+    bool plain64 = false;  // the D = 64 kernel of this file
     if constexpr (D == 32) {
         // one shape, the banded instantiation for every mask (full windows are windows of T)
         smem = bwdg_smem(32, 8, 32, true);
@@ -766,6 +793,7 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
                4 * (size_t)(2 * 32 * (64 + 4) + 4 * 32 * 64);
         kern_dq = tdp_bwd_rows_kernel<E, 64, true, SV>;
         kern_nodq = tdp_bwd_rows_kernel<E, 64, false, SV>;
+        plain64 = true;
     }
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_dq), smem); e != hipSuccess) return e;
     if (hipError_t e = ensure_dynamic_smem(reinterpret_cast<const void*>(kern_nodq), smem); e != hipSuccess) return e;
@@ -779,6 +807,11 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     const bool first_in_f32 = a.causal != 0;
     const long long pairs = (long long)(a.k2_window + 1) * std::min(a.k1_window + 1, a.kk_left + a.kk_right + 1);
     const bool all_in_f32 = first_in_f32 && a.windowed && pairs <= 1024 && !a.split;
+    // tile 0's backward workgroups ride at the end of the first rows launch below where that is the D = 64 kernel
+    // (tdp_bwd_rows_tile0_kernel); otherwise they are a launch of their own
+    bool fuse_tile0 = false;
+    [[maybe_unused]] F32BwdParams<E> t0_r0{}, t0_r1{};
+    [[maybe_unused]] int t0_roles = 0, t0_rounds = 0;
     if (first_in_f32) {
         FirstTileArgs f{};
         f.q = a.q; f.d_o = a.d_o; f.k1 = a.k1; f.u = u; f.k2 = a.k2; f.v2 = a.v2;
@@ -793,7 +826,14 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
         f.want_q = want_q; f.want_k2 = want_k2; f.want_k1 = want_k1;
         f.tiles = all_in_f32 ? p.nqt : 1;
         f.round_parts = (dqacc || !want_q) ? std::min(splits, f32_round_parts(a.BH, a.T)) : 1;
-        if (hipError_t e = f32_mfma_tdp_bwd_first_tile(f, st); e != hipSuccess) return e;
+        if constexpr (D == 64) {
+            if (plain64 && !all_in_f32 && p.nqt > 1 && (want_q || want_k2 || want_k1)) {
+                if (hipError_t e = tile0_prepare<E, 64>(f, st, t0_r0, t0_r1, t0_roles, t0_rounds); e != hipSuccess) return e;
+                fuse_tile0 = true;
+            }
+        }
+        if (!fuse_tile0)
+            if (hipError_t e = f32_mfma_tdp_bwd_first_tile(f, st); e != hipSuccess) return e;
     }
     const int tiles_here = all_in_f32 ? 0 : p.nqt - (first_in_f32 ? 1 : 0);
     p.grid_tiles = std::max(tiles_here, 1);  // the tiles the grid covers: nqt - 1 .. nqt - grid_tiles
@@ -804,16 +844,34 @@ static hipError_t launch_bwd(const MfmaBwdArgs& a, hipStream_t st) {
     p.at_row_k = a.at_k2; p.at_row_v = a.at_v2; p.at_st_k = a.at_k1; p.at_st_v = at_u;
     p.acc_k = dk2acc; p.acc_v = dv2acc; p.bit_k = kPoisonDK2; p.bit_v = kPoisonDV2;
     p.wa = a.k1_window; p.wb = a.k2_window; p.lab = a.kk_left; p.rab = a.kk_right;
+    hipError_t launch_error = hipSuccess;
+    auto launch_rows = [&](bool with_dq) {
+        if constexpr (D == 64) {
+            if (fuse_tile0) {  // the first launch takes tile 0 along
+                auto fused = with_dq ? tdp_bwd_rows_tile0_kernel<E, 64, true, SV> : tdp_bwd_rows_tile0_kernel<E, 64, false, SV>;
+                launch_error = ensure_dynamic_smem(reinterpret_cast<const void*>(fused), std::max(smem, f32_bwd_smem<64>()));
+                if (launch_error != hipSuccess) return;
+                const int t0_x = 8 * xcd_slots(a.BH, 1);
+                const int t0_first = tiles < 1024 ? 1 : 0;
+                hipLaunchKernelGGL(fused, dim3(grid.x + t0_x * 2 * t0_rounds), dim3(512), std::max(smem, f32_bwd_smem<64>()),
+                                   st, p, t0_r0, t0_r1, t0_roles, (int)grid.x, t0_x, t0_first);
+                fuse_tile0 = false;
+                return;
+            }
+        }
+        hipLaunchKernelGGL(with_dq ? kern_dq : kern_nodq, grid, dim3(nthreads), smem, st, p);
+    };
     // a launch whose gradients the caller does not want (null outputs) is skipped
-    if (tiles_here > 0 && want_q) hipLaunchKernelGGL(kern_dq, grid, dim3(nthreads), smem, st, p);
-    else if (tiles_here > 0 && want_k2) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
+    if (tiles_here > 0 && want_q) launch_rows(true);
+    else if (tiles_here > 0 && want_k2) launch_rows(false);
     // rows = (K1, U), streamed = (K2, V2): dK1, dU
     p.row_k = (const E*)a.k1; p.row_v = u;
     p.st_k = (const E*)a.k2; p.st_v = (const E*)a.v2; p.st_kt = k2t; p.st_vt = v2t;
     p.at_row_k = a.at_k1; p.at_row_v = at_u; p.at_st_k = a.at_k2; p.at_st_v = a.at_v2;
     p.acc_k = dk1acc; p.acc_v = duacc; p.bit_k = kPoisonDK1; p.bit_v = kPoisonDU;
     p.wa = a.k2_window; p.wb = a.k1_window; p.lab = a.kk_right; p.rab = a.kk_left;  // the mask with j and k exchanged
-    if (tiles_here > 0 && want_k1) hipLaunchKernelGGL(kern_nodq, grid, dim3(nthreads), smem, st, p);
+    if (tiles_here > 0 && want_k1) launch_rows(false);
+    if (launch_error != hipSuccess) return launch_error;
 
     const size_t n = (size_t)a.BH * a.T * D;
     size_t gridf = (n + 255) / 256;
