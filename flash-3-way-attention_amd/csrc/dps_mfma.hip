@@ -409,7 +409,7 @@ struct AttnBwdP {
 };
 
 template <typename E, int D, int kW, bool SV>
-__global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_kernel(AttnBwdP<E, SV> p) {
+__device__ __forceinline__ void attn_bwd_row_body(const AttnBwdP<E, SV>& p) {
     using M = Mma<E>;
     using v8 = typename M::v8;
     constexpr int KS = D / 16, DT = D / 32;
@@ -548,6 +548,17 @@ __global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_
         *reinterpret_cast<v8*>(p.dx + off) = ov;
     }
     }  // owner tiles of this workgroup
+}
+
+template <typename E, int D, int kW, bool SV>
+__global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_mfma_kernel(AttnBwdP<E, SV> p) {
+    attn_bwd_row_body<E, D, kW, SV>(p);
+}
+// Two row passes in one grid (blockIdx.y picks the pass): the outer pass's dQ and the inner pass's dK2 depend on
+// nothing of each other, and one pass alone gives a SIMD a single latency-bound wave.
+template <typename E, int D, int kW, bool SV>
+__global__ __launch_bounds__(64 * kW, (D <= 64 ? 2 : 1)) void attn_bwd_row_pair_kernel(AttnBwdP<E, SV> p0, AttnBwdP<E, SV> p1) {
+    attn_bwd_row_body<E, D, kW, SV>(blockIdx.y == 0 ? p0 : p1);
 }
 
 // --------------------------------------------------------------------------- backward, columns
@@ -1181,8 +1192,11 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
             hipLaunchKernelGGL(scol_out, grid_shared, dim3(64 * kSW), ColShape::smem, st, o);
         }
     }
+    // the two row passes share a launch when their grids are the same (attn_bwd_row_pair_kernel); the outer one then
+    // waits for the outer column pass, which the inner one needs
+    const bool rows_together = !shared && pair_out == pair_in;
     if (!shared) {
-        hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_out), dim3(64 * kW), (row_smem<D, kW>()), st, o);
+        if (!rows_together) hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_out), dim3(64 * kW), (row_smem<D, kW>()), st, o);
         hipLaunchKernelGGL(kcol_link, attn_grid(a, Tp, pair_out), dim3(64 * kW), (col_smem<D, kW, kRing>()), st, o);
     }
 
@@ -1209,7 +1223,14 @@ hipError_t run_bwd(const MfmaDpsArgs& a, hipStream_t st) {
         }
     }
     if (!shared) {
-        hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_in), dim3(64 * kW), (row_smem<D, kW>()), st, i);
+        if (rows_together) {
+            auto krow2 = attn_bwd_row_pair_kernel<E, D, kW, SV>;
+            if (e = allow_smem(krow2, row_smem<D, kW>()); e != hipSuccess) return e;
+            const dim3 g1 = attn_grid(a, Tp, pair_in);
+            hipLaunchKernelGGL(krow2, dim3(g1.x, 2), dim3(64 * kW), (row_smem<D, kW>()), st, o, i);
+        } else {
+            hipLaunchKernelGGL(krow, attn_grid(a, Tp, pair_in), dim3(64 * kW), (row_smem<D, kW>()), st, i);
+        }
         hipLaunchKernelGGL(kcol, attn_grid(a, Tp, pair_in), dim3(64 * kW), (col_smem<D, kW, kRing>()), st, i);
     }
     return hipGetLastError();
