@@ -31,13 +31,13 @@ NOMINAL_CLOCK_MHZ = 2400.0  # the clock behind the published peak
 # default workload only, scaled by a plain 256 MiB copy (summary and commands:
 # profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt).  Reported only when the workload is the default one.
 TRAFFIC_SOURCE = "profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt (rocprofv3 --pmc, default workload only)"
-# 26.8 MiB fetched + 15.0 MiB written: the algorithmic 20 + 4 MiB, and 28 bytes per lane that the kernel's prologue
+# 27.4 MiB fetched + 15.0 MiB written: the algorithmic 20 + 4 MiB, and 28 bytes per lane that the kernel's prologue
 # spills (a million lanes: ~11 MiB written once; spill-free builds of the kernel measured 2 % slower)
-TRAFFIC_FWD = 43.8e6
-# average of the two launches: 558 / 527 MiB written by 64-bit atomics, 35 / 42 MiB fetched (some runs: up to 440 MiB in the first
+TRAFFIC_FWD = 44.4e6
+# average of the two launches: 568 / 527 MiB written by 64-bit atomics, 36 / 39 MiB fetched (some runs: up to 440 MiB in the first
 # launch, when its accumulators fall out of their XCD's L2; the bytes are L2 <-> fabric traffic, which the 256 MB Infinity
 # Cache absorbs)
-TRAFFIC_BWD_ROWS = 609e6
+TRAFFIC_BWD_ROWS = 614e6
 
 
 def triples(B, H, T, causal=True):
@@ -502,10 +502,13 @@ def main():
                    "peak_used": "2.5 PFLOP/s bf16 dense (256 CUs x 4096 flop/clk x 2.4 GHz nominal)",
                    # measured in this run: what a pure-MFMA kernel reaches, and the clock that implies
                    "mfma_probe": probe},
-        # dominant kernel by time: tdp_bwd_rows_kernel, launched twice per backward (dQ,dK2,dV2 then
-        # dK1,dU).  Each launch is credited half of the backward's algorithmic flops (6*D*N) and
-        # half of the event-timed backward (the prep/finish kernels in that time are < 1 %).
-        "roofline": {"bound": "mfma", "kernel": "tdp_bwd_rows_kernel<bf16,64> (avg of its 2 launches)",
+        # dominant kernel by time: the rows kernel of the backward, launched twice (dQ,dK2,dV2 then dK1,dU; the
+        # first launch is tdp_bwd_rows_tile0_kernel, the same body with the 128 fp32 workgroups of query tile 0 in
+        # its grid, the second tdp_bwd_rows_kernel).  Each launch is credited half of the backward's algorithmic
+        # flops (6*D*N) and half of the event-timed backward (the prep/finish kernels in that time are < 1 %).
+        "roofline": {"bound": "mfma",
+                     "kernel": "tdp_bwd_rows_tile0_kernel<bf16,64,true> + tdp_bwd_rows_kernel<bf16,64,false> (the rows "
+                               "kernel's two launches, averaged)",
                      "achieved": bwd_tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": bwd_tf / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BWD_ROWS if default_workload else None,
                      "traffic_source": TRAFFIC_SOURCE if default_workload else None,
