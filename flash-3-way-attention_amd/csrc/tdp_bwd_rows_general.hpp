@@ -262,6 +262,15 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
     const int krow_off = key_of_row(n);
     const int fperm = D == 32 ? swz_t(krow_off) : swz_perm(krow_off);
 
+    // STAG (the split-operand kernel under full windows, where a step is long enough for it to pay: 17.2 -> 16.9 ms
+    // at B=4 H=8 T=1024; the windowed and the D = 32 instantiations measured 1-8 % slower with it): the two waves
+    // of a SIMD (w and w + 4) run half a step apart, as in tdp_bwd_rows_kernel.  The barrier of step g then stands
+    // for "stage g + 1 has landed for every wave, every wave is done with stage g - 1"; the first wave of a SIMD
+    // crosses it at the top of its step, the second after its score products, and a wave's priority is low over
+    // its score products and high over the rest of the step.
+    constexpr bool STAG = SPLIT && !WIN && D == 64 && NW == 8;
+    [[maybe_unused]] const bool late = STAG && ((wave >> 2) & 1);
+    if constexpr (STAG) barrier_keep_loads<LW>();  // stage 0 and the first round's rows have landed for every wave
     for (int m = m_lo; m < m_hi; ++m) {
         const int mb = m & 1;
         const int k = m * NW + wave;
@@ -291,10 +300,14 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             // this wave's part of stage gstage (and, at a round's first step, its part of the round's
             // rows) has landed; after the barrier that holds for every wave's part, and every wave is
             // done with the buffer the next fetch overwrites
-            barrier_keep_loads<LW>();
-            if (st == st_first && m + 1 < m_hi) issue_round(m + 1, mb ^ 1);  // older than the stage loads
-            issue_stage(st_ahead, (gstage + 2) % NBUF);
-            advance();
+            auto stage_barrier = [&]() {
+                if constexpr (STAG) barrier_keep_loads<0>();
+                else barrier_keep_loads<LW>();
+                if (st == st_first && m + 1 < m_hi) issue_round(m + 1, mb ^ 1);  // older than the stage loads
+                issue_stage(st_ahead, (gstage + 2) % NBUF);
+                advance();
+            };
+            if (!late) stage_barrier();
             if (!built) {
                 // B operands of the score products of this round: alpha log2e Q (.) K2[k] and dO (.) V2[k]
                 built = true;
@@ -377,6 +390,7 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             __builtin_amdgcn_sched_barrier(0);
             // S starts from 0, or from -3e4 where (q, j, k) is invalid; element i of a lane is key
             // jb + key_of(0, i) + 8 g.  The extra k-step subtracts LSE2[q] / Delta[q].
+            if constexpr (STAG) __builtin_amdgcn_s_setprio(0);
             f32x16 s, dp;
             {
                 f32x16 c;
@@ -416,6 +430,11 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                     dp = M::mma(au[ks & 3], bg[ks], dp);
                 }
                 __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (STAG) {
+                if (late) stage_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_setprio(1);
             }
             v8 bt[DT][2], bk[DT][2];
 #pragma unroll
@@ -527,7 +546,8 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
         }
         // all waves are done with this round's K2/V2 rows; the next round's have landed (they are older
         // than the stage loads kept in flight)
-        barrier_keep_loads<2 * LW>();
+        if constexpr (STAG) barrier_keep_loads<LW>();  // the round's load is older than the one stage in flight
+        else barrier_keep_loads<2 * LW>();
         if constexpr (WITH_DQ) {
             if (k <= jend && (wave & 1) == 1) add_dq();
         }
