@@ -350,3 +350,55 @@ def test_layouts_the_library_refuses():
                                               1, T, _lib.ptr(ws), need, flags, _lib.stream_ptr(o.device))
         assert st == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("variant", ["tdp", "dps"])
+@pytest.mark.parametrize("shape,dtype", [((2, 4, 256, 64), torch.bfloat16), ((1, 3, 150, 128), torch.float16),
+                                         ((2, 2, 100, 32), torch.bfloat16), ((1, 2, 96, 32), torch.float32)])
+@pytest.mark.parametrize("strided", ["dO", "inputs"])
+def test_only_one_side_is_strided(variant, shape, dtype, strided):
+    """The layout of a model's backward: dense q, k1, k2, v1, v2 and an incoming gradient that is a [B,T,H,D] tensor
+    transposed (what autograd hands back when the output is transposed for the next projection), and the reverse
+    (transposed projections in, a dense gradient).  The C ABI then gets a null layout array for the dense side.  All
+    five gradients bitwise those of the call on dense copies."""
+    from flash_trittention.triple_dot_product.flash_trittention import flash_trittention
+    from flash_trittention.dot_product_sum.trittention_triton import TrittentionTriton
+
+    B, H, T, D = shape
+    print(f"case one side strided: {variant} {shape} {dtype} strided={strided}", flush=True)
+    if strided == "inputs":
+        ins = [bthd_view(B, H, T, D, dtype, seed=20 + i) for i in range(5)]
+        d_o = torch.randn(B, H, T, D, generator=torch.Generator().manual_seed(7)).to(dtype).cuda()
+    else:
+        g = torch.Generator().manual_seed(8)
+        ins = [torch.randn(B, H, T, D, generator=g).to(dtype).cuda() for _ in range(5)]
+        d_o = bthd_view(B, H, T, D, dtype, seed=9)
+    assert d_o.is_contiguous() == (strided == "inputs")
+    alpha = 1 / math.sqrt(D)
+    if variant == "tdp":
+        fn = lambda *t: flash_trittention(*t, softmax_scale=alpha, k1_window=None, k2_window=None, kk_left=None,
+                                          kk_right=None, causal=True)
+    else:
+        mod = TrittentionTriton(causal=True, softmax_scale=alpha, k_diff=T)
+        fn = lambda *t: mod(*t)[0]
+
+    def grads(tensors, go):
+        leaves = [t.detach().clone(memory_format=torch.preserve_format).requires_grad_(True) for t in tensors]
+        # clone() of a transposed view keeps its strides: the leaves are laid out like the tensors handed in
+        assert all(a.stride() == b.stride() for a, b in zip(leaves, tensors))
+        out = fn(*leaves)
+        out.backward(go)
+        return [out.detach()] + [t.grad for t in leaves]
+
+    got = grads(ins, d_o)
+    want = grads([t.contiguous() for t in ins], d_o.contiguous())
+    for name, a, b in zip(("out",) + tuple(util.NAMES), got, want):
+        assert torch.equal(a.contiguous(), b.contiguous()), name
+    if variant == "tdp":
+        z, _, ref = util.oracle_tdp(dense_inputs(ins, d_o), alpha, True)
+    else:
+        z, _, ref = util.oracle_dps(dense_inputs(ins, d_o), alpha, True, T)
+    tol = FP32 if dtype == torch.float32 else LOWP
+    util.assert_close("out", got[0].float().cpu(), z, **tol)
+    for name, a, b in zip(util.NAMES, got[1:], ref):
+        util.assert_close(name, a.float().cpu(), b, **tol)
