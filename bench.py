@@ -230,6 +230,7 @@ def dps_times(torch, dev, B, H, T, D, steps, warmup, dtype=None, k_diff=None):
     from flash_trittention import _ops
     with torch.no_grad():
         o_op, lse_op = _ops.dps_fwd_impl(*ins[:5], alpha, True, k_diff, 0)
+        ms_f_op = time_events(lambda: _ops.dps_fwd_impl(*ins[:5], alpha, True, k_diff, 0), steps, max(warmup, 3), torch)
         ms_b_op = time_events(lambda: _ops.dps_bwd_impl(*ins[:5], o_op, lse_op, ins[5], alpha, True, k_diff, 0), steps,
                               max(warmup, 3), torch)
     n3 = B * H * T * (T + 1) * (T + 2) // 6   # valid (q,s,t) triples of the reference's formulation, k_diff = T
@@ -240,7 +241,7 @@ def dps_times(torch, dev, B, H, T, D, steps, warmup, dtype=None, k_diff=None):
     peak = PEAK_F32_TFLOPS if dtype == torch.float32 else PEAK_BF16_TFLOPS
     bytes_f, bytes_b = 6 * B * H * T * D * elem + 4 * B * H * T, 12 * B * H * T * D * elem + 8 * B * H * T
     tf_f, tf_b = 4 * D * (n_in + n_out) / ms_f / 1e9, 10 * D * (n_in + n_out) / ms_b / 1e9
-    row = {"fwd_ms": ms_f, "bwd_ms": ms_b, "bwd_ms_operator_call": ms_b_op,
+    row = {"fwd_ms": ms_f, "bwd_ms": ms_b, "fwd_ms_operator_call": ms_f_op, "bwd_ms_operator_call": ms_b_op,
            "executed_fwd_tflops": tf_f, "executed_bwd_tflops": tf_b,
            "mfma_frac_fwd": tf_f / peak, "mfma_frac_bwd": tf_b / peak,
            "algorithmic_bytes_fwd": bytes_f, "algorithmic_bytes_bwd": bytes_b,
