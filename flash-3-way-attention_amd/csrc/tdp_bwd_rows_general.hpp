@@ -434,7 +434,8 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
             if constexpr (STAG) {
                 if (late) stage_barrier();
                 __builtin_amdgcn_sched_barrier(0);
-                __builtin_amdgcn_s_setprio(1);
+                if (late) __builtin_amdgcn_s_setprio(2);  // one level above the first wave: the two never tie
+                else __builtin_amdgcn_s_setprio(1);
             }
             v8 bt[DT][2], bk[DT][2];
 #pragma unroll
