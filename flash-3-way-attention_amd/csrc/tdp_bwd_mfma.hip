@@ -171,6 +171,7 @@ __device__ __forceinline__ void tdp_bwd_rows_body(const BwdParams<E>& p, const i
     const int jend = p.causal ? qlast : T - 1;  // last j (and last k) any query of the tile needs
     const int jfull = p.causal ? q0 : T - 1;    // keys / rows 0 .. jfull are valid for every column
     const int nst = jend / 64 + 1, nrounds = jend / 8 + 1;
+    const bool dead_tail = (jend & 63) < 32;  // the last stage's second step lies past every query's last key
     const int per_split = (nrounds + p.splits - 1) / p.splits;
     const int m_lo = split * per_split, m_hi = min(nrounds, m_lo + per_split);
     if (m_lo >= m_hi) return;  // fewer rounds than shares (uniform over the workgroup, before any barrier)
@@ -359,10 +360,15 @@ __device__ __forceinline__ void tdp_bwd_rows_body(const BwdParams<E>& p, const i
                     st_ahead = st_ahead + 1 < nst ? st_ahead + 1 : 0;
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                // a step past every query's last key (the second half of the last stage, for every other tile) has
+                // S = -3e4 from the C operand above, so P = dS = 0 whatever the other k-steps would add: they are skipped
+                const bool dead = half == 1 && dead_tail && st == nst - 1;
+                if (!dead) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    if (ks > 0) s = M::mma(ak[ks], bq[ks], s);
-                    if (ks > 0) dp = M::mma(au[ks], bg[ks], dp);
+                    for (int ks = 0; ks < KS; ++ks) {
+                        if (ks > 0) s = M::mma(ak[ks], bq[ks], s);
+                        if (ks > 0) dp = M::mma(au[ks], bg[ks], dp);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 // (the second wave of the SIMD one level above the first, so that the two never tie: another 0.8 %)
@@ -391,26 +397,30 @@ __device__ __forceinline__ void tdp_bwd_rows_body(const BwdParams<E>& p, const i
                     pa[h][e] = pp[0]; pa[h][e + 1] = pp[1];
                     da[h][e] = dd[0]; da[h][e + 1] = dd[1];
                 };
-#pragma unroll
-                for (int r = 0; r < 4; ++r) softmax_pair(r);
-                __builtin_amdgcn_sched_barrier(0);
                 static_assert(DT == 2, "interleave written for D = 64");
+                if (!dead) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[0], bt[r >> 1][0], accT[r >> 1]);
-                    else accQ[r >> 1] = M::mma(da[0], bk[r >> 1][0], accQ[r >> 1]);
+                    for (int r = 0; r < 4; ++r) softmax_pair(r);
                     __builtin_amdgcn_sched_barrier(0);
-                    softmax_pair(4 + r);
-                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[0], bt[r >> 1][0], accT[r >> 1]);
+                        else accQ[r >> 1] = M::mma(da[0], bk[r >> 1][0], accQ[r >> 1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        softmax_pair(4 + r);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
                 // the row operands are dead: read those of the next step (second half of this stage,
                 // or first half of the next one, which has landed for everyone since the barrier)
                 load_rows(half == 0 ? sb : (gstage + 1) % NBUF, half ^ 1);
                 __builtin_amdgcn_sched_barrier(0);
+                if (!dead) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[1], bt[r >> 1][1], accT[r >> 1]);
-                    else accQ[r >> 1] = M::mma(da[1], bk[r >> 1][1], accQ[r >> 1]);
+                    for (int r = 0; r < 4; ++r) {
+                        if ((r & 1) == 0) accT[r >> 1] = M::mma(pa[1], bt[r >> 1][1], accT[r >> 1]);
+                        else accQ[r >> 1] = M::mma(da[1], bk[r >> 1][1], accQ[r >> 1]);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 // The stage's one workgroup barrier: the next stage has landed for every wave, everyone is
