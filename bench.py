@@ -34,10 +34,10 @@ TRAFFIC_SOURCE = "profiles/tdp_fwd_bwd_B4_H8_T1024_D64_bf16_counters.txt (rocpro
 # 27.4 MiB fetched + 15.0 MiB written: the algorithmic 20 + 4 MiB, and 28 bytes per lane that the kernel's prologue
 # spills (a million lanes: ~11 MiB written once; spill-free builds of the kernel measured 2 % slower)
 TRAFFIC_FWD = 44.4e6
-# average of the two launches: 568 / 527 MiB written by 64-bit atomics, 36 / 39 MiB fetched (some runs: up to 440 MiB in the first
+# average of the two launches: 587 / 527 MiB written (64-bit atomics; the first launch also spills 16-20 bytes per lane), 36 / 39 MiB fetched (some runs: up to 440 MiB in the first
 # launch, when its accumulators fall out of their XCD's L2; the bytes are L2 <-> fabric traffic, which the 256 MB Infinity
 # Cache absorbs)
-TRAFFIC_BWD_ROWS = 614e6
+TRAFFIC_BWD_ROWS = 624e6
 
 
 def triples(B, H, T, causal=True):
