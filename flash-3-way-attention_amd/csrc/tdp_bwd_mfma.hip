@@ -434,9 +434,11 @@ __device__ __forceinline__ void tdp_bwd_rows_body(const BwdParams<E>& p, const i
         }
 
         // ---- round epilogue (rows of the accumulators = the 32 queries, column = d) ---------------
-        [[maybe_unused]] auto add_dq = [&]() {  // slice += Yq (.) K2[k]
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
+        // columns 32 dt .. + 31 of the slice += Yq (.) K2[k]; dt at compile time (a run-time choice of registers would be
+        // indexed through M0, which the direct loads own)
+        [[maybe_unused]] auto add_dq = [&](auto dt_c) {
+            constexpr int dt = decltype(dt_c)::value;
+            {
                 const float kd = (float)sKr[(mb * 8 + wave) * D + dt * 32 + n];
 #pragma unroll
                 for (int i4 = 0; i4 < 4; ++i4) {
@@ -473,14 +475,23 @@ __device__ __forceinline__ void tdp_bwd_rows_body(const BwdParams<E>& p, const i
                 }
             }
         }
+        // The two waves of a pair add their tiles to the pair's slice half and half: before the barrier the even wave
+        // its columns 0-31 and the odd wave its columns 32-63, after it the other halves.  (One wave before and one
+        // after puts two chains of eight dependent LDS round trips on the workgroup's path per round instead of two of four.)
         if constexpr (WITH_DQ) {
-            if (k <= jend && (wave & 1) == 0) add_dq();
+            if (k <= jend) {
+                if (wave & 1) add_dq(std::integral_constant<int, 1>{});
+                else add_dq(std::integral_constant<int, 0>{});
+            }
         }
         // all waves are done with this round's K2/V2 rows; the next round's have landed: they are older than the newest
         // stage's loads, the only ones allowed to stay in flight (a tile of a single stage issues both in its one step)
         barrier_keep_loads<LW>();
         if constexpr (WITH_DQ) {
-            if (k <= jend && (wave & 1) == 1) add_dq();
+            if (k <= jend) {
+                if (wave & 1) add_dq(std::integral_constant<int, 0>{});
+                else add_dq(std::integral_constant<int, 1>{});
+            }
         }
     }
     wait_vmcnt<0>();  // the stages fetched ahead land in the buffers reused below

@@ -496,12 +496,15 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
         }
 
         // ---- round epilogue (rows of the accumulators = the 32 queries, column = c0 + 32 dt + n)
-        [[maybe_unused]] auto add_dq = [&]() {  // slice += Yq (.) K2[k]
+        // registers 8 part .. 8 part + 7 of every accumulator tile: slice += Yq (.) K2[k]
+        [[maybe_unused]] auto add_dq = [&](auto part_c) {
+            constexpr int part = decltype(part_c)::value;  // compile time: a run-time choice of registers would be
+                                                           // indexed through M0, which the direct loads own
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const float kd = (float)sKr[(mb * RR + wave) * D + c0 + dt * 32 + n];
 #pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
+                for (int i4 = 2 * part; i4 < 2 * part + 2; ++i4) {
                     float4* slot4 = reinterpret_cast<float4*>(sDQ + ((dt * 4 + i4) * 64 + lane) * 4);
                     float4 v = *slot4;
                     v.x += accQ[dt][i4 * 4] * kd; v.y += accQ[dt][i4 * 4 + 1] * kd;
@@ -542,15 +545,25 @@ __global__ __launch_bounds__(64 * NW) void tdp_bwd_rows_general_kernel(BwdParams
                 }
             }
         }
+        // the two waves of a pair add their tiles to the pair's slice half and half: before the barrier the even wave
+        // its first eight registers per tile and the odd wave its last eight, after it the other halves (one wave
+        // before and one after would put two chains of dependent LDS round trips of twice the length on the
+        // workgroup's path)
         if constexpr (WITH_DQ) {
-            if (k <= jend && (wave & 1) == 0) add_dq();
+            if (k <= jend) {
+                if (wave & 1) add_dq(std::integral_constant<int, 1>{});
+                else add_dq(std::integral_constant<int, 0>{});
+            }
         }
         // all waves are done with this round's K2/V2 rows; the next round's have landed (they are older
         // than the stage loads kept in flight)
         if constexpr (STAG) barrier_keep_loads<LW>();  // the round's load is older than the one stage in flight
         else barrier_keep_loads<2 * LW>();
         if constexpr (WITH_DQ) {
-            if (k <= jend && (wave & 1) == 1) add_dq();
+            if (k <= jend) {
+                if (wave & 1) add_dq(std::integral_constant<int, 0>{});
+                else add_dq(std::integral_constant<int, 1>{});
+            }
         }
     }
     wait_vmcnt<0>();  // the stages fetched ahead land in LDS before the workgroup ends
